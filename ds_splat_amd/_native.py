@@ -1,0 +1,87 @@
+"""ctypes binding of libdsx.so (the C ABI declared in include/dsx.h).
+
+The library is built in-tree by ``__graft_entry__.build()`` (or ``make -C ds_splat_amd/csrc``)
+into ``ds_splat_amd/lib/libdsx.so``.  There is no fallback: if the library is missing or a
+symbol is absent, loading raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdsx.so")
+
+SPLAT_FLOATS = 12
+GRAD_FLOATS = 12
+PROJ_BLOCK = 256
+TILE = 16
+
+
+class Camera(C.Structure):
+    """struct dsx_camera"""
+    _fields_ = [
+        ("image_height", C.c_int32),
+        ("image_width", C.c_int32),
+        ("tanfovx", C.c_float),
+        ("tanfovy", C.c_float),
+        ("scale_modifier", C.c_float),
+        ("sh_degree", C.c_int32),
+        ("max_sh_degree", C.c_int32),
+        ("view", C.c_void_p),
+        ("proj", C.c_void_p),
+        ("campos", C.c_void_p),
+        ("bg", C.c_void_p),
+    ]
+
+
+_P = C.c_void_p
+_I64 = C.c_int64
+_I32 = C.c_int32
+_CAM = C.POINTER(Camera)
+
+# name -> (restype, argtypes); must list every function include/dsx.h declares
+SIGNATURES = {
+    "dsx_error_string": (C.c_char_p, [C.c_int]),
+    "dsx_version": (C.c_int, []),
+    "dsx_num_blocks": (_I64, [_I64]),
+    "dsx_num_tiles": (_I32, [_I32, _I32]),
+    "dsx_sort_passes": (_I32, [_I32]),
+    "dsx_workspace_bytes": (C.c_size_t, [_I64, _I64, _I32, _I32]),
+    "dsx_project_fwd": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P] * 4 + [_P]),
+    "dsx_scan_u32": (C.c_int, [_I64, _P, _P, _P]),
+    "dsx_emit_keys": (C.c_int, [_CAM, _I64, _I64, _P, _P, _P, _P, _P]),
+    "dsx_sort_pairs": (C.c_int, [_I64, _I32, _P, _P, _P, C.c_size_t, _P]),
+    "dsx_tile_ranges": (C.c_int, [_I64, _P, _I32, _P, _P]),
+    "dsx_blend_fwd": (C.c_int, [_CAM] + [_P] * 6 + [_P]),
+    "dsx_blend_bwd": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P]),
+    "dsx_gaussian_bwd": (C.c_int, [_CAM, _I64, _I32] + [_P] * 7 + [_P] * 8 + [_P]),
+    "dsx_forward_project": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P] * 5 + [C.POINTER(_I64), _P]),
+    "dsx_forward_finish": (C.c_int, [_CAM, _I64, _I64] + [_P] * 7 + [_P, C.c_size_t, _P]),
+    "dsx_backward": (C.c_int, [_CAM, _I64, _I32] + [_P] * 11 + [_P] * 9 + [_P]),
+    "dsx_forward_core": (C.c_int, [_P] * 5 + [_I64] + [_P] * 3 + [_I32, _I32, C.c_float, C.c_float, C.c_float,
+                                                                    _I32, _I32, _P, _P]),
+}
+
+_lib = None
+
+
+def load():
+    """Loads libdsx.so once and attaches prototypes.  Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "ds_splat_amd: native library %s is missing — build it with "
+            "`python -c 'import __graft_entry__ as g; g.build()'` or `make -C ds_splat_amd/csrc`" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != 0:
+        raise RuntimeError(load().dsx_error_string(status).decode())

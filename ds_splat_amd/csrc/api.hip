@@ -1,0 +1,357 @@
+// extern "C" surface of libdsx: argument checks, stage sequencing, the one host
+// synchronisation of the forward (read-back of the key count) and error strings.
+#include "dsx_common.h"
+
+using namespace dsx;
+
+namespace
+{
+
+inline hipStream_t as_stream(void* s)
+{
+    return static_cast<hipStream_t>(s);
+}
+
+int check_camera(const dsx_camera* cam)
+{
+    if(cam == nullptr)
+        return DSX_ERR_BAD_ARG;
+    if(cam->image_width <= 0 || cam->image_height <= 0)
+        return DSX_ERR_BAD_ARG;
+    if(cam->view == nullptr || cam->proj == nullptr || cam->campos == nullptr || cam->bg == nullptr)
+        return DSX_ERR_BAD_ARG;
+    // the reference asserts 0 <= sh_degree <= 4 and max_sh_degree == 3
+    // (cpp/rasterizer_torch.cu:124-129); degree 4 has no forward there, so 0..3 it is
+    if(cam->sh_degree < 0 || cam->sh_degree > 3 || cam->max_sh_degree < cam->sh_degree || cam->max_sh_degree > 3)
+        return DSX_ERR_BAD_ARG;
+    return DSX_OK;
+}
+
+} // namespace
+
+extern "C" const char* dsx_error_string(int status)
+{
+    switch(status)
+    {
+        case DSX_OK: return "ok";
+        case DSX_ERR_BAD_ARG: return "dsx: bad argument (null pointer, negative size or unsupported SH degree)";
+        case DSX_ERR_LAUNCH: return "dsx: kernel launch failed";
+        case DSX_ERR_RUNTIME: return "dsx: HIP runtime call failed";
+        case DSX_ERR_TOO_LARGE: return "dsx: too many tile keys for 32-bit key indexing (K >= 2^30)";
+        case DSX_ERR_WORKSPACE: return "dsx: workspace too small (see dsx_workspace_bytes)";
+        default: return "dsx: unknown status";
+    }
+}
+
+extern "C" int dsx_version(void)
+{
+    return 100;
+}
+
+extern "C" int64_t dsx_num_blocks(int64_t n)
+{
+    return n <= 0 ? 0 : (n + kProjBlock - 1) / kProjBlock;
+}
+
+extern "C" int32_t dsx_num_tiles(int32_t width, int32_t height)
+{
+    return tiles_x(width) * tiles_y(height);
+}
+
+extern "C" int32_t dsx_sort_passes(int32_t num_tiles)
+{
+    return sort_passes(num_tiles);
+}
+
+extern "C" size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height)
+{
+    (void)n;
+    return forward_workspace(k < 0 ? 0 : k, dsx_num_tiles(width, height)).bytes;
+}
+
+extern "C" int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
+                               const float* quats, const float* opacities, const float* shs,
+                               const float* cov3d_precomp, const float* colors_precomp, float* splats,
+                               int32_t* radii, float* cov3d, uint32_t* block_sums, void* stream)
+{
+    if(int rc = check_camera(cam))
+        return rc;
+    if(n < 0)
+        return DSX_ERR_BAD_ARG;
+    if(n == 0)
+        return DSX_OK;
+    if(!means3d || !opacities || !splats || !radii || !cov3d || !block_sums)
+        return DSX_ERR_BAD_ARG;
+    if(!cov3d_precomp && (!scales || !quats))
+        return DSX_ERR_BAD_ARG;
+    if(!colors_precomp && !shs)
+        return DSX_ERR_BAD_ARG;
+    return launch_project_fwd(*cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp, splats,
+                              radii, cov3d, block_sums, as_stream(stream));
+}
+
+extern "C" int dsx_scan_u32(int64_t count, uint32_t* data, uint32_t* total, void* stream)
+{
+    if(count < 0 || !total || (count > 0 && !data))
+        return DSX_ERR_BAD_ARG;
+    return launch_scan_u32(count, data, total, as_stream(stream));
+}
+
+extern "C" int dsx_emit_keys(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
+                             const uint32_t* block_offsets, int64_t* keys, int32_t* values, void* stream)
+{
+    if(int rc = check_camera(cam))
+        return rc;
+    if(n < 0 || k < 0)
+        return DSX_ERR_BAD_ARG;
+    if(n == 0 || k == 0)
+        return DSX_OK;
+    if(!splats || !block_offsets || !keys || !values)
+        return DSX_ERR_BAD_ARG;
+    return launch_emit_keys(*cam, n, k, splats, block_offsets, keys, values, as_stream(stream));
+}
+
+extern "C" int dsx_sort_pairs(int64_t k, int32_t num_tiles, int64_t* keys, int32_t* values, void* workspace,
+                              size_t workspace_bytes, void* stream)
+{
+    if(k < 0 || num_tiles < 0)
+        return DSX_ERR_BAD_ARG;
+    if(k <= 1)
+        return DSX_OK;
+    if(!keys || !values || !workspace)
+        return DSX_ERR_BAD_ARG;
+    if(k >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
+    const SortWorkspace w = sort_workspace(k, num_tiles);
+    if(workspace_bytes < w.bytes)
+        return DSX_ERR_WORKSPACE;
+    char* base = static_cast<char*>(workspace);
+    int64_t* keys_b = reinterpret_cast<int64_t*>(base + w.keys_alt);
+    int32_t* values_b = reinterpret_cast<int32_t*>(base + w.values_alt);
+    int64_t* ko;
+    int32_t* vo;
+    int rc = launch_sort_pairs(k, num_tiles, keys, values, keys_b, values_b, workspace, as_stream(stream), &ko, &vo);
+    if(rc)
+        return rc;
+    if(ko != keys)
+    {
+        if(hipMemcpyAsync(keys, ko, (size_t)k * 8, hipMemcpyDeviceToDevice, as_stream(stream)) != hipSuccess ||
+           hipMemcpyAsync(values, vo, (size_t)k * 4, hipMemcpyDeviceToDevice, as_stream(stream)) != hipSuccess)
+            return DSX_ERR_RUNTIME;
+    }
+    return DSX_OK;
+}
+
+extern "C" int dsx_tile_ranges(int64_t k, const int64_t* sorted_keys, int32_t num_tiles, int32_t* ranges,
+                               void* stream)
+{
+    if(k < 0 || num_tiles < 0 || !ranges || (k > 0 && !sorted_keys))
+        return DSX_ERR_BAD_ARG;
+    if(k >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
+    return launch_tile_ranges(k, sorted_keys, num_tiles, ranges, as_stream(stream));
+}
+
+extern "C" int dsx_blend_fwd(const dsx_camera* cam, const int32_t* ranges, const int32_t* sorted_ids,
+                             const float* splats, float* image, float* final_T, int32_t* final_idx, void* stream)
+{
+    if(int rc = check_camera(cam))
+        return rc;
+    if(!ranges || !image || !final_T || !final_idx)
+        return DSX_ERR_BAD_ARG;
+    return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream));
+}
+
+extern "C" int dsx_blend_bwd(const dsx_camera* cam, int64_t n, const int32_t* ranges, const int32_t* sorted_ids,
+                             const float* splats, const float* final_T, const int32_t* final_idx,
+                             const float* v_image, float* grads, void* stream)
+{
+    if(int rc = check_camera(cam))
+        return rc;
+    if(n < 0)
+        return DSX_ERR_BAD_ARG;
+    if(n == 0)
+        return DSX_OK;
+    if(!ranges || !final_T || !final_idx || !v_image || !grads || !splats)
+        return DSX_ERR_BAD_ARG;
+    return launch_blend_bwd(*cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
+                            as_stream(stream));
+}
+
+extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+                                const float* scales, const float* quats, const float* splats, const float* cov3d,
+                                const int32_t* radii, const float* grads, float* v_mean3d, float* v_means2d,
+                                float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
+                                float* v_cov3d, void* stream)
+{
+    if(int rc = check_camera(cam))
+        return rc;
+    if(n < 0 || num_bases < 0 || num_bases > 16)
+        return DSX_ERR_BAD_ARG;
+    if(n == 0)
+        return DSX_OK;
+    if(!means3d || !splats || !cov3d || !radii || !grads || !v_mean3d || !v_means2d || !v_colors || !v_opacity ||
+       !v_scale || !v_quat || !v_cov3d)
+        return DSX_ERR_BAD_ARG;
+    if((scales == nullptr) != (quats == nullptr))
+        return DSX_ERR_BAD_ARG;
+    return launch_gaussian_bwd(*cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
+                               v_means2d, num_bases > 0 ? v_shs : nullptr, v_colors, v_opacity, v_scale, v_quat,
+                               v_cov3d, as_stream(stream));
+}
+
+extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
+                                   const float* quats, const float* opacities, const float* shs,
+                                   const float* cov3d_precomp, const float* colors_precomp, float* splats,
+                                   int32_t* radii, float* cov3d, uint32_t* block_sums, uint32_t* k_scratch,
+                                   int64_t* num_keys, void* stream)
+{
+    if(!num_keys || !k_scratch)
+        return DSX_ERR_BAD_ARG;
+    *num_keys = 0;
+    int rc = dsx_project_fwd(cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp, splats,
+                             radii, cov3d, block_sums, stream);
+    if(rc || n == 0)
+        return rc;
+    rc = launch_scan_u32(dsx_num_blocks(n), block_sums, k_scratch, as_stream(stream));
+    if(rc)
+        return rc;
+    uint32_t k_host = 0;
+    if(hipMemcpyAsync(&k_host, k_scratch, sizeof(uint32_t), hipMemcpyDeviceToHost, as_stream(stream)) != hipSuccess)
+        return DSX_ERR_RUNTIME;
+    if(hipStreamSynchronize(as_stream(stream)) != hipSuccess)
+        return DSX_ERR_RUNTIME;
+    *num_keys = (int64_t)k_host;
+    return k_host >= (1u << 30) ? DSX_ERR_TOO_LARGE : DSX_OK;
+}
+
+extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
+                                  const uint32_t* block_offsets, int32_t* sorted_ids, int32_t* ranges,
+                                  float* image, float* final_T, int32_t* final_idx, void* workspace,
+                                  size_t workspace_bytes, void* stream)
+{
+    if(int rc = check_camera(cam))
+        return rc;
+    if(n < 0 || k < 0 || !ranges || !image || !final_T || !final_idx)
+        return DSX_ERR_BAD_ARG;
+    if(k >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
+    hipStream_t s = as_stream(stream);
+    const int num_tiles = dsx_num_tiles(cam->image_width, cam->image_height);
+    const int64_t* sorted_keys = nullptr;
+    if(k > 0)
+    {
+        if(!splats || !block_offsets || !sorted_ids || !workspace)
+            return DSX_ERR_BAD_ARG;
+        const ForwardWorkspace fw = forward_workspace(k, num_tiles);
+        if(workspace_bytes < fw.bytes)
+            return DSX_ERR_WORKSPACE;
+        const SortWorkspace sw = sort_workspace(k, num_tiles);
+        char* base = static_cast<char*>(workspace);
+        char* sbase = base + fw.sort;
+        // ping-pong parity: start so that the last pass lands the ids in the caller's buffer
+        int64_t* keys_x = reinterpret_cast<int64_t*>(base + fw.keys);
+        int64_t* keys_y = reinterpret_cast<int64_t*>(sbase + sw.keys_alt);
+        int32_t* vals_final = sorted_ids;
+        int32_t* vals_other = reinterpret_cast<int32_t*>(sbase + sw.values_alt);
+        const bool even = (sw.passes % 2) == 0 || k <= 1;
+        int64_t* keys_a = keys_x;
+        int64_t* keys_b = keys_y;
+        int32_t* vals_a = even ? vals_final : vals_other;
+        int32_t* vals_b = even ? vals_other : vals_final;
+        int rc = launch_emit_keys(*cam, n, k, splats, block_offsets, keys_a, vals_a, s);
+        if(rc)
+            return rc;
+        int64_t* ko;
+        int32_t* vo;
+        rc = launch_sort_pairs(k, num_tiles, keys_a, vals_a, keys_b, vals_b, sbase, s, &ko, &vo);
+        if(rc)
+            return rc;
+        if(vo != sorted_ids)
+            return DSX_ERR_RUNTIME;
+        sorted_keys = ko;
+    }
+    int rc = launch_tile_ranges(k, sorted_keys, num_tiles, ranges, s);
+    if(rc)
+        return rc;
+    return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, s);
+}
+
+extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+                            const float* scales, const float* quats, const float* splats, const float* cov3d,
+                            const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
+                            const float* final_T, const int32_t* final_idx, const float* v_image, float* grads,
+                            float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors, float* v_opacity,
+                            float* v_scale, float* v_quat, float* v_cov3d, void* stream)
+{
+    int rc = dsx_blend_bwd(cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads, stream);
+    if(rc)
+        return rc;
+    return dsx_gaussian_bwd(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
+                            v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, stream);
+}
+
+extern "C" int dsx_forward_core(const float* means3d, const float* shs, const float* opacities, const float* scales,
+                                const float* quats, int64_t n, const float* view, const float* proj,
+                                const float* campos, int32_t image_width, int32_t image_height, float tanfovx,
+                                float tanfovy, float scale_modifier, int32_t max_sh_degree, int32_t sh_degree,
+                                float* image, void* stream)
+{
+    hipStream_t s = as_stream(stream);
+    dsx_camera cam;
+    cam.image_height = image_height;
+    cam.image_width = image_width;
+    cam.tanfovx = tanfovx;
+    cam.tanfovy = tanfovy;
+    cam.scale_modifier = scale_modifier;
+    cam.sh_degree = sh_degree;
+    cam.max_sh_degree = max_sh_degree;
+    cam.view = view;
+    cam.proj = proj;
+    cam.campos = campos;
+    cam.bg = campos; // unused by the forward
+    if(int rc = check_camera(&cam))
+        return rc;
+    if(n < 0 || !image)
+        return DSX_ERR_BAD_ARG;
+    const int64_t P = (int64_t)image_width * image_height;
+    const int num_tiles = dsx_num_tiles(image_width, image_height);
+    const int64_t nb = dsx_num_blocks(n);
+
+    auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    size_t o_splats = 0, o_radii, o_cov3d, o_bs, o_k, o_ranges, o_T, o_idx, stage1;
+    o_radii = align(o_splats + (size_t)n * 48);
+    o_cov3d = align(o_radii + (size_t)n * 4);
+    o_bs = align(o_cov3d + (size_t)n * 24);
+    o_k = align(o_bs + (size_t)nb * 4);
+    o_ranges = align(o_k + 4);
+    o_T = align(o_ranges + (size_t)(num_tiles + 1) * 4);
+    o_idx = align(o_T + (size_t)P * 4);
+    stage1 = align(o_idx + (size_t)P * 4);
+    char* buf = nullptr;
+    if(hipMallocAsync(reinterpret_cast<void**>(&buf), stage1 + 256, s) != hipSuccess)
+        return DSX_ERR_RUNTIME;
+    int64_t k = 0;
+    int rc = dsx_forward_project(&cam, n, means3d, scales, quats, opacities, shs, nullptr, nullptr,
+                                 reinterpret_cast<float*>(buf + o_splats), reinterpret_cast<int32_t*>(buf + o_radii),
+                                 reinterpret_cast<float*>(buf + o_cov3d), reinterpret_cast<uint32_t*>(buf + o_bs),
+                                 reinterpret_cast<uint32_t*>(buf + o_k), &k, stream);
+    char* buf2 = nullptr;
+    if(rc == DSX_OK)
+    {
+        const size_t ws = forward_workspace(k, num_tiles).bytes;
+        const size_t o_ids = align(ws);
+        if(hipMallocAsync(reinterpret_cast<void**>(&buf2), o_ids + (size_t)k * 4 + 256, s) != hipSuccess)
+            rc = DSX_ERR_RUNTIME;
+        else
+            rc = dsx_forward_finish(&cam, n, k, reinterpret_cast<float*>(buf + o_splats),
+                                    reinterpret_cast<uint32_t*>(buf + o_bs), reinterpret_cast<int32_t*>(buf2 + o_ids),
+                                    reinterpret_cast<int32_t*>(buf + o_ranges), image,
+                                    reinterpret_cast<float*>(buf + o_T), reinterpret_cast<int32_t*>(buf + o_idx),
+                                    buf2, ws, stream);
+    }
+    if(buf2)
+        (void)hipFreeAsync(buf2, s);
+    (void)hipFreeAsync(buf, s);
+    return rc;
+}

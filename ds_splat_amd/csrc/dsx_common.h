@@ -1,0 +1,174 @@
+// Internal declarations shared by the HIP translation units of libdsx (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "dsx.h"
+
+#define DSX_WAVE 64
+#define DSX_LAUNCH_CHECK()                                                                         \
+    do                                                                                             \
+    {                                                                                              \
+        if(hipGetLastError() != hipSuccess)                                                        \
+            return DSX_ERR_LAUNCH;                                                                 \
+    } while(0)
+
+namespace dsx
+{
+
+constexpr int kTile = DSX_TILE;
+constexpr int kTilePixels = DSX_TILE * DSX_TILE;
+constexpr int kProjBlock = DSX_PROJ_BLOCK;
+
+// Radix sort geometry: 8-bit digits, 256 threads, kSortItems keys per thread per tile.
+constexpr int kRadixBits = 8;
+constexpr int kRadix = 1 << kRadixBits;
+constexpr int kSortThreads = 256;
+constexpr int kSortItems = 16;
+constexpr int kSortTile = kSortThreads * kSortItems;
+
+inline int tiles_x(int w)
+{
+    return (w + kTile - 1) / kTile;
+}
+inline int tiles_y(int h)
+{
+    return (h + kTile - 1) / kTile;
+}
+
+// Bits of the sortable image of a key: 32 depth bits + enough for tile ids 0..num_tiles
+// (tile + 1; slot 0 holds the negative keys).
+inline int sort_key_bits(int num_tiles)
+{
+    int b = 0;
+    while((1ll << b) < (long long)num_tiles + 1)
+        ++b;
+    return 32 + b;
+}
+inline int sort_passes(int num_tiles)
+{
+    return (sort_key_bits(num_tiles) + kRadixBits - 1) / kRadixBits;
+}
+
+// Workspace layout of the sort for k keys (all offsets 256-byte aligned).
+struct SortWorkspace
+{
+    size_t keys_alt;    // int64[k]
+    size_t values_alt;  // int32[k]
+    size_t global_hist; // uint32[passes * 256]
+    size_t status;      // uint32[passes * tiles * 256]
+    size_t counters;    // uint32[passes + 1]: dynamic tile ids per pass, [passes] = error flag
+    size_t bytes;
+    int passes;
+    int64_t tiles;
+};
+SortWorkspace sort_workspace(int64_t k, int num_tiles);
+
+struct ForwardWorkspace
+{
+    size_t keys;   // int64[k]   emitted / sorted keys
+    size_t values; // int32[k]   only used when the pass count is odd (ping-pong parity)
+    size_t sort;   // SortWorkspace
+    size_t bytes;
+};
+ForwardWorkspace forward_workspace(int64_t k, int num_tiles);
+
+// launchers (each returns a dsx_status)
+int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, const float* scales,
+                       const float* quats, const float* opacities, const float* shs,
+                       const float* cov3d_precomp, const float* colors_precomp, float* splats,
+                       int32_t* radii, float* cov3d, uint32_t* block_sums, hipStream_t stream);
+int launch_scan_u32(int64_t count, uint32_t* data, uint32_t* total, hipStream_t stream);
+int launch_emit_keys(const dsx_camera& cam, int64_t n, int64_t k, const float* splats,
+                     const uint32_t* block_offsets, int64_t* keys, int32_t* values,
+                     hipStream_t stream);
+// Sorts (keys_a, values_a); the result lands in (keys_a, values_a) when `passes` is even and
+// in the workspace's alternate buffers when odd, unless want_in_place (then it is copied).
+int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values_a, int64_t* keys_b,
+                      int32_t* values_b, void* sort_ws, hipStream_t stream, int64_t** keys_out,
+                      int32_t** values_out);
+int launch_tile_ranges(int64_t k, const int64_t* sorted_keys, int num_tiles, int32_t* ranges,
+                       hipStream_t stream);
+int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids,
+                     const float* splats, float* image, float* final_T, int32_t* final_idx,
+                     hipStream_t stream);
+int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges,
+                     const int32_t* sorted_ids, const float* splats, const float* final_T,
+                     const int32_t* final_idx, const float* v_image, float* grads,
+                     hipStream_t stream);
+int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d,
+                        const float* scales, const float* quats, const float* splats,
+                        const float* cov3d, const int32_t* radii, const float* grads,
+                        float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
+                        float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d,
+                        hipStream_t stream);
+int launch_fill_u32(uint32_t* p, int64_t count, uint32_t value, hipStream_t stream);
+
+#ifdef __HIPCC__
+// ---- device helpers -------------------------------------------------------------------
+__device__ __forceinline__ int lane_id()
+{
+    return __lane_id();
+}
+
+// float -> int32 with the hardware conversion's semantics made explicit (saturate, NaN -> 0).
+__device__ __forceinline__ int f2i_sat(float x)
+{
+    if(x != x)
+        return 0;
+    if(x >= 2147483648.0f)
+        return 0x7fffffff;
+    if(x <= -2147483648.0f)
+        return (int)0x80000000;
+    return (int)x;
+}
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v)
+{
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, DSX_WAVE);
+    return v;
+}
+
+typedef float dsx_v4f __attribute__((ext_vector_type(4)));
+
+// streaming (non-temporal) 16-byte load / store: data that is touched once
+__device__ __forceinline__ float4 nt_load_f4(const float4* p)
+{
+    const dsx_v4f v = __builtin_nontemporal_load(reinterpret_cast<const dsx_v4f*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void nt_store_f4(float4* p, float4 v)
+{
+    dsx_v4f t;
+    t.x = v.x;
+    t.y = v.y;
+    t.z = v.z;
+    t.w = v.w;
+    __builtin_nontemporal_store(t, reinterpret_cast<dsx_v4f*>(p));
+}
+
+struct TileRect
+{
+    int sx, ex, sy, ey;
+};
+
+// Tile rectangle of a splat: truncation toward zero, +1 on the upper bound, clamped to the
+// tile grid.  Pure IEEE ops on powers of two, so it is exact on any target.
+__device__ __forceinline__ TileRect tile_rect(float px, float py, int radius, int ntx, int nty)
+{
+    const float cx = px / 16.0f;
+    const float cy = py / 16.0f;
+    const float d = (float)radius / 16.0f;
+    TileRect r;
+    r.sx = min(max(0, f2i_sat(cx - d)), ntx);
+    r.ex = min(max(0, f2i_sat((cx + d) + 1.0f)), ntx);
+    r.sy = min(max(0, f2i_sat(cy - d)), nty);
+    r.ey = min(max(0, f2i_sat((cy + d) + 1.0f)), nty);
+    return r;
+}
+#endif
+
+} // namespace dsx

@@ -1,0 +1,615 @@
+// Stages 2 and 3 for gfx950: block-sum scan, tile-key emission, 64-bit LSD radix sort
+// (one-sweep: one global histogram pass, then one chained-scan scatter pass per digit) and
+// tile-range identification.  Integer work only; everything is HBM-bandwidth bound.
+#include "dsx_common.h"
+
+namespace dsx
+{
+
+// ---------------------------------------------------------------------------------------
+// small wave/block primitives
+// ---------------------------------------------------------------------------------------
+
+__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t v, int lane)
+{
+#pragma unroll
+    for(int o = 1; o < DSX_WAVE; o <<= 1)
+    {
+        const uint32_t t = __shfl_up(v, o, DSX_WAVE);
+        if(lane >= o)
+            v += t;
+    }
+    return v;
+}
+
+__device__ __forceinline__ int wave_incl_max_i32(int v, int lane)
+{
+#pragma unroll
+    for(int o = 1; o < DSX_WAVE; o <<= 1)
+    {
+        const int t = __shfl_up(v, o, DSX_WAVE);
+        if(lane >= o)
+            v = max(v, t);
+    }
+    return v;
+}
+
+// lanes of the wavefront that hold the same 8-bit digit (and are valid); call in uniform flow
+__device__ __forceinline__ uint64_t match_digit(uint32_t d, bool valid)
+{
+    uint64_t mask = __ballot(valid);
+#pragma unroll
+    for(int b = 0; b < kRadixBits; ++b)
+    {
+        const bool bit = (d >> b) & 1u;
+        const uint64_t m = __ballot(bit);
+        mask &= bit ? m : ~m;
+    }
+    return mask;
+}
+
+__device__ __forceinline__ uint64_t lanemask_lt(int lane)
+{
+    return (1ull << lane) - 1ull;
+}
+
+// Sortable image of a key: negative keys (tile field all ones, produced by negative depths)
+// sort first in signed order, so they take tile slot 0 and every real tile moves up by one.
+__device__ __forceinline__ uint64_t sortable(int64_t key)
+{
+    return key < 0 ? ((uint64_t)key & 0xffffffffull) : (uint64_t)key + (1ull << 32);
+}
+
+// ---------------------------------------------------------------------------------------
+// fill
+// ---------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* p, int64_t count, uint32_t value)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
+        p[i] = value;
+}
+
+int launch_fill_u32(uint32_t* p, int64_t count, uint32_t value, hipStream_t stream)
+{
+    if(count <= 0)
+        return DSX_OK;
+    const int64_t blocks = min((int64_t)4096, (count + 255) / 256);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, count, value);
+    DSX_LAUNCH_CHECK();
+    return DSX_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// exclusive scan of a (short) uint32 array by one workgroup
+// ---------------------------------------------------------------------------------------
+
+constexpr int kScanThreads = 1024;
+constexpr int kScanItems = 4;
+
+__global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* data, int64_t count, uint32_t* total)
+{
+    __shared__ uint32_t wave_tot[kScanThreads / DSX_WAVE];
+    __shared__ uint32_t carry_s;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    if(tid == 0)
+        carry_s = 0;
+    __syncthreads();
+    for(int64_t base = 0; base < count; base += kScanThreads * kScanItems)
+    {
+        const int64_t i0 = base + (int64_t)tid * kScanItems;
+        uint32_t v[kScanItems];
+        uint32_t sum = 0;
+#pragma unroll
+        for(int j = 0; j < kScanItems; ++j)
+        {
+            v[j] = (i0 + j < count) ? data[i0 + j] : 0u;
+            sum += v[j];
+        }
+        const uint32_t incl = wave_incl_scan_u32(sum, lane);
+        if(lane == 63)
+            wave_tot[wave] = incl;
+        __syncthreads();
+        uint32_t wave_prefix = 0;
+        for(int w = 0; w < wave; ++w)
+            wave_prefix += wave_tot[w];
+        uint32_t run = carry_s + wave_prefix + incl - sum;
+#pragma unroll
+        for(int j = 0; j < kScanItems; ++j)
+        {
+            if(i0 + j < count)
+                data[i0 + j] = run;
+            run += v[j];
+        }
+        __syncthreads();
+        if(tid == kScanThreads - 1)
+            carry_s = run;
+        __syncthreads();
+    }
+    if(tid == 0)
+        *total = carry_s;
+}
+
+int launch_scan_u32(int64_t count, uint32_t* data, uint32_t* total, hipStream_t stream)
+{
+    hipLaunchKernelGGL(scan_u32_kernel, dim3(1), dim3(kScanThreads), 0, stream, data, count, total);
+    DSX_LAUNCH_CHECK();
+    return DSX_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// key emission: one workgroup per 256 Gaussians (the same partition as the projection), one
+// thread per OUTPUT key, so stores are contiguous however uneven the per-Gaussian tile counts
+// ---------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(kProjBlock) void emit_keys_kernel(const float4* __restrict__ splats,
+                                                               const uint32_t* __restrict__ block_offsets,
+                                                               int64_t n, int64_t k, int ntx, int nty,
+                                                               int64_t* __restrict__ keys,
+                                                               int32_t* __restrict__ values)
+{
+    __shared__ uint32_t s_off[kProjBlock + 1];
+    __shared__ int s_sx[kProjBlock], s_sy[kProjBlock], s_w[kProjBlock], s_depth[kProjBlock];
+    __shared__ uint32_t wave_tot[4];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int64_t g0 = (int64_t)blockIdx.x * kProjBlock;
+    const int64_t i = g0 + tid;
+
+    uint32_t count = 0;
+    if(i < n)
+    {
+        const float4 q0 = splats[3 * i];
+        const int radius = __float_as_int(q0.w);
+        const TileRect r = tile_rect(q0.x, q0.y, radius, ntx, nty);
+        const int w = r.ex - r.sx;
+        count = (uint32_t)(w * (r.ey - r.sy) * (radius > 0 ? 1 : 0));
+        if(i == n - 1)
+            count = 0; // the last Gaussian never emits (its end index is forced to K)
+        s_sx[tid] = r.sx;
+        s_sy[tid] = r.sy;
+        s_w[tid] = w;
+        s_depth[tid] = __float_as_int(q0.z);
+    }
+    const uint32_t incl = wave_incl_scan_u32(count, lane);
+    if(lane == 63)
+        wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t prefix = 0;
+    for(int w = 0; w < wave; ++w)
+        prefix += wave_tot[w];
+    s_off[tid] = prefix + incl - count;
+    if(tid == kProjBlock - 1)
+        s_off[kProjBlock] = prefix + incl;
+    __syncthreads();
+
+    const uint32_t total = s_off[kProjBlock];
+    const int64_t base = block_offsets[blockIdx.x];
+    for(uint32_t j = tid; j < total; j += kProjBlock)
+    {
+        // largest g with s_off[g] <= j
+        int lo = 0, hi = kProjBlock;
+        while(hi - lo > 1)
+        {
+            const int mid = (lo + hi) >> 1;
+            if(s_off[mid] <= j)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        const uint32_t r = j - s_off[lo];
+        const uint32_t w = (uint32_t)s_w[lo];
+        const uint32_t ry = r / w;
+        const uint32_t rx = r - ry * w;
+        const int64_t tile = (int64_t)(s_sy[lo] + (int)ry) * ntx + (s_sx[lo] + (int)rx);
+        const int64_t depth = (int64_t)s_depth[lo]; // sign-extending, as the reference does
+        const int64_t out = base + j;
+        if(out < k)
+        {
+            keys[out] = (int64_t)((uint64_t)tile << 32) | depth;
+            values[out] = (int32_t)(g0 + lo);
+        }
+    }
+}
+
+int launch_emit_keys(const dsx_camera& cam, int64_t n, int64_t k, const float* splats,
+                     const uint32_t* block_offsets, int64_t* keys, int32_t* values, hipStream_t stream)
+{
+    if(n == 0 || k == 0)
+        return DSX_OK;
+    const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
+    hipLaunchKernelGGL(emit_keys_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
+                       reinterpret_cast<const float4*>(splats), block_offsets, n, k, tiles_x(cam.image_width),
+                       tiles_y(cam.image_height), keys, values);
+    DSX_LAUNCH_CHECK();
+    return DSX_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// radix sort
+// ---------------------------------------------------------------------------------------
+
+SortWorkspace sort_workspace(int64_t k, int num_tiles)
+{
+    auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    SortWorkspace w;
+    w.passes = sort_passes(num_tiles);
+    w.tiles = (k + kSortTile - 1) / kSortTile;
+    size_t off = 0;
+    w.keys_alt = off;
+    off = align(off + (size_t)k * 8);
+    w.values_alt = off;
+    off = align(off + (size_t)k * 4);
+    w.global_hist = off;
+    off = align(off + (size_t)w.passes * kRadix * 4);
+    w.counters = off;
+    off = align(off + (size_t)(w.passes + 1) * 4);
+    w.status = off;
+    off = align(off + (size_t)w.passes * (size_t)w.tiles * kRadix * 4);
+    w.bytes = off;
+    return w;
+}
+
+ForwardWorkspace forward_workspace(int64_t k, int num_tiles)
+{
+    auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    ForwardWorkspace w;
+    size_t off = 0;
+    w.keys = off;
+    off = align(off + (size_t)k * 8);
+    w.values = off;
+    off = align(off + (size_t)k * 4);
+    w.sort = off;
+    off += sort_workspace(k, num_tiles).bytes;
+    w.bytes = align(off);
+    return w;
+}
+
+// Histogram of every digit of every key in one read of the keys.  Lanes that hold the same
+// digit are merged with ballots first, so the LDS atomics never collide inside a wavefront
+// (emission order puts long runs of equal depth bits next to each other).
+__global__ __launch_bounds__(256) void radix_hist_kernel(const int64_t* __restrict__ keys, int64_t k, int passes,
+                                                         uint32_t* __restrict__ global_hist)
+{
+    __shared__ uint32_t hist[8 * kRadix];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    for(int j = tid; j < passes * kRadix; j += 256)
+        hist[j] = 0;
+    __syncthreads();
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const int64_t rounds = (k + stride - 1) / stride;
+    for(int64_t r = 0; r < rounds; ++r)
+    {
+        const int64_t i = r * stride + (int64_t)blockIdx.x * 256 + tid;
+        const bool valid = i < k;
+        const uint64_t s = valid ? sortable(keys[i]) : 0ull;
+        for(int p = 0; p < passes; ++p)
+        {
+            const uint32_t d = (uint32_t)(s >> (p * kRadixBits)) & (kRadix - 1);
+            const uint64_t m = match_digit(d, valid);
+            if(valid && (m & lanemask_lt(lane)) == 0)
+                atomicAdd(&hist[p * kRadix + d], (uint32_t)__popcll(m));
+        }
+    }
+    __syncthreads();
+    for(int j = tid; j < passes * kRadix; j += 256)
+        if(hist[j])
+            atomicAdd(&global_hist[j], hist[j]);
+}
+
+// exclusive scan of each pass's 256 bins (one wave-sized job per pass)
+__global__ __launch_bounds__(256) void radix_hist_scan_kernel(uint32_t* global_hist)
+{
+    __shared__ uint32_t wave_tot[4];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    uint32_t* h = global_hist + blockIdx.x * kRadix;
+    const uint32_t v = h[tid];
+    const uint32_t incl = wave_incl_scan_u32(v, lane);
+    if(lane == 63)
+        wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t prefix = 0;
+    for(int w = 0; w < wave; ++w)
+        prefix += wave_tot[w];
+    h[tid] = prefix + incl - v;
+}
+
+constexpr uint32_t kFlagAggregate = 1u << 30;
+constexpr uint32_t kFlagInclusive = 2u << 30;
+constexpr uint32_t kFlagMask = 3u << 30;
+constexpr uint32_t kValueMask = ~kFlagMask;
+constexpr int kSpinLimit = 1 << 18; // bounded wait: a stuck predecessor ends in an error flag, not a hang
+
+// One digit pass.  Tile = 4096 consecutive keys, taken in arrival order through a dynamic
+// counter so that every tile a workgroup waits for has already started.  Stable ranking:
+// wave-local rank by ballot matching (item by item, lane by lane), waves in tile order,
+// tiles in chained-scan order.  Keys are reordered through LDS so that global stores of one
+// digit are contiguous.
+__global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
+    const int64_t* __restrict__ keys_in, const int32_t* __restrict__ vals_in, int64_t* __restrict__ keys_out,
+    int32_t* __restrict__ vals_out, int64_t k, int shift, const uint32_t* __restrict__ hist_excl,
+    uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag)
+{
+    __shared__ int64_t s_keys[kSortTile];
+    __shared__ int32_t s_vals[kSortTile];
+    __shared__ uint32_t s_whist[4][kRadix];
+    __shared__ uint32_t s_digit_start[kRadix];
+    __shared__ uint32_t s_gbase[kRadix];
+    __shared__ uint32_t s_wave_tot[4];
+    __shared__ uint32_t s_tile;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+
+    if(tid == 0)
+        s_tile = atomicAdd(tile_counter, 1u);
+#pragma unroll
+    for(int w = 0; w < 4; ++w)
+        s_whist[w][tid] = 0;
+    __syncthreads();
+    const int64_t tile = s_tile;
+    const int64_t tile_base = tile * kSortTile;
+    const int tile_n = (int)min((int64_t)kSortTile, k - tile_base);
+
+    // ---- load (striped inside each wavefront: coalesced, order = (item, lane)) -------------
+    int64_t key[kSortItems];
+    int32_t val[kSortItems];
+    uint32_t rank[kSortItems];
+#pragma unroll
+    for(int it = 0; it < kSortItems; ++it)
+    {
+        const int local = wave * (kSortItems * 64) + it * 64 + lane;
+        if(local < tile_n)
+        {
+            key[it] = __builtin_nontemporal_load(keys_in + tile_base + local);
+            val[it] = __builtin_nontemporal_load(vals_in + tile_base + local);
+        }
+        else
+        {
+            key[it] = 0;
+            val[it] = 0;
+        }
+    }
+
+    // ---- wave-local stable rank -----------------------------------------------------------
+    volatile uint32_t* wh = s_whist[wave];
+#pragma unroll
+    for(int it = 0; it < kSortItems; ++it)
+    {
+        const int local = wave * (kSortItems * 64) + it * 64 + lane;
+        const bool valid = local < tile_n;
+        const uint32_t d = (uint32_t)(sortable(key[it]) >> shift) & (kRadix - 1);
+        const uint64_t m = match_digit(d, valid);
+        const uint32_t below = (uint32_t)__popcll(m & lanemask_lt(lane));
+        const uint32_t old = wh[d];
+        __builtin_amdgcn_wave_barrier();
+        if(valid && below == 0)
+            wh[d] = old + (uint32_t)__popcll(m);
+        __builtin_amdgcn_wave_barrier();
+        rank[it] = old + below;
+    }
+    __syncthreads();
+
+    // ---- per-digit totals of the tile (thread d <-> digit d), wave offsets, digit starts ----
+    uint32_t total;
+    {
+        const uint32_t c0 = s_whist[0][tid], c1 = s_whist[1][tid], c2 = s_whist[2][tid], c3 = s_whist[3][tid];
+        s_whist[0][tid] = 0;
+        s_whist[1][tid] = c0;
+        s_whist[2][tid] = c0 + c1;
+        s_whist[3][tid] = c0 + c1 + c2;
+        total = c0 + c1 + c2 + c3;
+    }
+    // publish this tile's count as soon as it is known
+    uint32_t* my_status = status + tile * kRadix + tid;
+    __hip_atomic_store(my_status, total | (tile == 0 ? kFlagInclusive : kFlagAggregate), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    {
+        const uint32_t incl = wave_incl_scan_u32(total, lane);
+        if(lane == 63)
+            s_wave_tot[wave] = incl;
+        __syncthreads();
+        uint32_t prefix = 0;
+        for(int w = 0; w < wave; ++w)
+            prefix += s_wave_tot[w];
+        s_digit_start[tid] = prefix + incl - total;
+    }
+    __syncthreads();
+
+    // ---- keys into LDS in tile-sorted order ----------------------------------------------
+#pragma unroll
+    for(int it = 0; it < kSortItems; ++it)
+    {
+        const int local = wave * (kSortItems * 64) + it * 64 + lane;
+        if(local < tile_n)
+        {
+            const uint32_t d = (uint32_t)(sortable(key[it]) >> shift) & (kRadix - 1);
+            const uint32_t pos = s_digit_start[d] + s_whist[wave][d] + rank[it];
+            s_keys[pos] = key[it];
+            s_vals[pos] = val[it];
+        }
+    }
+
+    // ---- chained scan over earlier tiles (decoupled look-back), one thread per digit -------
+    {
+        uint32_t excl = 0;
+        if(tile > 0)
+        {
+            int64_t t = tile - 1;
+            int spins = 0;
+            while(true)
+            {
+                const uint32_t v =
+                    __hip_atomic_load(status + t * kRadix + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if((v & kFlagMask) == 0)
+                {
+                    if(++spins > kSpinLimit)
+                    {
+                        *error_flag = 1u;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                    continue;
+                }
+                excl += v & kValueMask;
+                if((v & kFlagInclusive) || t == 0)
+                    break;
+                --t;
+            }
+            __hip_atomic_store(my_status, ((excl + total) & kValueMask) | kFlagInclusive, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        s_gbase[tid] = hist_excl[tid] + excl - s_digit_start[tid];
+    }
+    __syncthreads();
+
+    // ---- scatter: consecutive threads -> consecutive addresses inside a digit's run --------
+#pragma unroll
+    for(int it = 0; it < kSortItems; ++it)
+    {
+        const int j = it * kSortThreads + tid;
+        if(j < tile_n)
+        {
+            const int64_t kk = s_keys[j];
+            const uint32_t d = (uint32_t)(sortable(kk) >> shift) & (kRadix - 1);
+            const uint32_t out = s_gbase[d] + (uint32_t)j;
+            keys_out[out] = kk;
+            vals_out[out] = s_vals[j];
+        }
+    }
+}
+
+int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values_a, int64_t* keys_b,
+                      int32_t* values_b, void* sort_ws, hipStream_t stream, int64_t** keys_out,
+                      int32_t** values_out)
+{
+    *keys_out = keys_a;
+    *values_out = values_a;
+    if(k <= 1)
+        return DSX_OK;
+    if(k >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
+    const SortWorkspace w = sort_workspace(k, num_tiles);
+    char* base = static_cast<char*>(sort_ws);
+    uint32_t* global_hist = reinterpret_cast<uint32_t*>(base + w.global_hist);
+    uint32_t* counters = reinterpret_cast<uint32_t*>(base + w.counters);
+    uint32_t* status = reinterpret_cast<uint32_t*>(base + w.status);
+    // global_hist, counters and status are adjacent: clear them with one fill
+    const int64_t clear_words = (int64_t)((w.bytes - w.global_hist) / 4);
+    int rc = launch_fill_u32(global_hist, clear_words, 0u, stream);
+    if(rc)
+        return rc;
+    const int hist_blocks = (int)min((int64_t)2048, (k + 255) / 256);
+    hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks), dim3(256), 0, stream, keys_a, k, w.passes, global_hist);
+    DSX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(radix_hist_scan_kernel, dim3(w.passes), dim3(256), 0, stream, global_hist);
+    DSX_LAUNCH_CHECK();
+    int64_t* kin = keys_a;
+    int32_t* vin = values_a;
+    int64_t* kout = keys_b;
+    int32_t* vout = values_b;
+    for(int p = 0; p < w.passes; ++p)
+    {
+        hipLaunchKernelGGL(radix_onesweep_kernel, dim3((unsigned)w.tiles), dim3(kSortThreads), 0, stream, kin, vin,
+                           kout, vout, k, p * kRadixBits, global_hist + p * kRadix,
+                           status + (size_t)p * w.tiles * kRadix, counters + p, counters + w.passes);
+        DSX_LAUNCH_CHECK();
+        int64_t* tk = kin;
+        kin = kout;
+        kout = tk;
+        int32_t* tv = vin;
+        vin = vout;
+        vout = tv;
+    }
+    *keys_out = kin;
+    *values_out = vin;
+    return DSX_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// tile ranges
+// ---------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void ranges_init_kernel(int32_t* ranges, int num_tiles, int32_t k)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if(i < num_tiles)
+        ranges[i] = 0;
+    else if(i == num_tiles)
+        ranges[i] = k;
+}
+
+// where the tile field changes between neighbours, the next index starts the following tile
+__global__ __launch_bounds__(256) void ranges_boundaries_kernel(const int64_t* __restrict__ keys, int64_t k,
+                                                                int32_t* ranges)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if(i + 1 < k)
+    {
+        const int32_t cur = (int32_t)(keys[i] >> 32);
+        const int32_t nxt = (int32_t)(keys[i + 1] >> 32);
+        if(cur != nxt)
+            ranges[cur + 1] = (int32_t)(i + 1);
+    }
+}
+
+// inclusive running maximum over num_tiles+1 entries (one workgroup): empty tiles inherit the
+// end of the previous run
+__global__ __launch_bounds__(1024) void ranges_maxscan_kernel(int32_t* ranges, int count)
+{
+    __shared__ int wave_max[16];
+    __shared__ int carry_s;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    if(tid == 0)
+        carry_s = INT32_MIN;
+    __syncthreads();
+    for(int base = 0; base < count; base += 1024)
+    {
+        const int i = base + tid;
+        const int v = i < count ? ranges[i] : INT32_MIN;
+        int incl = wave_incl_max_i32(v, lane);
+        if(lane == 63)
+            wave_max[wave] = incl;
+        __syncthreads();
+        int prev = carry_s;
+        for(int w = 0; w < wave; ++w)
+            prev = max(prev, wave_max[w]);
+        incl = max(incl, prev);
+        if(i < count)
+            ranges[i] = incl;
+        __syncthreads();
+        if(tid == 1023)
+            carry_s = incl;
+        __syncthreads();
+    }
+}
+
+int launch_tile_ranges(int64_t k, const int64_t* sorted_keys, int num_tiles, int32_t* ranges, hipStream_t stream)
+{
+    const int count = num_tiles + 1;
+    hipLaunchKernelGGL(ranges_init_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, ranges, num_tiles,
+                       (int32_t)k);
+    DSX_LAUNCH_CHECK();
+    if(k > 1)
+    {
+        hipLaunchKernelGGL(ranges_boundaries_kernel, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, stream,
+                           sorted_keys, k, ranges);
+        DSX_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(ranges_maxscan_kernel, dim3(1), dim3(1024), 0, stream, ranges, count);
+    DSX_LAUNCH_CHECK();
+    return DSX_OK;
+}
+
+} // namespace dsx

@@ -1,0 +1,370 @@
+// Stage 1: per-Gaussian projection for gfx950.
+//
+// One thread per Gaussian, 256 per workgroup (4 wave64).  Each wavefront copies the
+// spherical-harmonics rows of its 64 Gaussians (a contiguous 12 KB span at degree 3) into LDS
+// with 16-byte coalesced loads and then every lane reads its own row back with an odd LDS
+// pitch (conflict free), so the 192-byte AoS rows never produce strided HBM traffic; only
+// the columns the active degree needs are fetched.
+//
+// This translation unit is compiled with floating-point contraction OFF and uses only
+// + - * / sqrt on binary32: radii, tile counts and depth keys are integers derived from these
+// floats and must not depend on the compiler's choice of fused multiply-adds.
+// Behaviour follows cpp/rasterizer_kernels.cu:57-161 of the reference; rsqrtf there (an
+// approximate instruction) is evaluated as 1/sqrt so results are reproducible.
+#include "dsx_common.h"
+
+#pragma clang fp contract(off)
+
+namespace dsx
+{
+
+constexpr int kShPitch = 49; // floats per row in LDS (48 coefficients, odd pitch)
+
+struct ProjectParams
+{
+    int64_t n;
+    const float* means3d;
+    const float* scales;
+    const float* quats;
+    const float* opacities;
+    const float* shs;
+    const float* cov3d_precomp;
+    const float* colors_precomp;
+    const float* view;
+    const float* proj;
+    const float* campos;
+    float4* splats;
+    int32_t* radii;
+    float* cov3d;
+    uint32_t* block_sums;
+    float focal_x, focal_y, tanfovx, tanfovy, c_x, c_y, scale_modifier;
+    int sh_degree, sh_stride; // active degree; floats per shs row
+    int ntx, nty;
+};
+
+// cov3D = (R S)(R S)^T from scale and (w,x,y,z) quaternion; cpp/rasterizer_kernels.cu:615-659
+__device__ __forceinline__ void cov3d_from_scale_rot(const float* sc, float4 q, float mod, float* out)
+{
+    float r = q.x, x = q.y, y = q.z, z = q.w;
+    const float inv_norm = 1.0f / sqrtf(r * r + x * x + y * y + z * z);
+    r = r * inv_norm;
+    x = x * inv_norm;
+    y = y * inv_norm;
+    z = z * inv_norm;
+    const float s0 = sc[0] * mod, s1 = sc[1] * mod, s2 = sc[2] * mod;
+    const float r00 = 1.0f - 2.0f * (y * y + z * z);
+    const float r01 = 2.0f * (x * y - r * z);
+    const float r02 = 2.0f * (x * z + r * y);
+    const float r10 = 2.0f * (x * y + r * z);
+    const float r11 = 1.0f - 2.0f * (x * x + z * z);
+    const float r12 = 2.0f * (y * z - r * x);
+    const float r20 = 2.0f * (x * z - r * y);
+    const float r21 = 2.0f * (y * z + r * x);
+    const float r22 = 1.0f - 2.0f * (x * x + y * y);
+    const float m00 = s0 * r00, m01 = s1 * r01, m02 = s2 * r02;
+    const float m10 = s0 * r10, m11 = s1 * r11, m12 = s2 * r12;
+    const float m20 = s0 * r20, m21 = s1 * r21, m22 = s2 * r22;
+    out[0] = m00 * m00 + m01 * m01 + m02 * m02;
+    out[1] = m00 * m10 + m01 * m11 + m02 * m12;
+    out[2] = m00 * m20 + m01 * m21 + m02 * m22;
+    out[3] = m10 * m10 + m11 * m11 + m12 * m12;
+    out[4] = m10 * m20 + m11 * m21 + m12 * m22;
+    out[5] = m20 * m20 + m21 * m21 + m22 * m22;
+}
+
+// SH degree 0..3 -> RGB (+0.5, clamped at 0); f = this Gaussian's coefficient row in LDS.
+// Term order as cpp/rasterizer_kernels.cu:433-554.
+__device__ __forceinline__ float3 sh_to_rgb(int deg, const float* f, float3 mean, float3 cam)
+{
+    const float C0 = 0.28209479177387814f;
+    float rx = 0.0f + C0 * f[0];
+    float ry = 0.0f + C0 * f[1];
+    float rz = 0.0f + C0 * f[2];
+    if(deg >= 1)
+    {
+        const float dx = mean.x - cam.x, dy = mean.y - cam.y, dz = mean.z - cam.z;
+        const float inv_norm = 1.0f / sqrtf(dx * dx + dy * dy + dz * dz);
+        const float vx = dx * inv_norm, vy = dy * inv_norm, vz = dz * inv_norm;
+        const float C1 = 0.4886025119029199f;
+        rx += C1 * (-vy * f[3] + vz * f[6] - vx * f[9]);
+        ry += C1 * (-vy * f[4] + vz * f[7] - vx * f[10]);
+        rz += C1 * (-vy * f[5] + vz * f[8] - vx * f[11]);
+        if(deg >= 2)
+        {
+            const float xx = vx * vx, yy = vy * vy, zz = vz * vz;
+            const float xy = vx * vy, xz = vx * vz, yz = vy * vz;
+            const float A0 = 1.0925484305920792f, A1 = -1.0925484305920792f, A2 = 0.31539156525252005f,
+                        A3 = -1.0925484305920792f, A4 = 0.5462742152960396f;
+            const float q2 = 2.0f * zz - xx - yy, q4 = xx - yy;
+            rx += A0 * xy * f[12] + A1 * yz * f[15] + A2 * q2 * f[18] + A3 * xz * f[21] + A4 * q4 * f[24];
+            ry += A0 * xy * f[13] + A1 * yz * f[16] + A2 * q2 * f[19] + A3 * xz * f[22] + A4 * q4 * f[25];
+            rz += A0 * xy * f[14] + A1 * yz * f[17] + A2 * q2 * f[20] + A3 * xz * f[23] + A4 * q4 * f[26];
+            if(deg >= 3)
+            {
+                const float B0 = -0.5900435899266435f, B1 = 2.890611442640554f, B2 = -0.4570457994644658f,
+                            B3 = 0.3731763325901154f, B4 = -0.4570457994644658f, B5 = 1.445305721320277f,
+                            B6 = -0.5900435899266435f;
+                const float t0 = B0 * vy * (3.0f * xx - yy);
+                const float t1 = B1 * xy * vz;
+                const float t2 = B2 * vy * (4.0f * zz - xx - yy);
+                const float t3 = B3 * vz * (2.0f * zz - 3.0f * xx - 3.0f * yy);
+                const float t4 = B4 * vx * (4.0f * zz - xx - yy);
+                const float t5 = B5 * vz * (xx - yy);
+                const float t6 = B6 * vx * (xx - 3.0f * yy);
+                rx += t0 * f[27] + t1 * f[30] + t2 * f[33] + t3 * f[36] + t4 * f[39] + t5 * f[42] + t6 * f[45];
+                ry += t0 * f[28] + t1 * f[31] + t2 * f[34] + t3 * f[37] + t4 * f[40] + t5 * f[43] + t6 * f[46];
+                rz += t0 * f[29] + t1 * f[32] + t2 * f[35] + t3 * f[38] + t4 * f[41] + t5 * f[44] + t6 * f[47];
+            }
+        }
+    }
+    return make_float3(fmaxf(rx + 0.5f, 0.0f), fmaxf(ry + 0.5f, 0.0f), fmaxf(rz + 0.5f, 0.0f));
+}
+
+__global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectParams p)
+{
+    __shared__ float sh_lds[4][64 * kShPitch];
+    __shared__ uint32_t wave_sums[4];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int64_t i = (int64_t)blockIdx.x * kProjBlock + tid;
+    const bool live = i < p.n;
+
+    // ---- stage this wavefront's SH rows through LDS (coalesced) -----------------------------
+    const bool use_sh = p.colors_precomp == nullptr;
+    if(use_sh)
+    {
+        const int64_t row0 = (int64_t)blockIdx.x * kProjBlock + wave * 64;
+        const int rows = (int)max((int64_t)0, min((int64_t)64, p.n - row0));
+        const int need = (p.sh_degree + 1) * (p.sh_degree + 1) * 3; // floats per row actually used
+        float* dst = sh_lds[wave];
+        if(p.sh_stride == 48 && ((uintptr_t)p.shs & 15) == 0)
+        {
+            const float4* src = reinterpret_cast<const float4*>(p.shs + row0 * 48);
+            const int chunks = rows * 12;
+            const int need4 = (need + 3) >> 2;
+#pragma unroll
+            for(int j = 0; j < 12; ++j)
+            {
+                const int e = j * 64 + lane;
+                const int row = e / 12;
+                const int c4 = e - row * 12;
+                if(e < chunks && c4 < need4)
+                {
+                    const float4 v = nt_load_f4(src + e);
+                    float* d = dst + row * kShPitch + c4 * 4;
+                    d[0] = v.x;
+                    d[1] = v.y;
+                    d[2] = v.z;
+                    d[3] = v.w;
+                }
+            }
+        }
+        else
+        {
+            const float* src = p.shs + row0 * p.sh_stride;
+            const int total = rows * p.sh_stride;
+            for(int e = lane; e < total; e += 64)
+            {
+                const int row = e / p.sh_stride;
+                const int c = e - row * p.sh_stride;
+                if(c < need)
+                    dst[row * kShPitch + c] = src[e];
+            }
+        }
+    }
+    __syncthreads();
+
+    uint32_t count = 0;
+    if(live)
+    {
+        const float3 mean = make_float3(p.means3d[3 * i], p.means3d[3 * i + 1], p.means3d[3 * i + 2]);
+
+        float c3[6];
+        if(p.cov3d_precomp)
+        {
+#pragma unroll
+            for(int j = 0; j < 6; ++j)
+                c3[j] = p.cov3d_precomp[6 * i + j];
+        }
+        else
+        {
+            const float sc[3] = {p.scales[3 * i], p.scales[3 * i + 1], p.scales[3 * i + 2]};
+            const float4 q = reinterpret_cast<const float4*>(p.quats)[i];
+            cov3d_from_scale_rot(sc, q, p.scale_modifier, c3);
+        }
+        {
+            float2* o = reinterpret_cast<float2*>(p.cov3d + 6 * i);
+            o[0] = make_float2(c3[0], c3[1]);
+            o[1] = make_float2(c3[2], c3[3]);
+            o[2] = make_float2(c3[4], c3[5]);
+        }
+
+        float3 rgb;
+        if(use_sh)
+        {
+            float f[48];
+            const float* row = sh_lds[wave] + lane * kShPitch;
+            const int need = (p.sh_degree + 1) * (p.sh_degree + 1) * 3;
+#pragma unroll
+            for(int j = 0; j < 48; ++j)
+                f[j] = j < need ? row[j] : 0.0f;
+            const float3 cam = make_float3(p.campos[0], p.campos[1], p.campos[2]);
+            rgb = sh_to_rgb(p.sh_degree, f, mean, cam);
+        }
+        else
+        {
+            rgb = make_float3(p.colors_precomp[3 * i], p.colors_precomp[3 * i + 1], p.colors_precomp[3 * i + 2]);
+        }
+
+        // frustum test on the centre: strict NDC box, z_ndc > 0.1 (cpp/rasterizer_kernels.cu:7-24)
+        const float* P = p.proj;
+        const float inv_w = 1.0f / (P[12] * mean.x + P[13] * mean.y + P[14] * mean.z + P[15]);
+        const float nx = inv_w * (P[0] * mean.x + P[1] * mean.y + P[2] * mean.z + P[3]);
+        const float ny = inv_w * (P[4] * mean.x + P[5] * mean.y + P[6] * mean.z + P[7]);
+        const float nz = inv_w * (P[8] * mean.x + P[9] * mean.y + P[10] * mean.z + P[11]);
+        const bool in_frustum = nx > -1.0f && nx < 1.0f && ny > -1.0f && ny < 1.0f && nz > 0.1f;
+
+        // view-space position (cpp/rasterizer_kernels.cu:325-330)
+        const float* V = p.view;
+        const float vx = V[0] * mean.x + V[1] * mean.y + V[2] * mean.z + V[3];
+        const float vy = V[4] * mean.x + V[5] * mean.y + V[6] * mean.z + V[7];
+        const float vz = V[8] * mean.x + V[9] * mean.y + V[10] * mean.z + V[11];
+
+        // EWA covariance (cpp/rasterizer_kernels.cu:174-231): sums start from 0 and add the
+        // three products in index order, zero Jacobian entries included
+        const float limx = 1.3f * p.tanfovx;
+        const float limy = 1.3f * p.tanfovy;
+        const float txtz = vx / vz;
+        const float tytz = vy / vz;
+        const float t0 = fminf(limx, fmaxf(-limx, txtz)) * vz;
+        const float t1 = fminf(limy, fmaxf(-limy, tytz)) * vz;
+        const float t2 = vz;
+        const float J[3][3] = {{p.focal_x / t2, 0.0f, -(p.focal_x * t0) / (t2 * t2)},
+                               {0.0f, p.focal_y / t2, -(p.focal_y * t1) / (t2 * t2)},
+                               {0.0f, 0.0f, 0.0f}};
+        const float Wm[3][3] = {{V[0], V[4], V[8]}, {V[1], V[5], V[9]}, {V[2], V[6], V[10]}};
+        float T[3][3];
+#pragma unroll
+        for(int a = 0; a < 3; ++a)
+#pragma unroll
+            for(int b = 0; b < 3; ++b)
+            {
+                float acc = 0.0f;
+#pragma unroll
+                for(int k = 0; k < 3; ++k)
+                    acc += Wm[a][k] * J[b][k];
+                T[a][b] = acc;
+            }
+        const float S3[3][3] = {{c3[0], c3[1], c3[2]}, {c3[1], c3[3], c3[4]}, {c3[2], c3[4], c3[5]}};
+        float tmp[3][3];
+#pragma unroll
+        for(int a = 0; a < 3; ++a)
+#pragma unroll
+            for(int b = 0; b < 3; ++b)
+            {
+                float acc = 0.0f;
+#pragma unroll
+                for(int k = 0; k < 3; ++k)
+                    acc += T[k][a] * S3[k][b];
+                tmp[a][b] = acc;
+            }
+        float cov[2][2];
+#pragma unroll
+        for(int a = 0; a < 2; ++a)
+#pragma unroll
+            for(int b = 0; b < 2; ++b)
+            {
+                float acc = 0.0f;
+#pragma unroll
+                for(int k = 0; k < 3; ++k)
+                    acc += tmp[a][k] * T[k][b];
+                cov[a][b] = acc;
+            }
+        const float ca = cov[0][0] + 0.3f;
+        const float cb = cov[0][1];
+        const float cc = cov[1][1] + 0.3f;
+
+        // pixel mean (cpp/rasterizer_kernels.cu:332-337)
+        const float z_inv = 1.0f / (vz + 1e-6f);
+        const float px = p.focal_x * vx * z_inv + p.c_x;
+        const float py = p.focal_y * vy * z_inv + p.c_y;
+
+        // radius = ceil(3 sigma_max), zero when culled (cpp/rasterizer_kernels.cu:163-172)
+        const float det = ca * cc - cb * cb;
+        const float mid = 0.5f * (ca + cc);
+        const float diff = mid * mid - det;
+        const float root = sqrtf(fmaxf(0.1f, diff));
+        const float lambda1 = mid + root;
+        const float lambda2 = mid - root;
+        const float keep = (det > 1e-6f && in_frustum) ? 1.0f : 0.0f;
+        const int radius = f2i_sat(ceilf(3.0f * sqrtf(fmaxf(lambda1, lambda2))) * keep);
+
+        const TileRect r = tile_rect(px, py, radius, p.ntx, p.nty);
+        const int tiles = (r.ex - r.sx) * (r.ey - r.sy) * (radius > 0 ? 1 : 0);
+
+        // conic (cpp/rasterizer_kernels.cu:49-55)
+        const float det_inv = 1.0f / (det + 1e-6f);
+        const float opacity = p.opacities[i];
+
+        float4* rec = p.splats + 3 * i;
+        rec[0] = make_float4(px, py, vz, __int_as_float(radius));
+        rec[1] = make_float4(cc * det_inv, -cb * det_inv, ca * det_inv, opacity);
+        rec[2] = make_float4(rgb.x, rgb.y, rgb.z, __int_as_float(tiles));
+        p.radii[i] = radius;
+
+        // the last Gaussian never emits keys (cpp/rasterizer_torch.cu:99-104)
+        count = (i == p.n - 1) ? 0u : (uint32_t)tiles;
+    }
+
+    const uint32_t ws = wave_sum_u32(count);
+    if(lane == 0)
+        wave_sums[wave] = ws;
+    __syncthreads();
+    if(tid == 0)
+        p.block_sums[blockIdx.x] = wave_sums[0] + wave_sums[1] + wave_sums[2] + wave_sums[3];
+}
+
+int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, const float* scales,
+                       const float* quats, const float* opacities, const float* shs,
+                       const float* cov3d_precomp, const float* colors_precomp, float* splats, int32_t* radii,
+                       float* cov3d, uint32_t* block_sums, hipStream_t stream)
+{
+    if(n == 0)
+        return DSX_OK;
+    ProjectParams p;
+    p.n = n;
+    p.means3d = means3d;
+    p.scales = scales;
+    p.quats = quats;
+    p.opacities = opacities;
+    p.shs = shs;
+    p.cov3d_precomp = cov3d_precomp;
+    p.colors_precomp = colors_precomp;
+    p.view = cam.view;
+    p.proj = cam.proj;
+    p.campos = cam.campos;
+    p.splats = reinterpret_cast<float4*>(splats);
+    p.radii = radii;
+    p.cov3d = cov3d;
+    p.block_sums = block_sums;
+    // cpp/rasterizer_torch.cu:144-147
+    p.focal_y = cam.image_height / (2 * cam.tanfovy);
+    p.focal_x = cam.image_width / (2 * cam.tanfovx);
+    p.c_x = cam.image_width / 2.0f;
+    p.c_y = cam.image_height / 2.0f;
+    p.tanfovx = cam.tanfovx;
+    p.tanfovy = cam.tanfovy;
+    p.scale_modifier = cam.scale_modifier;
+    p.sh_degree = cam.sh_degree;
+    p.sh_stride = (cam.max_sh_degree + 1) * (cam.max_sh_degree + 1) * 3;
+    p.ntx = tiles_x(cam.image_width);
+    p.nty = tiles_y(cam.image_height);
+    const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
+    hipLaunchKernelGGL(project_fwd_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, p);
+    DSX_LAUNCH_CHECK();
+    return DSX_OK;
+}
+
+} // namespace dsx

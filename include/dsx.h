@@ -1,0 +1,190 @@
+/*
+ * dsx — C ABI of the MI355X (gfx950) 3D-Gaussian-Splatting rasterizer.
+ *
+ * Plain pointers and sizes only; no torch types.  Every pointer is DEVICE memory unless it
+ * is marked "host".  `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ * The library allocates nothing on the device: outputs and workspace are the caller's.
+ * All functions return 0 on success or a negative dsx_status; dsx_error_string() explains it.
+ * Functions are re-entrant: no global mutable state, so different streams / devices may be
+ * driven concurrently by different host threads (each call uses the current HIP device).
+ *
+ * What each entry point replaces in the reference (deepsense-ai/ds-splat) is cited as
+ * file:line next to it.  Matrices are row-major, math convention (translation in elements
+ * 3, 7, 11): what the reference's native code receives after ds_splat/rasterizer.py:147-148
+ * transposed the user's matrices.
+ */
+#ifndef DSX_H_
+#define DSX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DSX_TILE 16            /* cpp/rasterizer_kernels.cuh:6 */
+#define DSX_SPLAT_FLOATS 12    /* projected record, 48 bytes (3 x float4) */
+#define DSX_GRAD_FLOATS 12     /* screen-space gradient accumulator record, 48 bytes */
+#define DSX_PROJ_BLOCK 256     /* Gaussians per workgroup in the per-Gaussian kernels */
+
+typedef enum dsx_status
+{
+    DSX_OK = 0,
+    DSX_ERR_BAD_ARG = -1,      /* NULL where data is required, negative size, bad degree ... */
+    DSX_ERR_LAUNCH = -2,       /* hipGetLastError() after a launch reported a failure       */
+    DSX_ERR_RUNTIME = -3,      /* a HIP runtime call (memcpy, sync, event) failed           */
+    DSX_ERR_TOO_LARGE = -4,    /* sizes beyond 32-bit indexing of keys (K >= 2^30)          */
+    DSX_ERR_WORKSPACE = -5     /* workspace smaller than dsx_workspace_bytes() asks for     */
+} dsx_status;
+
+/* Mirrors TorchRasterizationSettings, cpp/ds_cuda_rasterizer/rasterizer_torch.hpp:7-22.
+ * `prefiltered` and `debug` are carried by the reference but never read; they are omitted. */
+typedef struct dsx_camera
+{
+    int32_t image_height;
+    int32_t image_width;
+    float tanfovx;
+    float tanfovy;
+    float scale_modifier;
+    int32_t sh_degree;      /* active degree, 0..3                                  */
+    int32_t max_sh_degree;  /* row stride of shs is (max_sh_degree+1)^2 * 3 floats  */
+    const float* view;      /* device float[16], row-major world->view              */
+    const float* proj;      /* device float[16], row-major world->clip              */
+    const float* campos;    /* device float[3]                                      */
+    const float* bg;        /* device float[3]                                      */
+} dsx_camera;
+
+/*
+ * Projected record ("splat"), one per Gaussian, DSX_SPLAT_FLOATS floats:
+ *   [0] pixel x   [1] pixel y   [2] view depth   [3] radius (int32 bits)
+ *   [4] conic a   [5] conic b   [6] conic c      [7] opacity
+ *   [8] red       [9] green     [10] blue        [11] tiles touched (int32 bits)
+ * It plays the role of the reference's 48-byte `Gaussian` (cpp/rasterizer_kernels.cuh:18-26).
+ *
+ * Gradient accumulator record, DSX_GRAD_FLOATS floats:
+ *   [0] v_x [1] v_y [2] v_conic_a [3] v_conic_b [4] v_conic_c [5] v_opacity
+ *   [6] v_red [7] v_green [8] v_blue [9..11] unused
+ */
+
+const char* dsx_error_string(int status);
+int dsx_version(void);
+
+/* number of workgroups of the per-Gaussian kernels = entries of `block_sums` */
+int64_t dsx_num_blocks(int64_t n);
+/* tiles of an image, and radix passes the sort runs for that many tiles */
+int32_t dsx_num_tiles(int32_t width, int32_t height);
+int32_t dsx_sort_passes(int32_t num_tiles);
+/* bytes of `workspace` dsx_forward_finish / dsx_sort_pairs need for k keys */
+size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height);
+
+/* ------------------------------------------------------------------------------------ */
+/* Per-stage entry points (each one individually parity-tested and timed)                */
+/* ------------------------------------------------------------------------------------ */
+
+/* Stage 1 — replaces rasterizer_preprocessing_kernel, cpp/rasterizer_kernels.cu:57-161 and
+ * its launcher cpp/rasterizer_torch.cu:115-168.  Writes splats[n*12], radii[n], cov3d[n*6]
+ * and block_sums[dsx_num_blocks(n)] (tile count of each 256-Gaussian block; the last
+ * Gaussian counts as zero, cpp/rasterizer_torch.cu:99-104).  shs may be NULL iff
+ * colors_precomp is given; scales/quats may be NULL iff cov3d_precomp is given (then cov3d
+ * receives a copy). */
+int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
+                    const float* quats, const float* opacities, const float* shs,
+                    const float* cov3d_precomp, const float* colors_precomp, float* splats,
+                    int32_t* radii, float* cov3d, uint32_t* block_sums, void* stream);
+
+/* Exclusive prefix of `count` uint32 values in place, total written to *total (device).
+ * Replaces the in-block Hillis-Steele scan of cpp/rasterizer_kernels.cu:131-142 together
+ * with thrust::exclusive_scan, cpp/rasterizer_torch.cu:95. */
+int dsx_scan_u32(int64_t count, uint32_t* data, uint32_t* total, void* stream);
+
+/* Stage 2a — replaces calculate_keys_and_indices_kernel, cpp/rasterizer_kernels.cu:252-306.
+ * block_offsets = scanned block_sums.  keys[k] = (tile << 32) | sign-extended depth bits,
+ * values[k] = Gaussian index, in emission order. */
+int dsx_emit_keys(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
+                  const uint32_t* block_offsets, int64_t* keys, int32_t* values, void* stream);
+
+/* Stage 2b — replaces thrust::sort_by_key, cpp/rasterizer_torch.cu:70-76: stable ascending
+ * sort of (int64 key, int32 value) pairs where every key is (tile << 32 | depth bits) with
+ * tile in [0, num_tiles) or a negative key (tile field all ones).  keys/values are sorted
+ * in place; workspace needs dsx_workspace_bytes(0, k, ...) bytes. */
+int dsx_sort_pairs(int64_t k, int32_t num_tiles, int64_t* keys, int32_t* values, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/* Stage 3 — replaces identify_tile_ranges + identify_tile_ranges_kernel +
+ * thrust::inclusive_scan(max), cpp/rasterizer_torch.cu:23-42, cpp/rasterizer_kernels.cu:308-323.
+ * ranges has num_tiles+1 entries. */
+int dsx_tile_ranges(int64_t k, const int64_t* sorted_keys, int32_t num_tiles, int32_t* ranges,
+                    void* stream);
+
+/* Stage 4 — replaces rasterizer_cuda_forward + render_image_kernel,
+ * cpp/rasterizer_torch.cu:44-68, cpp/rasterizer_kernels.cu:341-431.
+ * image[H*W*3] (HWC, background not composited), final_T[H*W], final_idx[H*W]. */
+int dsx_blend_fwd(const dsx_camera* cam, const int32_t* ranges, const int32_t* sorted_ids,
+                  const float* splats, float* image, float* final_T, int32_t* final_idx,
+                  void* stream);
+
+/* Stage 5a — replaces rasterize_backward_tensor + rasterize_backward_kernel,
+ * cpp/gsplat/bindings.cu:140-194, cpp/gsplat/backward.cu:25-202.  grads[n*12] is zeroed by
+ * the call and then accumulated with float atomics.  v_image[H*W*3]. */
+int dsx_blend_bwd(const dsx_camera* cam, int64_t n, const int32_t* ranges,
+                  const int32_t* sorted_ids, const float* splats, const float* final_T,
+                  const int32_t* final_idx, const float* v_image, float* grads, void* stream);
+
+/* Stage 5b+5c — replaces compute_sh_backward_tensor/kernel (cpp/gsplat/bindings.cu:22-51,
+ * cpp/gsplat/sh.cuh:95-203), project_gaussians_backward_tensor/kernel
+ * (cpp/gsplat/bindings.cu:61-131, cpp/gsplat/backward.cu:216-393) and the ATen glue of
+ * rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:291-313.
+ * Outputs: v_mean3d[n*3], v_means2d[n*3] (xy gradient in pixels, z = 0), v_shs[n*num_bases*3]
+ * (may be NULL), v_colors[n*3], v_opacity[n], v_scale[n*3], v_quat[n*4], v_cov3d[n*6].
+ * scales/quats may be NULL when the forward used cov3d_precomp (v_scale, v_quat zeroed). */
+int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+                     const float* scales, const float* quats, const float* splats,
+                     const float* cov3d, const int32_t* radii, const float* grads, float* v_mean3d,
+                     float* v_means2d, float* v_shs, float* v_colors, float* v_opacity,
+                     float* v_scale, float* v_quat, float* v_cov3d, void* stream);
+
+/* ------------------------------------------------------------------------------------ */
+/* Whole forward / backward — what the PyTorch extension calls                           */
+/* ------------------------------------------------------------------------------------ */
+
+/* First half of rasterizer_forward_deepsense (cpp/rasterizer_torch.cu:170-208): projection,
+ * block scan and the read-back of K (the one host synchronisation of the forward, in place of
+ * the reference's two at cpp/rasterizer_torch.cu:103-104).  block_sums is scanned in place.
+ * k_scratch: device uint32[1]; *num_keys (host) receives K. */
+int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
+                        const float* scales, const float* quats, const float* opacities,
+                        const float* shs, const float* cov3d_precomp, const float* colors_precomp,
+                        float* splats, int32_t* radii, float* cov3d, uint32_t* block_sums,
+                        uint32_t* k_scratch, int64_t* num_keys /* host */, void* stream);
+
+/* Second half: key emission, sort, tile ranges, blend.  sorted_ids[k] and ranges[T+1] are
+ * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H). */
+int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
+                       const uint32_t* block_offsets, int32_t* sorted_ids, int32_t* ranges,
+                       float* image, float* final_T, int32_t* final_idx, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316. grads is scratch [n*12]. */
+int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+                 const float* scales, const float* quats, const float* splats, const float* cov3d,
+                 const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
+                 const float* final_T, const int32_t* final_idx, const float* v_image,
+                 float* grads, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
+                 float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, void* stream);
+
+/* Raw-pointer forward-only render, the role of rasterizer_forward_core_deepsense
+ * (cpp/ds_cuda_rasterizer/rasterizer_cuda.hpp:4-9, cpp/rasterizer_cuda.cu:128-158) without
+ * its truncation of the sort to the first n keys.  Unlike every other entry point this one
+ * allocates its temporaries itself (hipMallocAsync on `stream`) as the reference's does with
+ * thrust::device_vector.  All pointers are device pointers. */
+int dsx_forward_core(const float* means3d, const float* shs, const float* opacities,
+                     const float* scales, const float* quats, int64_t n, const float* view,
+                     const float* proj, const float* campos, int32_t image_width,
+                     int32_t image_height, float tanfovx, float tanfovy, float scale_modifier,
+                     int32_t max_sh_degree, int32_t sh_degree, float* image, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

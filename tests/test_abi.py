@@ -1,0 +1,76 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/dsx.h declares;
+the host-side helpers that need no device behave."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "dsx.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dsx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_list_the_same_functions():
+    from ds_splat_amd import _native
+    assert declared_functions() == sorted(_native.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    from ds_splat_amd import _native
+    lib = _native.load()
+    for name in declared_functions():
+        assert getattr(lib, name) is not None
+
+
+def test_host_helpers():
+    from ds_splat_amd import _native
+    lib = _native.load()
+    assert lib.dsx_version() >= 100
+    assert lib.dsx_num_blocks(0) == 0 and lib.dsx_num_blocks(1) == 1 and lib.dsx_num_blocks(257) == 2
+    assert lib.dsx_num_tiles(1920, 1080) == 120 * 68
+    assert lib.dsx_num_tiles(40, 30) == 6
+    # 32 depth bits + bits for tile ids 0..T (slot 0 = negative keys), 8 bits a pass
+    assert lib.dsx_sort_passes(8160) == 6 and lib.dsx_sort_passes(255) == 5 and lib.dsx_sort_passes(32400) == 6
+    assert lib.dsx_workspace_bytes(0, 0, 64, 64) >= 0
+    assert lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080) > (1 << 20) * 24
+    assert b"workspace" in lib.dsx_error_string(-5)
+    assert lib.dsx_error_string(0) == b"ok"
+
+
+def test_bad_arguments_are_rejected_without_touching_the_gpu():
+    from ds_splat_amd import _native
+    lib = _native.load()
+    assert lib.dsx_scan_u32(-1, None, None, None) == -1
+    assert lib.dsx_sort_pairs(-5, 10, None, None, None, 0, None) == -1
+    assert lib.dsx_sort_pairs(1 << 31, 10, 1, 1, 1, 0, None) == -4
+    assert lib.dsx_tile_ranges(10, None, 4, None, None) == -1
+    assert lib.dsx_project_fwd(None, 10, *([None] * 12)) == -1
+
+
+def test_python_api_surface():
+    import dataclasses
+    import ds_splat
+    from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
+    names = [f.name for f in dataclasses.fields(GaussianRasterizationSettings)]
+    assert names == ["image_height", "image_width", "tanfovx", "tanfovy", "bg", "scale_modifier", "viewmatrix",
+                     "projmatrix", "sh_degree", "max_sh_degree", "campos", "prefiltered", "debug"]
+    import inspect
+    sig = list(inspect.signature(GaussianRasterizer.forward).parameters)
+    assert sig == ["self", "means_3d", "means_2d", "shs", "colors_precomp", "opacities", "scales", "rotations",
+                   "cov_3d_precomp"]
+
+
+def test_input_checks_mirror_the_reference_messages():
+    import torch
+    from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
+    from ds_splat_amd.synthetic import make_scene
+    sc = make_scene("cfg0", n=8, width=32, height=32)
+    s = GaussianRasterizationSettings(32, 32, sc["tanfovx"], sc["tanfovy"], sc["bg"], 1.0, sc["viewmatrix"],
+                                      sc["projmatrix"], 0, 3, sc["campos"], False, False)
+    r = GaussianRasterizer(s)
+    with pytest.raises(RuntimeError, match="means_3d must be a CUDA tensor"):
+        r(sc["means_3d"], sc["means_3d"], sc["shs"], None, sc["opacities"], sc["scales"], sc["rotations"], None)

@@ -1,0 +1,292 @@
+"""GPU parity, stage by stage, through the C ABI (ds_splat_amd.stages -> libdsx.so) against
+the CPU oracle on identical seeded inputs.  Integer outputs (radii, tile counts, keys, sorted
+order, ranges) must be bit-exact; floats within rtol 1e-4 / atol 1e-5 (stated per test)."""
+import numpy as np
+import pytest
+import torch
+
+from ds_splat_amd.synthetic import make_scene
+from helpers import arrays, scene_settings
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _stages():
+    from ds_splat_amd import _native, stages
+    _native.load()
+    return stages
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.to(DEV)
+
+
+def pack_splats(S, radii, opac):
+    n = len(radii)
+    sp = np.zeros((n, 12), np.float32)
+    sp[:, 0:3] = S["means2d"]
+    sp[:, 3] = radii.astype(np.int32).view(np.float32)
+    sp[:, 4:7] = S["conic"]
+    sp[:, 7] = opac.reshape(-1)
+    sp[:, 8:11] = S["rgb"]
+    sp[:, 11] = S["tiles_touched"].astype(np.int32).view(np.float32)
+    return sp
+
+
+def oracle_scene(oracle, name="cfg0", n=20000, W=256, H=256, sh_degree=3, seed=None, scale_mul=1.0,
+                 flip_behind=0):
+    sc = make_scene(name, n=n, width=W, height=H, sh_degree=sh_degree, seed=seed)
+    A = arrays(sc)
+    A["scales"] = (A["scales"] * scale_mul).astype(np.float32)
+    if flip_behind:
+        A["means_3d"][:flip_behind, 2] *= -1.0
+    s = scene_settings(sc)
+    img, radii, st = oracle.forward(s, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["shs"],
+                                    keep_emitted=True)
+    S = oracle.state(s, st, n, emitted=True)
+    return sc, A, s, img, radii, st, S
+
+
+# ------------------------------------------------------------------------------- stage 1
+@pytest.mark.parametrize("sh_degree,n,W,H,flip", [(3, 20000, 256, 256, 0), (0, 16384, 256, 256, 0),
+                                                  (1, 5000, 200, 120, 0), (2, 777, 64, 48, 100),
+                                                  (3, 1, 32, 32, 0), (3, 257, 33, 17, 0)])
+def test_project_fwd_bit_exact(oracle, sh_degree, n, W, H, flip):
+    st_ = _stages()
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, sh_degree=sh_degree, seed=100 + n, scale_mul=2.0,
+                                               flip_behind=flip)
+    oracle.free(st)
+    cam = st_.camera_from_scene(sc, DEV)
+    splats, radii_g, cov3d, block_sums = st_.project_fwd(cam, dev(A["means_3d"]), dev(A["scales"]),
+                                                         dev(A["rotations"]), dev(A["opacities"]), dev(A["shs"]))
+    torch.cuda.synchronize()
+    sp = splats.cpu().numpy()
+    # integers: bit exact
+    assert (radii_g.cpu().numpy() == radii).all()
+    assert (sp[:, 3].view(np.int32) == radii).all()
+    assert (sp[:, 11].view(np.int32) == S["tiles_touched"]).all()
+    # the whole integer-determining float chain is IEEE op for op: bit exact too
+    assert (sp[:, 0:3].view(np.int32) == S["means2d"].view(np.int32)).all()
+    vis = radii > 0
+    np.testing.assert_array_equal(sp[vis, 4:7], S["conic"][vis])
+    np.testing.assert_array_equal(sp[:, 8:11], S["rgb"])
+    np.testing.assert_array_equal(cov3d.cpu().numpy(), S["cov3d"])
+    np.testing.assert_array_equal(sp[:, 7], A["opacities"].reshape(-1))
+    # block sums: 256 Gaussians a block, the last Gaussian counts as zero
+    tt = S["tiles_touched"].astype(np.int64).copy()
+    tt[-1] = 0
+    pad = np.zeros((-len(tt)) % 256, np.int64)
+    want = np.concatenate([tt, pad]).reshape(-1, 256).sum(1)
+    assert (block_sums.cpu().numpy().astype(np.int64) == want).all()
+
+
+def test_project_fwd_precomputed_inputs(oracle):
+    st_ = _stages()
+    sc = make_scene("cfg0", n=3000, width=128, height=128, sh_degree=2, seed=5)
+    A = arrays(sc)
+    s = scene_settings(sc)
+    base = oracle.project_fwd(s, A["means_3d"], A["scales"], A["rotations"], A["shs"])
+    cols = np.random.default_rng(0).uniform(0, 1, (3000, 3)).astype(np.float32)
+    want = oracle.project_fwd(s, A["means_3d"], A["scales"], A["rotations"], A["shs"], cov3d_precomp=base["cov3d"],
+                              colors_precomp=cols)
+    cam = st_.camera_from_scene(sc, DEV)
+    splats, radii_g, cov3d, _ = st_.project_fwd(cam, dev(A["means_3d"]), None, None, dev(A["opacities"]), None,
+                                                cov3d_precomp=dev(base["cov3d"]), colors_precomp=dev(cols))
+    sp = splats.cpu().numpy()
+    assert (radii_g.cpu().numpy() == want["radii"]).all()
+    np.testing.assert_array_equal(sp[:, 8:11], cols)
+    np.testing.assert_array_equal(cov3d.cpu().numpy(), base["cov3d"])
+    assert (sp[:, 11].view(np.int32) == want["tiles_touched"]).all()
+
+
+# ------------------------------------------------------------------------------- scan
+@pytest.mark.parametrize("count", [0, 1, 63, 64, 1000, 4096, 4097, 23438, 100001])
+def test_scan_u32(count):
+    st_ = _stages()
+    rng = np.random.default_rng(count)
+    a = rng.integers(0, 5000, count).astype(np.int32)
+    d = dev(a) if count else torch.empty(0, dtype=torch.int32, device=DEV)
+    total = st_.scan_u32(d)
+    torch.cuda.synchronize()
+    want = np.concatenate([[0], np.cumsum(a.astype(np.int64))])
+    assert (d.cpu().numpy().astype(np.int64) == want[:-1]).all()
+    assert int(total.item()) == int(want[-1])
+
+
+# ------------------------------------------------------------------------------- stage 2a
+@pytest.mark.parametrize("n,W,H,scale_mul,flip", [(20000, 256, 256, 2.0, 0), (3000, 200, 120, 12.0, 0),
+                                                  (500, 64, 48, 3.0, 120), (1, 32, 32, 1.0, 0)])
+def test_emit_keys_bit_exact(oracle, n, W, H, scale_mul, flip):
+    st_ = _stages()
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=7 + n, scale_mul=scale_mul,
+                                               flip_behind=flip)
+    oracle.free(st)
+    k = S["num_keys"]
+    cam = st_.camera_from_scene(sc, DEV)
+    splats = dev(pack_splats(S, radii, A["opacities"]))
+    tt = S["tiles_touched"].astype(np.int64).copy()
+    tt[-1] = 0
+    pad = np.zeros((-len(tt)) % 256, np.int64)
+    sums = np.concatenate([tt, pad]).reshape(-1, 256).sum(1)
+    offs = np.concatenate([[0], np.cumsum(sums)[:-1]]).astype(np.int32)
+    keys, vals = st_.emit_keys(cam, n, k, splats, dev(offs))
+    torch.cuda.synchronize()
+    assert (keys.cpu().numpy() == S["emitted_keys"]).all()
+    assert (vals.cpu().numpy() == S["emitted_values"]).all()
+    if flip:
+        assert (S["emitted_keys"] < 0).any()
+
+
+# ------------------------------------------------------------------------------- stage 2b
+def _random_keys(rng, k, num_tiles, neg_frac=0.0, depth_pool=None):
+    tiles = rng.integers(0, num_tiles, k).astype(np.int64)
+    if depth_pool is None:
+        depth = rng.uniform(0.2, 50.0, k).astype(np.float32).view(np.int32).astype(np.int64)
+    else:
+        depth = rng.choice(depth_pool, k).astype(np.float32).view(np.int32).astype(np.int64)
+    keys = (tiles << 32) | depth
+    if neg_frac > 0:
+        neg = rng.random(k) < neg_frac
+        nd = (-rng.uniform(0.2, 50.0, k)).astype(np.float32).view(np.int32).astype(np.int64)   # sign-extended
+        keys = np.where(neg, (tiles << 32) | nd, keys)
+    return keys
+
+
+@pytest.mark.parametrize("k,num_tiles,neg,ties", [(2, 6, 0.0, False), (1000, 6, 0.0, False), (4096, 256, 0.0, True),
+                                                  (4097, 8160, 0.1, False), (50000, 8160, 0.0, True),
+                                                  (1_000_003, 8160, 0.02, True), (300_000, 32400, 0.0, False),
+                                                  (70_000, 1, 0.3, True)])
+def test_sort_pairs_matches_stable_sort(k, num_tiles, neg, ties):
+    st_ = _stages()
+    rng = np.random.default_rng(k)
+    pool = rng.uniform(0.5, 30, 50) if ties else None       # many equal keys: exercises stability
+    keys = _random_keys(rng, k, num_tiles, neg, pool)
+    vals = np.arange(k, dtype=np.int32)
+    rng.shuffle(vals)
+    dk, dv = dev(keys), dev(vals)
+    st_.sort_pairs(dk, dv, num_tiles)
+    torch.cuda.synchronize()
+    order = np.argsort(keys, kind="stable")                  # signed int64 order, like thrust on int64
+    assert (dk.cpu().numpy() == keys[order]).all()
+    assert (dv.cpu().numpy() == vals[order]).all()
+
+
+def test_sort_pairs_vs_oracle_on_emitted_keys(oracle):
+    st_ = _stages()
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=60000, W=512, H=384, seed=77, scale_mul=3.0, flip_behind=500)
+    oracle.free(st)
+    dk, dv = dev(S["emitted_keys"]), dev(S["emitted_values"])
+    st_.sort_pairs(dk, dv, ((512 + 15) // 16) * ((384 + 15) // 16))
+    torch.cuda.synchronize()
+    assert S["num_keys"] > 200000
+    assert (dk.cpu().numpy() == S["sorted_keys"]).all()
+    assert (dv.cpu().numpy() == S["sorted_ids"]).all()
+
+
+# ------------------------------------------------------------------------------- stage 3
+def test_tile_ranges_reference_kats():
+    import json
+    import os
+    st_ = _stages()
+    g = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tile_ranges_kat.json")))
+    for case in g["cases"]:
+        keys = np.array([(t << 32) | d for t, d in case["tile_depth"]], np.int64)
+        got = st_.tile_ranges(dev(keys), 6)
+        assert got.cpu().numpy().tolist() == case["expected"], case["name"]
+
+
+@pytest.mark.parametrize("k,num_tiles,neg", [(0, 12, 0), (1, 12, 0), (300, 12, 0), (5000, 8160, 0),
+                                             (200_000, 8160, 0.05), (100_000, 40000, 0)])
+def test_tile_ranges_vs_oracle(oracle, k, num_tiles, neg):
+    st_ = _stages()
+    rng = np.random.default_rng(k + 1)
+    hi = max(1, num_tiles - 3)                              # leaves the last tiles empty: unclosed last run
+    keys = np.sort(_random_keys(rng, k, hi, neg)) if k else np.zeros(0, np.int64)
+    want = oracle.tile_ranges(keys, num_tiles)
+    d = dev(keys) if k else torch.empty(0, dtype=torch.int64, device=DEV)
+    got = st_.tile_ranges(d, num_tiles)
+    assert (got.cpu().numpy() == want).all()
+
+
+# ------------------------------------------------------------------------------- stage 4
+@pytest.mark.parametrize("n,W,H,scale_mul", [(20000, 256, 256, 2.0), (4000, 200, 120, 6.0), (300, 33, 17, 4.0)])
+def test_blend_fwd_vs_oracle(oracle, n, W, H, scale_mul):
+    st_ = _stages()
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=31 + n, scale_mul=scale_mul)
+    oracle.free(st)
+    cam = st_.camera_from_scene(sc, DEV)
+    splats = dev(pack_splats(S, radii, A["opacities"]))
+    image, final_T, final_idx = st_.blend_fwd(cam, dev(S["ranges"]), dev(S["sorted_ids"]), splats)
+    torch.cuda.synchronize()
+    ok = S["margin"] > 1e-4            # pixels whose threshold decisions are not within exp() noise
+    assert ok.mean() > 0.99
+    np.testing.assert_allclose(image.cpu().numpy()[ok], img[ok], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(final_T.cpu().numpy()[ok], S["final_T"][ok], rtol=1e-4, atol=1e-6)
+    assert (final_idx.cpu().numpy()[ok] == S["final_idx"][ok]).all()
+
+
+# ------------------------------------------------------------------------------- stage 5a
+@pytest.mark.parametrize("n,W,H,scale_mul,bg", [(20000, 256, 256, 2.0, (0, 0, 0)), (4000, 200, 120, 6.0, (0.3, 0.6, 0.1)),
+                                                (300, 33, 17, 4.0, (1, 1, 1))])
+def test_blend_bwd_vs_oracle(oracle, n, W, H, scale_mul, bg):
+    st_ = _stages()
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=41 + n, scale_mul=scale_mul)
+    oracle.free(st)
+    s.bg[:] = list(bg)
+    B = oracle.blend_bwd(s, S["ranges"], S["sorted_ids"], S["means2d"], S["conic"], S["rgb"], A["opacities"],
+                         S["final_T"], S["final_idx"], A["v_image"])
+    cam = st_.camera_from_scene(sc, DEV, bg=torch.tensor(bg, dtype=torch.float32))
+    splats = dev(pack_splats(S, radii, A["opacities"]))
+    grads = st_.blend_bwd(cam, n, dev(S["ranges"]), dev(S["sorted_ids"]), splats, dev(S["final_T"]),
+                          dev(S["final_idx"]), dev(A["v_image"]))
+    torch.cuda.synchronize()
+    g = grads.cpu().numpy()
+    ok = B["g_margin"] > 1e-4
+    assert ok.mean() > 0.99
+    # sums of many float terms of mixed sign in a different order: 1e-3 of the column's scale
+    for got, want, name in ((g[:, 0:2], B["v_xy"], "v_xy"), (g[:, 2:5], B["v_conic"], "v_conic"),
+                            (g[:, 5:6], B["v_opacity"], "v_opacity"), (g[:, 6:9], B["v_rgb"], "v_rgb")):
+        scale = max(1.0, float(np.abs(want[ok]).max()))
+        np.testing.assert_allclose(got[ok], want[ok], rtol=1e-3, atol=1e-4 * scale, err_msg=name)
+    assert (g[:, 9:] == 0).all()
+
+
+# ------------------------------------------------------------------------------- stage 5b+5c
+@pytest.mark.parametrize("sh_degree,num_bases,n", [(3, 16, 20000), (1, 16, 3000), (0, 16, 1000), (1, 4, 999),
+                                                    (2, 9, 300)])
+def test_gaussian_bwd_vs_oracle(oracle, sh_degree, num_bases, n):
+    st_ = _stages()
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=256, H=256, sh_degree=sh_degree, seed=51 + n,
+                                               scale_mul=2.0)
+    oracle.free(st)
+    rng = np.random.default_rng(n)
+    v_xy = rng.normal(size=(n, 2)).astype(np.float32)
+    v_conic = rng.normal(size=(n, 3)).astype(np.float32)
+    v_rgb = rng.normal(size=(n, 3)).astype(np.float32)
+    v_op = rng.normal(size=(n, 1)).astype(np.float32)
+    want = oracle.project_bwd(s, A["means_3d"], A["scales"], A["rotations"], S["conic"], S["cov3d"], radii, v_xy,
+                              v_conic)
+    want_shs = oracle.sh_bwd(s, num_bases, A["means_3d"], v_rgb)
+    grads = np.zeros((n, 12), np.float32)
+    grads[:, 0:2], grads[:, 2:5], grads[:, 5:6], grads[:, 6:9] = v_xy, v_conic, v_op, v_rgb
+    cam = st_.camera_from_scene(sc, DEV)
+    o = st_.gaussian_bwd(cam, num_bases, dev(A["means_3d"]), dev(A["scales"]), dev(A["rotations"]),
+                         dev(pack_splats(S, radii, A["opacities"])), dev(S["cov3d"]), dev(radii), dev(grads))
+    torch.cuda.synchronize()
+    for key, w in (("v_mean3d", want["v_mean3d"]), ("v_scale", want["v_scale"]), ("v_quat", want["v_quat"]),
+                   ("v_cov3d", want["v_cov3d"]), ("v_shs", want_shs)):
+        got = o[key].cpu().numpy()
+        scale = max(1e-6, float(np.abs(w).max()))
+        np.testing.assert_allclose(got, w, rtol=1e-4, atol=2e-6 * scale, err_msg=key)
+    np.testing.assert_array_equal(o["v_colors"].cpu().numpy(), v_rgb)
+    np.testing.assert_array_equal(o["v_opacity"].cpu().numpy(), v_op)
+    m2 = o["v_means2d"].cpu().numpy()
+    np.testing.assert_array_equal(m2[:, :2], v_xy)
+    assert (m2[:, 2] == 0).all()
+    culled = radii <= 0
+    assert culled.any() and (o["v_mean3d"].cpu().numpy()[culled] == 0).all()
