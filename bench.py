@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the rasterizer hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--no-cpu-baseline]
+
+A step is one forward + backward of the public API (GaussianRasterizer(...)(...) followed by
+image.backward(v_image)) on a synthetic scene whose inputs are already resident in HBM.
+Prints ONE JSON line: ms/iter for the workload, the roofline figure of the dominant kernel
+(per-kernel times come from events recorded on the launch stream during the timed steps)
+and the CPU oracle (OpenMP build) timed on the host cores for the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+VALU_PEAK_TFLOPS = 157.3       # MI355X vector FP32 (packed); scalar-FP32 code can reach half
+
+# algorithmic FP32 operations per evaluated (pixel, Gaussian) pair
+FWD_PAIR_FLOPS, FWD_REJECT_FLOPS = 25, 15
+BWD_PAIR_FLOPS, BWD_REJECT_FLOPS = 72, 15
+
+
+def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, passes, counters):
+    """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch."""
+    if kernel == "project_fwd_kernel":
+        return "hbm", n * (44 + 12 * coeffs + 8 + 64), "B"
+    if kernel == "gaussian_bwd_kernel":
+        return "hbm", n * (112 + 76 + 12 * coeffs), "B"
+    if kernel == "emit_keys_kernel":
+        return "hbm", 20 * n + 12 * k, "B"
+    if kernel == "radix_onesweep_kernel":
+        return "hbm", 24 * k, "B"
+    if kernel == "radix_hist_kernel":
+        return "hbm", 8 * k, "B"
+    if kernel == "ranges_boundaries_kernel":
+        return "hbm", 8 * k + 4 * (tiles + 1), "B"
+    if kernel == "blend_fwd_kernel" and counters is not None:
+        rej = counters.pairs_fwd - counters.pairs_fwd_applied
+        return "valu", counters.pairs_fwd_applied * FWD_PAIR_FLOPS + rej * FWD_REJECT_FLOPS, "FLOP"
+    if kernel == "blend_bwd_kernel" and counters is not None:
+        rej = counters.pairs_bwd - counters.pairs_bwd_valid
+        return "valu", counters.pairs_bwd_valid * BWD_PAIR_FLOPS + rej * BWD_REJECT_FLOPS, "FLOP"
+    return None, 0, ""
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg2")
+    ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians (debugging)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--verbose", action="store_true", help="per-kernel table on stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding "
+              "in this build)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
+    from ds_splat_amd import _native
+    from ds_splat_amd.synthetic import WORKLOADS, make_scene
+
+    _native.load()
+    spec = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    sc = make_scene(spec, n=args.n)
+    n, W, H = sc["n"], sc["width"], sc["height"]
+    coeffs = (sc["sh_degree"] + 1) ** 2
+    t = {k: (v.to(dev) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    settings = GaussianRasterizationSettings(
+        image_height=H, image_width=W, tanfovx=sc["tanfovx"], tanfovy=sc["tanfovy"], bg=t["bg"],
+        scale_modifier=1.0, viewmatrix=t["viewmatrix"], projmatrix=t["projmatrix"], sh_degree=sc["sh_degree"],
+        max_sh_degree=3, campos=t["campos"], prefiltered=False, debug=False)
+    rasterizer = GaussianRasterizer(settings)
+    do_backward = spec.backward
+    leaves = [t["means_3d"], torch.zeros_like(t["means_3d"]), t["shs"], t["opacities"], t["scales"], t["rotations"]]
+    if do_backward:
+        leaves = [x.clone().requires_grad_(True) for x in leaves]
+    means, means2d, shs, opac, scales, rots = leaves
+    v_image = t["v_image"]
+
+    def step():
+        image, radii = rasterizer(means, means2d, shs, None, opac, scales, rots, None)
+        if do_backward:
+            for p in leaves:
+                p.grad = None
+            image.backward(v_image)
+        return image
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    _native.trace_enable(True)
+    _native.trace_read()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    trace = _native.trace_read()
+    _native.trace_enable(False)
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    per_kernel = {}
+    for name, ms in trace:
+        tot, cnt = per_kernel.get(name, (0.0, 0))
+        per_kernel[name] = (tot + ms, cnt + 1)
+
+    # key count of this workload
+    from ds_splat_amd import stages
+    cam = stages.camera_from_scene(sc, dev)
+    _, st = stages.forward(cam, t["means_3d"], t["scales"], t["rotations"], t["opacities"], t["shs"])
+    torch.cuda.synchronize()
+    k = st.num_keys
+    tiles = cam.num_tiles
+    passes = int(_native.load().dsx_sort_passes(tiles))
+
+    # ---- CPU baseline: the oracle's OpenMP build on the host cores, same inputs -----------------
+    cpu_baseline = None
+    counters = None
+    if not args.no_cpu_baseline:
+        from oracle.binding import Oracle, make_settings
+        O = Oracle(omp=True)
+        s = make_settings(H, W, sc["tanfovx"], sc["tanfovy"], sc["bg"].numpy(), 1.0,
+                          sc["viewmatrix"].t().contiguous().numpy(), sc["projmatrix"].t().contiguous().numpy(),
+                          sc["sh_degree"], sc["campos"].numpy())
+        A = {kk: v.numpy() for kk, v in sc.items() if isinstance(v, torch.Tensor)}
+        c0 = time.perf_counter()
+        img_o, radii_o, ost = O.forward(s, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["shs"])
+        c1 = time.perf_counter()
+        if do_backward:
+            B = O.backward(s, ost, 16, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["v_image"])
+            counters = B["counters"]
+        else:
+            counters = O.state(s, ost, n)["counters"]
+        c2 = time.perf_counter()
+        k_cpu = int(O.lib.dsxo_state_num_keys(ost))
+        O.free(ost)
+        cpu_ms = (c2 - c0) * 1e3
+        cpu_baseline = {
+            "value": round(cpu_ms, 1), "unit": "ms/iter", "cores": O.num_threads(), "kind": "port",
+            "sample": "1 iteration of the full %s workload (forward %.0f ms%s), C++ oracle built -O3 -fopenmp"
+                      % (spec.name, (c1 - c0) * 1e3, (", backward %.0f ms" % ((c2 - c1) * 1e3)) if do_backward else ""),
+            "keys_match_gpu": bool(k_cpu == k),
+        }
+
+    # ---- roofline of the dominant kernel --------------------------------------------------------
+    table = []
+    for name, (tot, cnt) in per_kernel.items():
+        launches_per_step = cnt / args.steps
+        avg = tot / cnt
+        bound, work, unit = algorithmic_work(name, n, k, W * H, tiles, coeffs, passes, counters)
+        table.append((tot / args.steps, name, avg, launches_per_step, bound, work, unit))
+    table.sort(reverse=True)
+    roofline = None
+    for ms_step, name, avg, lps, bound, work, unit in table:
+        if bound is None:
+            continue
+        if bound == "hbm":
+            achieved = work / (avg * 1e-3) / 1e9
+            roofline = {"kernel": name, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                        "avg_launch_ms": round(avg, 4), "launches_per_step": lps,
+                        "algorithmic_bytes_per_launch": int(work)}
+        else:
+            achieved = work / (avg * 1e-3) / 1e12
+            roofline = {"kernel": name, "bound": "valu", "achieved": round(achieved, 2), "peak": VALU_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(achieved / VALU_PEAK_TFLOPS, 4), "traffic": None,
+                        "avg_launch_ms": round(avg, 4), "launches_per_step": lps,
+                        "algorithmic_flop_per_launch": int(work)}
+        break
+    if args.verbose:
+        for ms_step, name, avg, lps, bound, work, unit in table:
+            extra = ""
+            if bound == "hbm":
+                extra = "%8.1f GB/s (%.1f%% of HBM peak)" % (work / (avg * 1e-3) / 1e9,
+                                                            100 * work / (avg * 1e-3) / 1e9 / HBM_PEAK_GBS)
+            elif bound == "valu":
+                extra = "%8.2f TFLOP/s" % (work / (avg * 1e-3) / 1e12)
+            print("%-28s %8.3f ms/step  %7.4f ms/launch x %4.1f  %s" % (name, ms_step, avg, lps, extra),
+                  file=sys.stderr)
+        print("sum of kernels %.3f ms/step; wall %.3f ms/step; K = %d keys" %
+              (sum(r[0] for r in table), ms_per_step, k), file=sys.stderr)
+
+    out = {
+        "metric": "fwd+bwd ms/iter at 3M Gaussians 1080p SH3" if spec.name == "cfg2" else
+                  ("%s ms/iter (%s)" % ("fwd+bwd" if do_backward else "fwd", spec.name)),
+        "value": round(ms_per_step, 4), "unit": "ms/iter", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: %d Gaussians, %dx%d, SH degree %d, %s" %
+                               (spec.name, n, W, H, sc["sh_degree"], "forward+backward" if do_backward else "forward"),
+                   "num_keys": int(k), "tiles": int(tiles), "radix_passes": passes},
+        "mpix_per_s": round(W * H / (ms_per_step * 1e-3) / 1e6, 1),
+        "kernels_ms_per_step": {name: round(ms_step, 4) for ms_step, name, *_ in table},
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -61,6 +61,16 @@ SIGNATURES = {
                                                                     _I32, _I32, _P, _P]),
 }
 
+
+
+class TraceEntry(C.Structure):
+    """struct dsx_trace_entry"""
+    _fields_ = [("name", C.c_char * 48), ("milliseconds", C.c_float)]
+
+
+SIGNATURES["dsx_trace_enable"] = (C.c_int, [C.c_int])
+SIGNATURES["dsx_trace_read"] = (C.c_int, [C.POINTER(TraceEntry), C.c_int])
+
 _lib = None
 
 
@@ -85,3 +95,14 @@ def load():
 def check(status):
     if status != 0:
         raise RuntimeError(load().dsx_error_string(status).decode())
+
+
+def trace_enable(on):
+    check(load().dsx_trace_enable(1 if on else 0))
+
+
+def trace_read(max_entries=65536):
+    """Returns [(kernel name, milliseconds), ...] in launch order and clears the trace."""
+    buf = (TraceEntry * max_entries)()
+    count = load().dsx_trace_read(buf, max_entries)
+    return [(buf[i].name.decode(), float(buf[i].milliseconds)) for i in range(count)]

@@ -2,7 +2,80 @@
 // synchronisation of the forward (read-back of the key count) and error strings.
 #include "dsx_common.h"
 
+#include <mutex>
+#include <string.h>
+#include <vector>
+
 using namespace dsx;
+
+// ---- optional per-kernel timing -----------------------------------------------------------
+namespace
+{
+struct TraceSlot
+{
+    const char* name;
+    hipEvent_t start, stop;
+};
+bool g_trace_on = false;
+std::mutex g_trace_mutex;
+std::vector<TraceSlot> g_trace;
+} // namespace
+
+dsx::KernelTimer::KernelTimer(const char* name, hipStream_t s) : slot(-1), stream(s)
+{
+    if(!g_trace_on)
+        return;
+    TraceSlot t;
+    t.name = name;
+    if(hipEventCreate(&t.start) != hipSuccess)
+        return;
+    if(hipEventCreate(&t.stop) != hipSuccess)
+    {
+        (void)hipEventDestroy(t.start);
+        return;
+    }
+    (void)hipEventRecord(t.start, s);
+    std::lock_guard<std::mutex> lock(g_trace_mutex);
+    slot = (int)g_trace.size();
+    g_trace.push_back(t);
+}
+
+dsx::KernelTimer::~KernelTimer()
+{
+    if(slot < 0)
+        return;
+    std::lock_guard<std::mutex> lock(g_trace_mutex);
+    (void)hipEventRecord(g_trace[slot].stop, stream);
+}
+
+extern "C" int dsx_trace_enable(int on)
+{
+    std::lock_guard<std::mutex> lock(g_trace_mutex);
+    g_trace_on = on != 0;
+    return DSX_OK;
+}
+
+extern "C" int dsx_trace_read(dsx_trace_entry* out, int max_entries)
+{
+    std::lock_guard<std::mutex> lock(g_trace_mutex);
+    int count = 0;
+    for(const TraceSlot& t : g_trace)
+    {
+        float ms = 0.f;
+        const bool ok = hipEventSynchronize(t.stop) == hipSuccess && hipEventElapsedTime(&ms, t.start, t.stop) == hipSuccess;
+        if(ok && out && count < max_entries)
+        {
+            strncpy(out[count].name, t.name, sizeof(out[count].name) - 1);
+            out[count].name[sizeof(out[count].name) - 1] = 0;
+            out[count].milliseconds = ms;
+            ++count;
+        }
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+    }
+    g_trace.clear();
+    return count;
+}
 
 namespace
 {

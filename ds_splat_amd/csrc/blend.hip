@@ -109,9 +109,12 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
     if(ntx * nty == 0)
         return DSX_OK;
-    hipLaunchKernelGGL(blend_fwd_kernel, dim3(ntx * nty), dim3(kTilePixels), 0, stream, ranges, sorted_ids,
-                       reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                       cam.image_height, ntx);
+    {
+        DSX_TIMED("blend_fwd_kernel", stream);
+        hipLaunchKernelGGL(blend_fwd_kernel, dim3(ntx * nty), dim3(kTilePixels), 0, stream, ranges, sorted_ids,
+                           reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
+                           cam.image_height, ntx);
+    }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
 }
@@ -280,9 +283,12 @@ int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, co
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
     if(ntx * nty == 0 || n == 0)
         return DSX_OK;
-    hipLaunchKernelGGL(blend_bwd_kernel, dim3(ntx * nty), dim3(kTilePixels), 0, stream, ranges, sorted_ids,
-                       reinterpret_cast<const float4*>(splats), final_T, final_idx, v_image, cam.bg, grads,
-                       cam.image_width, cam.image_height, ntx);
+    {
+        DSX_TIMED("blend_bwd_kernel", stream);
+        hipLaunchKernelGGL(blend_bwd_kernel, dim3(ntx * nty), dim3(kTilePixels), 0, stream, ranges, sorted_ids,
+                           reinterpret_cast<const float4*>(splats), final_T, final_idx, v_image, cam.bg, grads,
+                           cam.image_width, cam.image_height, ntx);
+    }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
 }

@@ -105,6 +105,17 @@ int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const f
                         hipStream_t stream);
 int launch_fill_u32(uint32_t* p, int64_t count, uint32_t value, hipStream_t stream);
 
+// Optional per-kernel timing (diagnostics for benchmarks): when switched on through
+// dsx_trace_enable(), every launch is bracketed by two events on the launch stream.
+struct KernelTimer
+{
+    KernelTimer(const char* name, hipStream_t stream);
+    ~KernelTimer();
+    int slot;
+    hipStream_t stream;
+};
+#define DSX_TIMED(name, stream) dsx::KernelTimer dsx_timer_##__LINE__(name, stream)
+
 #ifdef __HIPCC__
 // ---- device helpers -------------------------------------------------------------------
 __device__ __forceinline__ int lane_id()

@@ -355,7 +355,10 @@ int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const f
     p.sh_degree = cam.sh_degree;
     p.num_bases = num_bases;
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
-    hipLaunchKernelGGL(gaussian_bwd_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, p);
+    {
+        DSX_TIMED("gaussian_bwd_kernel", stream);
+        hipLaunchKernelGGL(gaussian_bwd_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, p);
+    }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
 }

@@ -76,7 +76,10 @@ int launch_fill_u32(uint32_t* p, int64_t count, uint32_t value, hipStream_t stre
     if(count <= 0)
         return DSX_OK;
     const int64_t blocks = min((int64_t)4096, (count + 255) / 256);
-    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, count, value);
+    {
+        DSX_TIMED("fill_u32_kernel", stream);
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, count, value);
+    }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
 }
@@ -135,7 +138,10 @@ __global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* data, 
 
 int launch_scan_u32(int64_t count, uint32_t* data, uint32_t* total, hipStream_t stream)
 {
-    hipLaunchKernelGGL(scan_u32_kernel, dim3(1), dim3(kScanThreads), 0, stream, data, count, total);
+    {
+        DSX_TIMED("scan_u32_kernel", stream);
+        hipLaunchKernelGGL(scan_u32_kernel, dim3(1), dim3(kScanThreads), 0, stream, data, count, total);
+    }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
 }
@@ -223,9 +229,12 @@ int launch_emit_keys(const dsx_camera& cam, int64_t n, int64_t k, const float* s
     if(n == 0 || k == 0)
         return DSX_OK;
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
-    hipLaunchKernelGGL(emit_keys_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
-                       reinterpret_cast<const float4*>(splats), block_offsets, n, k, tiles_x(cam.image_width),
-                       tiles_y(cam.image_height), keys, values);
+    {
+        DSX_TIMED("emit_keys_kernel", stream);
+        hipLaunchKernelGGL(emit_keys_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
+                           reinterpret_cast<const float4*>(splats), block_offsets, n, k, tiles_x(cam.image_width),
+                           tiles_y(cam.image_height), keys, values);
+    }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
 }
@@ -509,9 +518,15 @@ int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values
     if(rc)
         return rc;
     const int hist_blocks = (int)min((int64_t)2048, (k + 255) / 256);
-    hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks), dim3(256), 0, stream, keys_a, k, w.passes, global_hist);
+    {
+        DSX_TIMED("radix_hist_kernel", stream);
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks), dim3(256), 0, stream, keys_a, k, w.passes, global_hist);
+    }
     DSX_LAUNCH_CHECK();
-    hipLaunchKernelGGL(radix_hist_scan_kernel, dim3(w.passes), dim3(256), 0, stream, global_hist);
+    {
+        DSX_TIMED("radix_hist_scan_kernel", stream);
+        hipLaunchKernelGGL(radix_hist_scan_kernel, dim3(w.passes), dim3(256), 0, stream, global_hist);
+    }
     DSX_LAUNCH_CHECK();
     int64_t* kin = keys_a;
     int32_t* vin = values_a;
@@ -519,9 +534,12 @@ int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values
     int32_t* vout = values_b;
     for(int p = 0; p < w.passes; ++p)
     {
-        hipLaunchKernelGGL(radix_onesweep_kernel, dim3((unsigned)w.tiles), dim3(kSortThreads), 0, stream, kin, vin,
-                           kout, vout, k, p * kRadixBits, global_hist + p * kRadix,
-                           status + (size_t)p * w.tiles * kRadix, counters + p, counters + w.passes);
+        {
+            DSX_TIMED("radix_onesweep_kernel", stream);
+            hipLaunchKernelGGL(radix_onesweep_kernel, dim3((unsigned)w.tiles), dim3(kSortThreads), 0, stream, kin, vin,
+                               kout, vout, k, p * kRadixBits, global_hist + p * kRadix,
+                               status + (size_t)p * w.tiles * kRadix, counters + p, counters + w.passes);
+        }
         DSX_LAUNCH_CHECK();
         int64_t* tk = kin;
         kin = kout;
@@ -598,16 +616,25 @@ __global__ __launch_bounds__(1024) void ranges_maxscan_kernel(int32_t* ranges, i
 int launch_tile_ranges(int64_t k, const int64_t* sorted_keys, int num_tiles, int32_t* ranges, hipStream_t stream)
 {
     const int count = num_tiles + 1;
-    hipLaunchKernelGGL(ranges_init_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, ranges, num_tiles,
-                       (int32_t)k);
+    {
+        DSX_TIMED("ranges_init_kernel", stream);
+        hipLaunchKernelGGL(ranges_init_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, ranges, num_tiles,
+                           (int32_t)k);
+    }
     DSX_LAUNCH_CHECK();
     if(k > 1)
     {
-        hipLaunchKernelGGL(ranges_boundaries_kernel, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, stream,
-                           sorted_keys, k, ranges);
+        {
+            DSX_TIMED("ranges_boundaries_kernel", stream);
+            hipLaunchKernelGGL(ranges_boundaries_kernel, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, stream,
+                               sorted_keys, k, ranges);
+        }
         DSX_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(ranges_maxscan_kernel, dim3(1), dim3(1024), 0, stream, ranges, count);
+    {
+        DSX_TIMED("ranges_maxscan_kernel", stream);
+        hipLaunchKernelGGL(ranges_maxscan_kernel, dim3(1), dim3(1024), 0, stream, ranges, count);
+    }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
 }

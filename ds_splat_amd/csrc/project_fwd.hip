@@ -362,7 +362,10 @@ int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, c
     p.ntx = tiles_x(cam.image_width);
     p.nty = tiles_y(cam.image_height);
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
-    hipLaunchKernelGGL(project_fwd_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, p);
+    {
+        DSX_TIMED("project_fwd_kernel", stream);
+        hipLaunchKernelGGL(project_fwd_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, p);
+    }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
 }

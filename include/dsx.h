@@ -184,6 +184,22 @@ int dsx_forward_core(const float* means3d, const float* shs, const float* opacit
                      int32_t image_height, float tanfovx, float tanfovy, float scale_modifier,
                      int32_t max_sh_degree, int32_t sh_degree, float* image, void* stream);
 
+/* ------------------------------------------------------------------------------------ */
+/* Diagnostics: per-kernel timing with events on the launch stream.  No counterpart in the  */
+/* reference (its test harness times whole calls on the host, tests/rasterizer_test.cpp:    */
+/* 112-143).  While enabled, every kernel launch of the library records a start/stop event  */
+/* pair; dsx_trace_read waits for them, returns up to max_entries (name, ms) records in     */
+/* launch order and clears the trace.  This is the only process-wide state of the library.  */
+/* ------------------------------------------------------------------------------------ */
+typedef struct dsx_trace_entry
+{
+    char name[48];
+    float milliseconds;
+} dsx_trace_entry;
+
+int dsx_trace_enable(int on);
+int dsx_trace_read(dsx_trace_entry* out /* host */, int max_entries);
+
 #ifdef __cplusplus
 }
 #endif

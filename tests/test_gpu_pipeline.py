@@ -1,0 +1,235 @@
+"""GPU parity of the whole path through the public Python API (GaussianRasterizer + autograd)
+against the CPU oracle, and size-independent properties at the benchmark's full sizes."""
+import numpy as np
+import pytest
+import torch
+
+from ds_splat_amd.synthetic import make_scene
+from helpers import arrays, scene_settings
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def api_run(sc, scale_mul=1.0, backward=True, bg=None, opac_shape=None, colors=None, cov3d=None):
+    from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    settings = GaussianRasterizationSettings(
+        image_height=sc["height"], image_width=sc["width"], tanfovx=sc["tanfovx"], tanfovy=sc["tanfovy"],
+        bg=t["bg"] if bg is None else torch.tensor(bg, dtype=torch.float32, device=DEV), scale_modifier=1.0,
+        viewmatrix=t["viewmatrix"], projmatrix=t["projmatrix"], sh_degree=sc["sh_degree"], max_sh_degree=3,
+        campos=t["campos"], prefiltered=False, debug=False)
+    opac = t["opacities"] if opac_shape is None else t["opacities"].reshape(opac_shape)
+    leaves = dict(means=t["means_3d"].clone(), means2d=torch.zeros_like(t["means_3d"]), shs=t["shs"].clone(),
+                  opac=opac.clone(), scales=(t["scales"] * scale_mul).clone(), rots=t["rotations"].clone())
+    if backward:
+        for v in leaves.values():
+            v.requires_grad_(True)
+    r = GaussianRasterizer(settings)
+    if colors is not None:
+        image, radii = r(leaves["means"], leaves["means2d"], None, colors, leaves["opac"], leaves["scales"],
+                         leaves["rots"], None)
+    elif cov3d is not None:
+        image, radii = r(leaves["means"], leaves["means2d"], leaves["shs"], None, leaves["opac"], None, None, cov3d)
+    else:
+        image, radii = r(leaves["means"], leaves["means2d"], leaves["shs"], None, leaves["opac"], leaves["scales"],
+                         leaves["rots"], None)
+    if backward:
+        image.backward(t["v_image"])
+    torch.cuda.synchronize()
+    return image, radii, leaves
+
+
+def oracle_run(oracle, sc, scale_mul=1.0, bg=None, backward=True):
+    A = arrays(sc)
+    A["scales"] = (A["scales"] * scale_mul).astype(np.float32)
+    s = scene_settings(sc, bg=bg)
+    img, radii, st = oracle.forward(s, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["shs"])
+    S = oracle.state(s, st, sc["n"])
+    B = oracle.backward(s, st, 16, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["v_image"]) \
+        if backward else None
+    oracle.free(st)
+    return img, radii, S, B
+
+
+def check_grads(leaves, B, ok):
+    pairs = (("means", "v_mean3d"), ("means2d", "v_means2d"), ("shs", "v_shs"), ("opac", "v_opacity"),
+             ("scales", "v_scale"), ("rots", "v_quat"))
+    for leaf, key in pairs:
+        got = leaves[leaf].grad.cpu().numpy().reshape(B[key].shape)[ok]
+        want = B[key][ok]
+        # atomics reorder the per-Gaussian sums: 1e-3 relative, floor at 1e-4 of the tensor's scale
+        scale = max(1.0, float(np.abs(want).max()))
+        np.testing.assert_allclose(got, want, rtol=1e-3, atol=1e-4 * scale, err_msg=key)
+
+
+@pytest.mark.parametrize("name,n,W,H,deg,scale_mul,bg", [
+    ("cfg0", 16384, 256, 256, 0, 1.0, None),            # BASELINE config 0 at full size
+    ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9)),
+    ("cfg1", 40000, 480, 270, 3, 1.0, None),            # config 1 distributions, reduced size
+    ("cfg4", 3000, 320, 180, 3, 0.5, None),             # heavy-overlap distributions, reduced size
+    ("cfg2", 30000, 333, 177, 2, 1.5, None),            # ragged image (not a multiple of 16)
+])
+def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, bg):
+    sc = make_scene(name, n=n, width=W, height=H, sh_degree=deg)
+    image, radii, leaves = api_run(sc, scale_mul, bg=bg)
+    img_o, radii_o, S, B = oracle_run(oracle, sc, scale_mul, bg=bg)
+    assert image.shape == (H, W, 3) and radii.dtype == torch.int32 and radii.shape == (n,)
+    assert (radii.cpu().numpy() == radii_o).all()
+    ok = S["margin"] > 1e-4
+    assert ok.mean() > 0.98
+    np.testing.assert_allclose(image.detach().cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
+    gok = B["g_margin"] > 1e-5
+    assert gok.mean() > 0.97
+    check_grads(leaves, B, gok)
+    assert leaves["opac"].grad.shape == leaves["opac"].shape
+    assert (leaves["means2d"].grad[:, 2] == 0).all()
+
+
+def test_api_internal_integers_bit_exact(oracle):
+    """sorted order (stable tie-break) and tile ranges of the whole forward, bit for bit."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg1", n=50000, width=640, height=360, sh_degree=1)
+    cam = stages.camera_from_scene(sc, DEV)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    image, st = stages.forward(cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
+    torch.cuda.synchronize()
+    img_o, radii_o, S, _ = oracle_run(oracle, sc, 2.0, backward=False)
+    assert st.num_keys == S["num_keys"] > 100000
+    assert (st.sorted_ids.cpu().numpy() == S["sorted_ids"]).all()
+    assert (st.ranges.cpu().numpy() == S["ranges"]).all()
+    assert (st.radii.cpu().numpy() == radii_o).all()
+    sp = st.splats.cpu().numpy()
+    assert (sp[:, 11].view(np.int32) == S["tiles_touched"]).all()
+    ok = S["margin"] > 1e-4
+    assert (st.final_idx.cpu().numpy()[ok] == S["final_idx"][ok]).all()
+
+
+def test_api_opacity_as_vector_and_empty_scene(oracle):
+    sc = make_scene("cfg0", n=2000, width=64, height=64, sh_degree=1)
+    image, radii, leaves = api_run(sc, 3.0, opac_shape=(2000,))
+    assert leaves["opac"].grad.shape == (2000,)
+    # everything behind / outside: K = 0, image must be all zeros and backward all zeros
+    sc2 = make_scene("cfg0", n=500, width=64, height=64, sh_degree=0)
+    sc2["means_3d"][:, 0] += 1000.0
+    image, radii, leaves = api_run(sc2)
+    assert (image == 0).all() and (radii == 0).all()
+    for v in leaves.values():
+        assert (v.grad == 0).all()
+
+
+def test_api_precomputed_colors_and_cov3d(oracle):
+    sc = make_scene("cfg0", n=5000, width=128, height=96, sh_degree=2)
+    A = arrays(sc)
+    s = scene_settings(sc)
+    base = oracle.project_fwd(s, A["means_3d"], A["scales"] * 2, A["rotations"], A["shs"])
+    cols = torch.rand(5000, 3, generator=torch.Generator().manual_seed(1))
+    img_o, radii_o, st = oracle.forward(s, A["means_3d"], A["scales"] * 2, A["rotations"], A["opacities"], A["shs"],
+                                        colors_precomp=cols.numpy())
+    S = oracle.state(s, st, 5000)
+    oracle.free(st)
+    image, radii, _ = api_run(sc, 2.0, backward=False, colors=cols.to(DEV))
+    ok = S["margin"] > 1e-4
+    np.testing.assert_allclose(image.cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
+    # cov3D_precomp path renders the same image as scales+rotations
+    img_a, radii_a, _ = api_run(sc, 2.0, backward=False)
+    img_b, radii_b, _ = api_run(sc, 2.0, backward=False, cov3d=torch.from_numpy(base["cov3d"]).to(DEV))
+    assert (radii_a == radii_b).all() and torch.equal(img_a, img_b)
+
+
+def test_forward_core_raw_pointer_entry(oracle):
+    """dsx_forward_core: device pointers in, image out (the reference's torch-free entry)."""
+    import ctypes as C
+    from ds_splat_amd import _native
+    lib = _native.load()
+    sc = make_scene("cfg0", n=8000, width=160, height=128, sh_degree=3)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    view = t["viewmatrix"].t().contiguous()
+    proj = t["projmatrix"].t().contiguous()
+    image = torch.empty(128, 160, 3, device=DEV)
+    p = lambda x: C.c_void_p(x.data_ptr())
+    rc = lib.dsx_forward_core(p(t["means_3d"]), p(t["shs"]), p(t["opacities"]), p(t["scales"]), p(t["rotations"]),
+                              8000, p(view), p(proj), p(t["campos"]), 160, 128, sc["tanfovx"], sc["tanfovy"], 1.0, 3,
+                              3, p(image), C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    img_o, _, S, _ = oracle_run(oracle, sc, backward=False)
+    ok = S["margin"] > 1e-4
+    np.testing.assert_allclose(image.cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
+
+
+# ------------------------------------------------------------------------- properties at full size
+def test_full_size_properties_cfg2():
+    """3M Gaussians, 1920x1080, SH3 (the headline shape): properties that need no oracle."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg2")
+    n = sc["n"]
+    cam = stages.camera_from_scene(sc, DEV)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    splats, radii, cov3d, block_sums = stages.project_fwd(cam, t["means_3d"], t["scales"], t["rotations"],
+                                                          t["opacities"], t["shs"])
+    tiles = splats[:, 11].view(torch.int32).to(torch.int64)
+    tiles_eff = tiles.clone()
+    tiles_eff[-1] = 0
+    total = stages.scan_u32(block_sums)
+    k = int(total.item())
+    assert k == int(tiles_eff.sum().item()) and k > 10_000_000
+    assert ((radii > 0) == (tiles > 0)).all() or ((radii > 0) | (tiles == 0)).all()
+    keys, vals = stages.emit_keys(cam, n, k, splats, block_sums)
+    # every Gaussian appears exactly tiles_touched times, keys carry its depth bits
+    counts = torch.bincount(vals.to(torch.int64), minlength=n)
+    assert torch.equal(counts, tiles_eff)
+    depth_bits = splats[:, 2].view(torch.int32).to(torch.int64)
+    assert torch.equal(keys & 0xFFFFFFFF, depth_bits[vals.to(torch.int64)])
+    checksum = int(keys.sum().item()) ^ int(vals.to(torch.int64).sum().item())
+    stages.sort_pairs(keys, vals, cam.num_tiles)
+    assert int(keys.sum().item()) ^ int(vals.to(torch.int64).sum().item()) == checksum   # a permutation
+    assert (keys[1:] >= keys[:-1]).all()                                                   # sorted
+    same = keys[1:] == keys[:-1]
+    assert (vals[1:][same] > vals[:-1][same]).all()                                        # stable tie-break
+    assert torch.equal(keys & 0xFFFFFFFF, depth_bits[vals.to(torch.int64)])                # pairs stay together
+    ranges = stages.tile_ranges(keys, cam.num_tiles)
+    assert (ranges[1:] >= ranges[:-1]).all() and int(ranges[-1]) == k and int(ranges[0]) == 0
+    tile_of = (keys >> 32).to(torch.int64)
+    r = ranges.to(torch.int64)
+    t_last = int(tile_of[-1])
+    probe = torch.randint(0, t_last, (2000,), device=DEV)
+    for tt in probe.tolist()[:200]:
+        seg = tile_of[int(r[tt]):int(r[tt + 1])]
+        assert (seg == tt).all()
+    image, final_T, final_idx = stages.blend_fwd(cam, ranges, vals, splats)
+    assert torch.isfinite(image).all() and (image >= 0).all()
+    assert (final_T <= 1).all() and (final_T >= 9.9e-5).all()
+    # all-white scene: image telescopes to 1 - final_T in every channel
+    white = splats.clone()
+    white[:, 8:11] = 1.0
+    img_w, T_w, _ = stages.blend_fwd(cam, ranges, vals, white)
+    assert torch.allclose(img_w, (1 - T_w).unsqueeze(-1).expand(-1, -1, 3), rtol=0, atol=2e-5)
+    assert torch.equal(T_w, final_T)
+    # determinism of the forward, linearity of the backward in the upstream gradient
+    image2, _, _ = stages.blend_fwd(cam, ranges, vals, splats)
+    assert torch.equal(image, image2)
+    g1 = stages.blend_bwd(cam, n, ranges, vals, splats, final_T, final_idx, t["v_image"])
+    g2 = stages.blend_bwd(cam, n, ranges, vals, splats, final_T, final_idx, 2.0 * t["v_image"])
+    assert torch.allclose(g2, 2.0 * g1, rtol=2e-3, atol=2e-3 * float(g1.abs().max()))
+    # v_rgb of a Gaussian nobody blended is zero; gradient of culled Gaussians is zero
+    assert (g1[radii <= 0] == 0).all()
+    o = stages.gaussian_bwd(cam, 16, t["means_3d"], t["scales"], t["rotations"], splats, cov3d, radii, g1)
+    for key in ("v_mean3d", "v_scale", "v_quat", "v_cov3d", "v_shs"):
+        assert torch.isfinite(o[key]).all()
+        assert (o[key][radii <= 0] == 0).all()
+
+
+def test_full_size_forward_cfg3_4k():
+    """6M Gaussians at 3840x2160 (forward only): runs, sorted, deterministic."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg3")
+    cam = stages.camera_from_scene(sc, DEV)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    image, st = stages.forward(cam, t["means_3d"], t["scales"], t["rotations"], t["opacities"], t["shs"])
+    image2, st2 = stages.forward(cam, t["means_3d"], t["scales"], t["rotations"], t["opacities"], t["shs"])
+    torch.cuda.synchronize()
+    assert st.num_keys == st2.num_keys > 1_000_000
+    assert torch.equal(st.sorted_ids, st2.sorted_ids) and torch.equal(image, image2)
+    assert (st.ranges[1:] >= st.ranges[:-1]).all() and int(st.ranges[-1]) == st.num_keys
+    assert torch.isfinite(image).all()

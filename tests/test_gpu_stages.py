@@ -246,7 +246,7 @@ def test_blend_bwd_vs_oracle(oracle, n, W, H, scale_mul, bg):
                           dev(S["final_idx"]), dev(A["v_image"]))
     torch.cuda.synchronize()
     g = grads.cpu().numpy()
-    ok = B["g_margin"] > 1e-4
+    ok = B["g_margin"] > 1e-5
     assert ok.mean() > 0.99
     # sums of many float terms of mixed sign in a different order: 1e-3 of the column's scale
     for got, want, name in ((g[:, 0:2], B["v_xy"], "v_xy"), (g[:, 2:5], B["v_conic"], "v_conic"),
