@@ -123,13 +123,28 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
 // backward: cpp/gsplat/backward.cu:25-202
 // -----------------------------------------------------------------------------------------
 
-__device__ __forceinline__ float wave_sum_f32(float v)
+// Sum over the 64 lanes of a wavefront with data-parallel-primitive adds only (no LDS
+// traffic): two quad permutes, two row mirrors, then the row broadcasts.  The total is valid
+// in lane 63.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_add(float v)
 {
-#pragma unroll
-    for(int o = 32; o > 0; o >>= 1)
-        v += __shfl_xor(v, o, DSX_WAVE);
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xf, false);
+    return v + __int_as_float(moved);
+}
+
+__device__ __forceinline__ float wave_sum_to_lane63(float v)
+{
+    v = dpp_add<0xB1, 0xf>(v);  // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xf>(v);  // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xf>(v); // row_half_mirror
+    v = dpp_add<0x140, 0xf>(v); // row_mirror: every lane of a row holds the row sum
+    v = dpp_add<0x142, 0xa>(v); // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xc>(v); // row_bcast:31 into rows 2 and 3
     return v;
 }
+
+constexpr int kGradVals = 9;
 
 __global__ __launch_bounds__(kTilePixels) void blend_bwd_kernel(
     const int32_t* __restrict__ ranges, const int32_t* __restrict__ ids, const float4* __restrict__ splats,
@@ -140,6 +155,7 @@ __global__ __launch_bounds__(kTilePixels) void blend_bwd_kernel(
     __shared__ float4 s_b[kTilePixels]; // conic c, opacity, red, green
     __shared__ float s_c[kTilePixels];  // blue
     __shared__ int s_id[kTilePixels];
+    __shared__ float s_acc[kTilePixels * kGradVals]; // per-entry sums over the four wavefronts
     __shared__ int s_wave_max[4];
 
     const int tid = threadIdx.x;
@@ -170,7 +186,7 @@ __global__ __launch_bounds__(kTilePixels) void blend_bwd_kernel(
     const int start = ranges[tile];
     const int end = ranges[tile + 1];
 
-    // last entry any pixel of this tile blended
+    // last entry any pixel of this wavefront / of this tile blended
     int m = bin_final;
 #pragma unroll
     for(int o = 32; o > 0; o >>= 1)
@@ -187,7 +203,7 @@ __global__ __launch_bounds__(kTilePixels) void blend_bwd_kernel(
 
     for(int top = hi; top >= start; top -= kTilePixels)
     {
-        __syncthreads();
+        __syncthreads(); // previous batch fully consumed (staging and accumulators)
         const int e = top - tid;
         if(e >= start)
         {
@@ -199,6 +215,9 @@ __global__ __launch_bounds__(kTilePixels) void blend_bwd_kernel(
             s_c[tid] = q2.z;
             s_id[tid] = g;
         }
+#pragma unroll
+        for(int j = 0; j < kGradVals; ++j)
+            s_acc[j * kTilePixels + tid] = 0.f;
         __syncthreads();
         const int cnt = min(kTilePixels, top - start + 1);
         // entries beyond what any lane of this wavefront blended are skipped outright
@@ -221,16 +240,15 @@ __global__ __launch_bounds__(kTilePixels) void blend_bwd_kernel(
             }
             if(__ballot(valid) == 0)
                 continue;
-            float g_r = 0.f, g_g = 0.f, g_b = 0.f, g_ca = 0.f, g_cb = 0.f, g_cc = 0.f, g_x = 0.f, g_y = 0.f,
-                  g_o = 0.f;
+            float g[kGradVals] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             if(valid)
             {
                 const float ra = __builtin_amdgcn_rcpf(1.0f - alpha);
                 T *= ra;
                 const float fac = alpha * T;
-                g_r = fac * vo0;
-                g_g = fac * vo1;
-                g_b = fac * vo2;
+                g[6] = fac * vo0;
+                g[7] = fac * vo1;
+                g[8] = fac * vo2;
                 const float blue = s_c[t];
                 float v_alpha = (B.z * T - buf0 * ra) * vo0;
                 v_alpha += (B.w * T - buf1 * ra) * vo1;
@@ -240,34 +258,41 @@ __global__ __launch_bounds__(kTilePixels) void blend_bwd_kernel(
                 buf1 += B.w * fac;
                 buf2 += blue * fac;
                 const float v_sigma = -B.y * vis * v_alpha;
-                g_ca = 0.5f * v_sigma * dx * dx;
-                g_cb = v_sigma * dx * dy;
-                g_cc = 0.5f * v_sigma * dy * dy;
-                g_x = v_sigma * (A.z * dx + A.w * dy);
-                g_y = v_sigma * (A.w * dx + B.x * dy);
-                g_o = vis * v_alpha;
+                g[0] = v_sigma * (A.z * dx + A.w * dy);
+                g[1] = v_sigma * (A.w * dx + B.x * dy);
+                g[2] = 0.5f * v_sigma * dx * dx;
+                g[3] = v_sigma * dx * dy;
+                g[4] = 0.5f * v_sigma * dy * dy;
+                g[5] = vis * v_alpha;
             }
-            g_x = wave_sum_f32(g_x);
-            g_y = wave_sum_f32(g_y);
-            g_ca = wave_sum_f32(g_ca);
-            g_cb = wave_sum_f32(g_cb);
-            g_cc = wave_sum_f32(g_cc);
-            g_o = wave_sum_f32(g_o);
-            g_r = wave_sum_f32(g_r);
-            g_g = wave_sum_f32(g_g);
-            g_b = wave_sum_f32(g_b);
-            if(lane == 0)
+#pragma unroll
+            for(int j = 0; j < kGradVals; ++j)
+                g[j] = wave_sum_to_lane63(g[j]);
+            if(lane == 63)
             {
-                float* dst = grads + (int64_t)s_id[t] * DSX_GRAD_FLOATS;
-                unsafeAtomicAdd(dst + 0, g_x);
-                unsafeAtomicAdd(dst + 1, g_y);
-                unsafeAtomicAdd(dst + 2, g_ca);
-                unsafeAtomicAdd(dst + 3, g_cb);
-                unsafeAtomicAdd(dst + 4, g_cc);
-                unsafeAtomicAdd(dst + 5, g_o);
-                unsafeAtomicAdd(dst + 6, g_r);
-                unsafeAtomicAdd(dst + 7, g_g);
-                unsafeAtomicAdd(dst + 8, g_b);
+#pragma unroll
+                for(int j = 0; j < kGradVals; ++j)
+                    atomicAdd(&s_acc[j * kTilePixels + t], g[j]);
+            }
+        }
+        __syncthreads();
+        // one set of global atomics per (tile, entry): thread t flushes entry t
+        if(tid < cnt)
+        {
+            float v[kGradVals];
+            bool any = false;
+#pragma unroll
+            for(int j = 0; j < kGradVals; ++j)
+            {
+                v[j] = s_acc[j * kTilePixels + tid];
+                any = any || v[j] != 0.f;
+            }
+            if(any)
+            {
+                float* dst = grads + (int64_t)s_id[tid] * DSX_GRAD_FLOATS;
+#pragma unroll
+                for(int j = 0; j < kGradVals; ++j)
+                    unsafeAtomicAdd(dst + j, v[j]);
             }
         }
     }
