@@ -21,12 +21,19 @@ constexpr int kTile = DSX_TILE;
 constexpr int kTilePixels = DSX_TILE * DSX_TILE;
 constexpr int kProjBlock = DSX_PROJ_BLOCK;
 
-// Radix sort geometry: 8-bit digits, 256 threads, kSortItems keys per thread per tile.
-constexpr int kRadixBits = 8;
-constexpr int kRadix = 1 << kRadixBits;
-constexpr int kSortThreads = 256;
-constexpr int kSortItems = 16;
+// Radix sort geometry: digits of up to 9 bits (512 bins), kSortThreads x kSortItems keys per tile.
+constexpr int kRadixBitsMax = 9;
+constexpr int kRadix = 1 << kRadixBitsMax;
+#ifndef DSX_SORT_THREADS
+#define DSX_SORT_THREADS 768
+#endif
+#ifndef DSX_SORT_ITEMS
+#define DSX_SORT_ITEMS 8
+#endif
+constexpr int kSortThreads = DSX_SORT_THREADS;
+constexpr int kSortItems = DSX_SORT_ITEMS;
 constexpr int kSortTile = kSortThreads * kSortItems;
+constexpr int kMaxPasses = 8;
 
 inline int tiles_x(int w)
 {
@@ -46,9 +53,32 @@ inline int sort_key_bits(int num_tiles)
         ++b;
     return 32 + b;
 }
+
+// Digit plan: the fewest passes with digits of at most 9 bits, bits spread evenly.
+struct SortPlan
+{
+    int passes;
+    int shift[kMaxPasses];
+    int bits[kMaxPasses];
+};
+inline SortPlan sort_plan(int num_tiles)
+{
+    SortPlan pl;
+    const int total = sort_key_bits(num_tiles);
+    pl.passes = (total + kRadixBitsMax - 1) / kRadixBitsMax;
+    const int base = total / pl.passes, rem = total % pl.passes;
+    int shift = 0;
+    for(int p = 0; p < kMaxPasses; ++p)
+    {
+        pl.shift[p] = shift;
+        pl.bits[p] = p < pl.passes ? base + (p < rem ? 1 : 0) : 0;
+        shift += pl.bits[p];
+    }
+    return pl;
+}
 inline int sort_passes(int num_tiles)
 {
-    return (sort_key_bits(num_tiles) + kRadixBits - 1) / kRadixBits;
+    return sort_plan(num_tiles).passes;
 }
 
 // Workspace layout of the sort for k keys (all offsets 256-byte aligned).

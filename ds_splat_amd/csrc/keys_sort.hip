@@ -3,6 +3,8 @@
 // tile-range identification.  Integer work only; everything is HBM-bandwidth bound.
 #include "dsx_common.h"
 
+#include <mutex>
+
 namespace dsx
 {
 
@@ -34,12 +36,12 @@ __device__ __forceinline__ int wave_incl_max_i32(int v, int lane)
     return v;
 }
 
-// lanes of the wavefront that hold the same 8-bit digit (and are valid); call in uniform flow
+// lanes of the wavefront that hold the same (up to 9-bit) digit and are valid; call in uniform flow
 __device__ __forceinline__ uint64_t match_digit(uint32_t d, bool valid)
 {
     uint64_t mask = __ballot(valid);
 #pragma unroll
-    for(int b = 0; b < kRadixBits; ++b)
+    for(int b = 0; b < kRadixBitsMax; ++b)
     {
         const bool bit = (d >> b) & 1u;
         const uint64_t m = __ballot(bit);
@@ -279,43 +281,92 @@ ForwardWorkspace forward_workspace(int64_t k, int num_tiles)
     return w;
 }
 
-// Histogram of every digit of every key in one read of the keys.  Lanes that hold the same
-// digit are merged with ballots first, so the LDS atomics never collide inside a wavefront
-// (emission order puts long runs of equal depth bits next to each other).
-__global__ __launch_bounds__(256) void radix_hist_kernel(const int64_t* __restrict__ keys, int64_t k, int passes,
-                                                         uint32_t* __restrict__ global_hist)
+struct DigitPlan
 {
-    __shared__ uint32_t hist[8 * kRadix];
+    int passes;
+    int shift[kMaxPasses];
+    uint32_t mask[kMaxPasses];
+};
+
+static DigitPlan digit_plan(int num_tiles)
+{
+    const SortPlan sp = sort_plan(num_tiles);
+    DigitPlan d;
+    d.passes = sp.passes;
+    for(int p = 0; p < kMaxPasses; ++p)
+    {
+        d.shift[p] = sp.shift[p];
+        d.mask[p] = (1u << sp.bits[p]) - 1u;
+    }
+    return d;
+}
+
+// value of the lane below (lane 0 receives `first`): one DPP move, no LDS traffic
+__device__ __forceinline__ uint32_t lane_below(uint32_t v, uint32_t first)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)first, (int)v, 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+}
+
+// Histogram of every digit of every key in one read of the keys.  Emission order puts long
+// runs of equal digits next to each other (all keys of one Gaussian share their depth bits),
+// so each run of equal digits inside a wavefront is collapsed to one LDS atomic by its first
+// lane: heads are found with one lane shift and one ballot per digit.
+constexpr int kHistThreads = 256;
+constexpr int kHistItems = 8;
+
+__global__ __launch_bounds__(kHistThreads) void radix_hist_kernel(const int64_t* __restrict__ keys, int64_t k,
+                                                                  const DigitPlan plan,
+                                                                  uint32_t* __restrict__ global_hist)
+{
+    __shared__ uint32_t hist[kMaxPasses * kRadix];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    for(int j = tid; j < passes * kRadix; j += 256)
+    for(int j = tid; j < plan.passes * kRadix; j += kHistThreads)
         hist[j] = 0;
     __syncthreads();
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    const int64_t rounds = (k + stride - 1) / stride;
-    for(int64_t r = 0; r < rounds; ++r)
+    const int64_t chunk = (int64_t)kHistThreads * kHistItems;
+    const int64_t chunks = (k + chunk - 1) / chunk;
+    for(int64_t c = blockIdx.x; c < chunks; c += gridDim.x)
     {
-        const int64_t i = r * stride + (int64_t)blockIdx.x * 256 + tid;
-        const bool valid = i < k;
-        const uint64_t s = valid ? sortable(keys[i]) : 0ull;
-        for(int p = 0; p < passes; ++p)
+        uint64_t s[kHistItems];
+        bool valid[kHistItems];
+#pragma unroll
+        for(int it = 0; it < kHistItems; ++it)
         {
-            const uint32_t d = (uint32_t)(s >> (p * kRadixBits)) & (kRadix - 1);
-            const uint64_t m = match_digit(d, valid);
-            if(valid && (m & lanemask_lt(lane)) == 0)
-                atomicAdd(&hist[p * kRadix + d], (uint32_t)__popcll(m));
+            const int64_t i = c * chunk + it * kHistThreads + tid;
+            valid[it] = i < k;
+            s[it] = valid[it] ? sortable(__builtin_nontemporal_load(keys + i)) : 0ull;
+        }
+#pragma unroll
+        for(int it = 0; it < kHistItems; ++it)
+        {
+            const uint64_t vmask = __ballot(valid[it]); // valid lanes are a prefix of the wavefront
+            const int nvalid = __popcll(vmask);
+            for(int p = 0; p < plan.passes; ++p)
+            {
+                const uint32_t d = (uint32_t)(s[it] >> plan.shift[p]) & plan.mask[p];
+                const uint32_t below = lane_below(d, ~d);
+                const bool head = valid[it] && (lane == 0 || below != d);
+                const uint64_t heads = __ballot(head);
+                if(head)
+                {
+                    const uint64_t above = lane == 63 ? 0ull : (heads >> (lane + 1));
+                    const int run = above ? __ffsll((unsigned long long)above) : nvalid - lane;
+                    atomicAdd(&hist[p * kRadix + d], (uint32_t)run);
+                }
+            }
         }
     }
     __syncthreads();
-    for(int j = tid; j < passes * kRadix; j += 256)
+    for(int j = tid; j < plan.passes * kRadix; j += kHistThreads)
         if(hist[j])
             atomicAdd(&global_hist[j], hist[j]);
 }
 
-// exclusive scan of each pass's 256 bins (one wave-sized job per pass)
-__global__ __launch_bounds__(256) void radix_hist_scan_kernel(uint32_t* global_hist)
+// exclusive scan of each pass's 512 bins (one workgroup per pass)
+__global__ __launch_bounds__(kRadix) void radix_hist_scan_kernel(uint32_t* global_hist)
 {
-    __shared__ uint32_t wave_tot[4];
+    __shared__ uint32_t wave_tot[kRadix / DSX_WAVE];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -336,24 +387,31 @@ constexpr uint32_t kFlagInclusive = 2u << 30;
 constexpr uint32_t kFlagMask = 3u << 30;
 constexpr uint32_t kValueMask = ~kFlagMask;
 constexpr int kSpinLimit = 1 << 18; // bounded wait: a stuck predecessor ends in an error flag, not a hang
+constexpr int kLookBatch = 4;       // predecessor statuses fetched per round trip
+constexpr int kSortWaves = kSortThreads / DSX_WAVE;
 
-// One digit pass.  Tile = 4096 consecutive keys, taken in arrival order through a dynamic
+// One digit pass.  Tile = kSortTile consecutive keys, taken in arrival order through a dynamic
 // counter so that every tile a workgroup waits for has already started.  Stable ranking:
-// wave-local rank by ballot matching (item by item, lane by lane), waves in tile order,
-// tiles in chained-scan order.  Keys are reordered through LDS so that global stores of one
-// digit are contiguous.
+// wave-local rank by ballot matching (item by item, lane by lane), waves in tile order, tiles
+// in chained-scan order (decoupled look-back; thread d owns digit d and fetches several
+// predecessors per round trip).  Keys, then values, are reordered through the same LDS buffer
+// so that global stores of one digit are contiguous.  Large tiles matter twice: the status
+// traffic of the look-back falls with the number of tiles AND with the depth of the walk,
+// which itself shrinks when tiles start less often.
+constexpr size_t kSortLdsBytes = (size_t)kSortTile * 8 + (size_t)kSortWaves * kRadix * 2 + 2 * kRadix * 4 + 64 + 16;
+
 __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
     const int64_t* __restrict__ keys_in, const int32_t* __restrict__ vals_in, int64_t* __restrict__ keys_out,
-    int32_t* __restrict__ vals_out, int64_t k, int shift, const uint32_t* __restrict__ hist_excl,
+    int32_t* __restrict__ vals_out, int64_t k, int shift, uint32_t mask, const uint32_t* __restrict__ hist_excl,
     uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag)
 {
-    __shared__ int64_t s_keys[kSortTile];
-    __shared__ int32_t s_vals[kSortTile];
-    __shared__ uint32_t s_whist[4][kRadix];
-    __shared__ uint32_t s_digit_start[kRadix];
-    __shared__ uint32_t s_gbase[kRadix];
-    __shared__ uint32_t s_wave_tot[4];
-    __shared__ uint32_t s_tile;
+    extern __shared__ __align__(16) unsigned char smem[];
+    int64_t* s_keys = reinterpret_cast<int64_t*>(smem); // reused for the values in the second round
+    uint16_t(*s_whist)[kRadix] = reinterpret_cast<uint16_t(*)[kRadix]>(smem + (size_t)kSortTile * 8);
+    uint32_t* s_digit_start = reinterpret_cast<uint32_t*>(smem + (size_t)kSortTile * 8 + (size_t)kSortWaves * kRadix * 2);
+    uint32_t* s_gbase = s_digit_start + kRadix;
+    uint32_t* s_wave_tot = s_gbase + kRadix;
+    uint32_t& s_tile = s_wave_tot[16];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -361,9 +419,8 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
 
     if(tid == 0)
         s_tile = atomicAdd(tile_counter, 1u);
-#pragma unroll
-    for(int w = 0; w < 4; ++w)
-        s_whist[w][tid] = 0;
+    for(int j = tid; j < kSortWaves * kRadix; j += kSortThreads)
+        (&s_whist[0][0])[j] = 0;
     __syncthreads();
     const int64_t tile = s_tile;
     const int64_t tile_base = tile * kSortTile;
@@ -372,7 +429,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
     // ---- load (striped inside each wavefront: coalesced, order = (item, lane)) -------------
     int64_t key[kSortItems];
     int32_t val[kSortItems];
-    uint32_t rank[kSortItems];
+    uint32_t pos[kSortItems];
 #pragma unroll
     for(int it = 0; it < kSortItems; ++it)
     {
@@ -390,47 +447,55 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
     }
 
     // ---- wave-local stable rank -----------------------------------------------------------
-    volatile uint32_t* wh = s_whist[wave];
+    // plain LDS accesses: a wavefront's LDS instructions execute in program order, and the
+    // compiler keeps the load/store order because both may touch the same counter
+    uint16_t* wh = s_whist[wave];
 #pragma unroll
     for(int it = 0; it < kSortItems; ++it)
     {
         const int local = wave * (kSortItems * 64) + it * 64 + lane;
         const bool valid = local < tile_n;
-        const uint32_t d = (uint32_t)(sortable(key[it]) >> shift) & (kRadix - 1);
+        const uint32_t d = (uint32_t)(sortable(key[it]) >> shift) & mask;
         const uint64_t m = match_digit(d, valid);
         const uint32_t below = (uint32_t)__popcll(m & lanemask_lt(lane));
         const uint32_t old = wh[d];
         __builtin_amdgcn_wave_barrier();
         if(valid && below == 0)
-            wh[d] = old + (uint32_t)__popcll(m);
+            wh[d] = (uint16_t)(old + (uint32_t)__popcll(m));
         __builtin_amdgcn_wave_barrier();
-        rank[it] = old + below;
+        pos[it] = old + below;
     }
     __syncthreads();
 
     // ---- per-digit totals of the tile (thread d <-> digit d), wave offsets, digit starts ----
-    uint32_t total;
+    const bool digit_thread = tid < kRadix; // thread d owns digit d (workgroups may be larger)
+    uint32_t total = 0;
+    uint32_t* my_status = status + tile * kRadix + (digit_thread ? tid : 0);
+    if(digit_thread)
     {
-        const uint32_t c0 = s_whist[0][tid], c1 = s_whist[1][tid], c2 = s_whist[2][tid], c3 = s_whist[3][tid];
-        s_whist[0][tid] = 0;
-        s_whist[1][tid] = c0;
-        s_whist[2][tid] = c0 + c1;
-        s_whist[3][tid] = c0 + c1 + c2;
-        total = c0 + c1 + c2 + c3;
+#pragma unroll
+        for(int w = 0; w < kSortWaves; ++w)
+        {
+            const uint32_t c = s_whist[w][tid];
+            s_whist[w][tid] = (uint16_t)total;
+            total += c;
+        }
+        // publish this tile's count as soon as it is known
+        __hip_atomic_store(my_status, total | (tile == 0 ? kFlagInclusive : kFlagAggregate), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
     }
-    // publish this tile's count as soon as it is known
-    uint32_t* my_status = status + tile * kRadix + tid;
-    __hip_atomic_store(my_status, total | (tile == 0 ? kFlagInclusive : kFlagAggregate), __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
     {
         const uint32_t incl = wave_incl_scan_u32(total, lane);
-        if(lane == 63)
+        if(digit_thread && lane == 63)
             s_wave_tot[wave] = incl;
         __syncthreads();
-        uint32_t prefix = 0;
-        for(int w = 0; w < wave; ++w)
-            prefix += s_wave_tot[w];
-        s_digit_start[tid] = prefix + incl - total;
+        if(digit_thread)
+        {
+            uint32_t prefix = 0;
+            for(int w = 0; w < wave; ++w)
+                prefix += s_wave_tot[w];
+            s_digit_start[tid] = prefix + incl - total;
+        }
     }
     __syncthreads();
 
@@ -441,38 +506,51 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
         const int local = wave * (kSortItems * 64) + it * 64 + lane;
         if(local < tile_n)
         {
-            const uint32_t d = (uint32_t)(sortable(key[it]) >> shift) & (kRadix - 1);
-            const uint32_t pos = s_digit_start[d] + s_whist[wave][d] + rank[it];
-            s_keys[pos] = key[it];
-            s_vals[pos] = val[it];
+            const uint32_t d = (uint32_t)(sortable(key[it]) >> shift) & mask;
+            pos[it] += s_digit_start[d] + s_whist[wave][d];
+            s_keys[pos[it]] = key[it];
         }
     }
 
     // ---- chained scan over earlier tiles (decoupled look-back), one thread per digit -------
+    if(digit_thread)
     {
         uint32_t excl = 0;
         if(tile > 0)
         {
-            int64_t t = tile - 1;
+            int64_t t = tile - 1; // next predecessor to account for
             int spins = 0;
-            while(true)
+            bool done = false;
+            while(!done)
             {
-                const uint32_t v =
-                    __hip_atomic_load(status + t * kRadix + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if((v & kFlagMask) == 0)
+                uint32_t v[kLookBatch];
+#pragma unroll
+                for(int b = 0; b < kLookBatch; ++b)
+                    v[b] = (t - b >= 0) ? __hip_atomic_load(status + (t - b) * kRadix + tid, __ATOMIC_RELAXED,
+                                                            __HIP_MEMORY_SCOPE_AGENT)
+                                        : kFlagInclusive;
+#pragma unroll
+                for(int b = 0; b < kLookBatch; ++b)
                 {
-                    if(++spins > kSpinLimit)
+                    if(done)
+                        break;
+                    if((v[b] & kFlagMask) == 0)
                     {
-                        *error_flag = 1u;
+                        // not published yet: poll again from this predecessor
+                        if(++spins > kSpinLimit)
+                        {
+                            *error_flag = 1u;
+                            done = true;
+                        }
+                        else
+                            __builtin_amdgcn_s_sleep(1);
                         break;
                     }
-                    __builtin_amdgcn_s_sleep(1);
-                    continue;
+                    excl += v[b] & kValueMask;
+                    --t;
+                    if(v[b] & kFlagInclusive)
+                        done = true;
                 }
-                excl += v & kValueMask;
-                if((v & kFlagInclusive) || t == 0)
-                    break;
-                --t;
             }
             __hip_atomic_store(my_status, ((excl + total) & kValueMask) | kFlagInclusive, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
@@ -481,7 +559,8 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
     }
     __syncthreads();
 
-    // ---- scatter: consecutive threads -> consecutive addresses inside a digit's run --------
+    // ---- scatter keys: consecutive threads -> consecutive addresses inside a digit's run ----
+    uint32_t out[kSortItems];
 #pragma unroll
     for(int it = 0; it < kSortItems; ++it)
     {
@@ -489,11 +568,29 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
         if(j < tile_n)
         {
             const int64_t kk = s_keys[j];
-            const uint32_t d = (uint32_t)(sortable(kk) >> shift) & (kRadix - 1);
-            const uint32_t out = s_gbase[d] + (uint32_t)j;
-            keys_out[out] = kk;
-            vals_out[out] = s_vals[j];
+            const uint32_t d = (uint32_t)(sortable(kk) >> shift) & mask;
+            out[it] = s_gbase[d] + (uint32_t)j;
+            keys_out[out[it]] = kk;
         }
+    }
+    __syncthreads();
+
+    // ---- values through the same buffer, same positions ------------------------------------
+    int32_t* s_vals = reinterpret_cast<int32_t*>(s_keys);
+#pragma unroll
+    for(int it = 0; it < kSortItems; ++it)
+    {
+        const int local = wave * (kSortItems * 64) + it * 64 + lane;
+        if(local < tile_n)
+            s_vals[pos[it]] = val[it];
+    }
+    __syncthreads();
+#pragma unroll
+    for(int it = 0; it < kSortItems; ++it)
+    {
+        const int j = it * kSortThreads + tid;
+        if(j < tile_n)
+            vals_out[out[it]] = s_vals[j];
     }
 }
 
@@ -508,6 +605,7 @@ int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values
     if(k >= (1ll << 30))
         return DSX_ERR_TOO_LARGE;
     const SortWorkspace w = sort_workspace(k, num_tiles);
+    const DigitPlan plan = digit_plan(num_tiles);
     char* base = static_cast<char*>(sort_ws);
     uint32_t* global_hist = reinterpret_cast<uint32_t*>(base + w.global_hist);
     uint32_t* counters = reinterpret_cast<uint32_t*>(base + w.counters);
@@ -517,17 +615,28 @@ int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values
     int rc = launch_fill_u32(global_hist, clear_words, 0u, stream);
     if(rc)
         return rc;
-    const int hist_blocks = (int)min((int64_t)2048, (k + 255) / 256);
+    const int64_t hist_chunks = (k + kHistThreads * kHistItems - 1) / (kHistThreads * kHistItems);
+    const int hist_blocks = (int)min((int64_t)2048, hist_chunks);
     {
         DSX_TIMED("radix_hist_kernel", stream);
-        hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks), dim3(256), 0, stream, keys_a, k, w.passes, global_hist);
+        hipLaunchKernelGGL(radix_hist_kernel, dim3(hist_blocks), dim3(kHistThreads), 0, stream, keys_a, k, plan,
+                           global_hist);
     }
     DSX_LAUNCH_CHECK();
     {
         DSX_TIMED("radix_hist_scan_kernel", stream);
-        hipLaunchKernelGGL(radix_hist_scan_kernel, dim3(w.passes), dim3(256), 0, stream, global_hist);
+        hipLaunchKernelGGL(radix_hist_scan_kernel, dim3(w.passes), dim3(kRadix), 0, stream, global_hist);
     }
     DSX_LAUNCH_CHECK();
+    // more than 64 KB of LDS per workgroup has to be requested explicitly (once per process)
+    static std::once_flag lds_once;
+    static hipError_t lds_status = hipSuccess;
+    std::call_once(lds_once, [] {
+        lds_status = hipFuncSetAttribute(reinterpret_cast<const void*>(radix_onesweep_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSortLdsBytes);
+    });
+    if(lds_status != hipSuccess)
+        return DSX_ERR_RUNTIME;
     int64_t* kin = keys_a;
     int32_t* vin = values_a;
     int64_t* kout = keys_b;
@@ -536,8 +645,8 @@ int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values
     {
         {
             DSX_TIMED("radix_onesweep_kernel", stream);
-            hipLaunchKernelGGL(radix_onesweep_kernel, dim3((unsigned)w.tiles), dim3(kSortThreads), 0, stream, kin, vin,
-                               kout, vout, k, p * kRadixBits, global_hist + p * kRadix,
+            hipLaunchKernelGGL(radix_onesweep_kernel, dim3((unsigned)w.tiles), dim3(kSortThreads), kSortLdsBytes, stream, kin,
+                               vin, kout, vout, k, plan.shift[p], plan.mask[p], global_hist + p * kRadix,
                                status + (size_t)p * w.tiles * kRadix, counters + p, counters + w.passes);
         }
         DSX_LAUNCH_CHECK();

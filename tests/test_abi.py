@@ -33,8 +33,8 @@ def test_host_helpers():
     assert lib.dsx_num_blocks(0) == 0 and lib.dsx_num_blocks(1) == 1 and lib.dsx_num_blocks(257) == 2
     assert lib.dsx_num_tiles(1920, 1080) == 120 * 68
     assert lib.dsx_num_tiles(40, 30) == 6
-    # 32 depth bits + bits for tile ids 0..T (slot 0 = negative keys), 8 bits a pass
-    assert lib.dsx_sort_passes(8160) == 6 and lib.dsx_sort_passes(255) == 5 and lib.dsx_sort_passes(32400) == 6
+    # 32 depth bits + bits for tile ids 0..T (slot 0 = negative keys), at most 9 bits a pass
+    assert lib.dsx_sort_passes(8160) == 5 and lib.dsx_sort_passes(255) == 5 and lib.dsx_sort_passes(32400) == 6
     assert lib.dsx_workspace_bytes(0, 0, 64, 64) >= 0
     assert lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080) > (1 << 20) * 24
     assert b"workspace" in lib.dsx_error_string(-5)
