@@ -1,8 +1,6 @@
 // Stages 4 and 5a for gfx950: per-tile alpha blending, forward (front to back) and backward
-// (back to front).  One 256-thread workgroup (4 wave64, each covering 4 pixel rows of 16)
-// per 16x16 tile; batches of 256 sorted entries are gathered into LDS as two float4 arrays
-// plus one float array, so the inner loop reads each entry with two 128-bit and one 32-bit
-// LDS broadcast.
+// (back to front).  Sorted entries are gathered into LDS in batches as two float4 arrays plus
+// one float array, so an entry costs two 128-bit and one 32-bit LDS broadcast read.
 #include "dsx_common.h"
 
 namespace dsx
@@ -19,87 +17,119 @@ __device__ __forceinline__ float fast_exp(float x)
 // -----------------------------------------------------------------------------------------
 // forward: cpp/rasterizer_kernels.cu:341-431
 // -----------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kTilePixels) void blend_fwd_kernel(const int32_t* __restrict__ ranges,
-                                                                const int32_t* __restrict__ ids,
-                                                                const float4* __restrict__ splats,
-                                                                float* __restrict__ image,
-                                                                float* __restrict__ final_T,
-                                                                int32_t* __restrict__ final_idx, int W, int H,
-                                                                int ntx)
-{
-    __shared__ float4 s_a[kTilePixels]; // pixel x, pixel y, conic a, conic b
-    __shared__ float4 s_b[kTilePixels]; // conic c, opacity, red, green
-    __shared__ float s_c[kTilePixels];  // blue
+// One wavefront per 16x16 tile, four pixels per lane (lane l owns column l & 15 of rows
+// (l >> 4) + {0, 4, 8, 12}).  Every LDS broadcast read of an entry then feeds 256 pixel
+// updates instead of 64, which moves the kernel from the LDS pipe to the VALU, gives each
+// lane four independent dependency chains, and needs no workgroup barrier at all.
+constexpr int kFwdBatch = 128; // sorted entries staged in LDS per round (two per lane)
+constexpr int kFwdPix = 4;
 
-    const int tid = threadIdx.x;
+__global__ __launch_bounds__(DSX_WAVE) void blend_fwd_kernel(const int32_t* __restrict__ ranges,
+                                                             const int32_t* __restrict__ ids,
+                                                             const float4* __restrict__ splats,
+                                                             float* __restrict__ image, float* __restrict__ final_T,
+                                                             int32_t* __restrict__ final_idx, int W, int H, int ntx)
+{
+    __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic a, conic b
+    __shared__ float4 s_b[kFwdBatch]; // conic c, opacity, red, green
+    __shared__ float s_c[kFwdBatch];  // blue
+
+    const int lane = threadIdx.x;
     const int tile = blockIdx.x;
     const int tx = tile % ntx;
     const int ty = tile / ntx;
-    const int x = tx * kTile + (tid & 15);
-    const int y = ty * kTile + (tid >> 4);
-    const bool inside = x < W && y < H;
+    const int x = tx * kTile + (lane & 15);
+    const int y0 = ty * kTile + (lane >> 4);
     const float pxf = (float)x + 0.5f;
-    const float pyf = (float)y + 0.5f;
 
     const int start = ranges[tile];
     const int end = ranges[tile + 1];
 
-    float T = 1.0f, cr = 0.0f, cg = 0.0f, cb = 0.0f;
-    int last = 0;
-    bool done = !inside;
-
-    for(int b = start; b < end; b += kTilePixels)
+    float pyf[kFwdPix], T[kFwdPix], cr[kFwdPix], cg[kFwdPix], cb[kFwdPix];
+    int last[kFwdPix];
+    bool done[kFwdPix];
+#pragma unroll
+    for(int p = 0; p < kFwdPix; ++p)
     {
-        if(__syncthreads_and(done))
+        const int y = y0 + 4 * p;
+        pyf[p] = (float)y + 0.5f;
+        T[p] = 1.0f;
+        cr[p] = cg[p] = cb[p] = 0.0f;
+        last[p] = 0;
+        done[p] = !(x < W && y < H);
+    }
+
+    for(int b = start; b < end; b += kFwdBatch)
+    {
+        if(__ballot(!(done[0] && done[1] && done[2] && done[3])) == 0)
             break;
-        const int e = b + tid;
-        if(e < end)
+        __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
+#pragma unroll
+        for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
         {
-            const int g = ids[e];
-            const float4* rec = splats + 3 * (int64_t)g;
-            const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
-            s_a[tid] = make_float4(q0.x, q0.y, q1.x, q1.y);
-            s_b[tid] = make_float4(q1.z, q1.w, q2.x, q2.y);
-            s_c[tid] = q2.z;
+            const int slot = h * DSX_WAVE + lane;
+            const int e = b + slot;
+            if(e < end)
+            {
+                const int g = ids[e];
+                const float4* rec = splats + 3 * (int64_t)g;
+                const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
+                s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
+                s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
+                s_c[slot] = q2.z;
+            }
         }
         __syncthreads();
-        const int cnt = min(kTilePixels, end - b);
-        if(!done)
+        const int cnt = min(kFwdBatch, end - b);
+        for(int i0 = 0; i0 < cnt; i0 += 2)
         {
-            for(int i = 0; i < cnt; ++i)
+            if(__ballot(!(done[0] && done[1] && done[2] && done[3])) == 0)
+                break;
+#pragma unroll
+            for(int u = 0; u < 2; ++u)
             {
-                const float4 A = s_a[i];
-                const float4 B = s_b[i];
+                const int i = i0 + u; // an entry past cnt holds stale data and is masked off
+                const float4 A = s_a[i & (kFwdBatch - 1)];
+                const float4 B = s_b[i & (kFwdBatch - 1)];
+                const float C = s_c[i & (kFwdBatch - 1)];
                 const float dx = pxf - A.x;
-                const float dy = pyf - A.y;
-                const float power = -0.5f * (A.z * dx * dx + B.x * dy * dy) - A.w * dx * dy;
-                const float alpha = fminf(0.999f, B.y * fast_exp(power));
-                if(power >= 0.0f || alpha < kAlphaThreshold)
-                    continue;
-                const float Tn = (1.0f - alpha) * T;
-                if(Tn < 0.0001f)
+                const float bx = A.w * dx;           // conic b * dx
+                const float ax = -0.5f * A.z * dx * dx; // -1/2 conic a * dx^2
+#pragma unroll
+                for(int p = 0; p < kFwdPix; ++p)
                 {
-                    done = true;
-                    break;
+                    const float dy = pyf[p] - A.y;
+                    const float power = ax - (0.5f * B.x * dy + bx) * dy;
+                    const float alpha = fminf(0.999f, B.y * fast_exp(power));
+                    const bool pass = i < cnt && !done[p] && power < 0.0f && alpha >= kAlphaThreshold;
+                    const float Tn = (1.0f - alpha) * T[p];
+                    const bool stop = pass && Tn < 0.0001f;
+                    const bool apply = pass && !stop;
+                    done[p] = done[p] || stop;
+                    const float vis = apply ? alpha * T[p] : 0.0f;
+                    cr[p] += vis * B.z;
+                    cg[p] += vis * B.w;
+                    cb[p] += vis * C;
+                    T[p] = apply ? Tn : T[p];
+                    last[p] = apply ? b + i : last[p];
                 }
-                const float vis = alpha * T;
-                cr += vis * B.z;
-                cg += vis * B.w;
-                cb += vis * s_c[i];
-                T = Tn;
-                last = b + i;
             }
         }
     }
 
-    if(inside)
+#pragma unroll
+    for(int p = 0; p < kFwdPix; ++p)
     {
-        const int64_t pix = (int64_t)y * W + x;
-        image[3 * pix] = cr;
-        image[3 * pix + 1] = cg;
-        image[3 * pix + 2] = cb;
-        final_T[pix] = T;
-        final_idx[pix] = last;
+        const int y = y0 + 4 * p;
+        if(x < W && y < H)
+        {
+            const int64_t pix = (int64_t)y * W + x;
+            image[3 * pix] = cr[p];
+            image[3 * pix + 1] = cg[p];
+            image[3 * pix + 2] = cb[p];
+            final_T[pix] = T[p];
+            final_idx[pix] = last[p];
+        }
     }
 }
 
@@ -111,7 +141,7 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
         return DSX_OK;
     {
         DSX_TIMED("blend_fwd_kernel", stream);
-        hipLaunchKernelGGL(blend_fwd_kernel, dim3(ntx * nty), dim3(kTilePixels), 0, stream, ranges, sorted_ids,
+        hipLaunchKernelGGL(blend_fwd_kernel, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
                            reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
                            cam.image_height, ntx);
     }
@@ -144,155 +174,197 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v)
     return v;
 }
 
-constexpr int kGradVals = 9;
+typedef unsigned int dsx_u32x2 __attribute__((ext_vector_type(2)));
 
-__global__ __launch_bounds__(kTilePixels) void blend_bwd_kernel(
+template <int kCtrl>
+__device__ __forceinline__ float dpp_move(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
+}
+
+// Sums eight per-lane values over the wavefront in 30 VALU instructions instead of 48: the
+// first two steps are a reduce-scatter inside each quad (a lane keeps half of the values and
+// hands the other half to its partner), the rest reduces the two remaining values across
+// quads, rows and halves (every lane ends up with totals).  The lanes of the last quad are
+// the ones that use them: lane 60 + q holds out0 = total of v[4*(q&1) + 2*(q>>1)] and out1 = total of the next index.
+__device__ __forceinline__ void wave_sum8_to_last_quad(const float (&v)[8], int lane, float& out0, float& out1)
+{
+    const bool b0 = lane & 1, b1 = lane & 2;
+    float r[4];
+#pragma unroll
+    for(int i = 0; i < 4; ++i)
+    {
+        const float keep = b0 ? v[4 + i] : v[i];
+        const float send = b0 ? v[i] : v[4 + i];
+        r[i] = keep + dpp_move<0xB1>(send); // quad_perm [1,0,3,2]
+    }
+    float q[2];
+#pragma unroll
+    for(int i = 0; i < 2; ++i)
+    {
+        const float keep = b1 ? r[2 + i] : r[i];
+        const float send = b1 ? r[i] : r[2 + i];
+        q[i] = keep + dpp_move<0x4E>(send); // quad_perm [2,3,0,1]
+    }
+#pragma unroll
+    for(int i = 0; i < 2; ++i)
+    {
+        q[i] += dpp_move<0x124>(q[i]); // row_ror:4  -> two quads
+        q[i] += dpp_move<0x128>(q[i]); // row_ror:8  -> the whole row of 16
+        // across rows the lanes must keep their position inside the quad, so the row
+        // broadcasts of the single-value reduction cannot be used: swap rows, then halves
+        const dsx_u32x2 r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(q[i]), __float_as_uint(q[i]), false, false);
+        q[i] = __uint_as_float(r16.x) + __uint_as_float(r16.y);
+        const dsx_u32x2 r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(q[i]), __float_as_uint(q[i]), false, false);
+        q[i] = __uint_as_float(r32.x) + __uint_as_float(r32.y);
+    }
+    out0 = q[0];
+    out1 = q[1];
+}
+
+constexpr int kBwdBatch = 128; // sorted entries staged in LDS per round (two per lane)
+constexpr int kBwdPix = 4;
+
+// One wavefront per 16x16 tile, four pixels per lane (same pixel ownership as the forward).
+// The per-Gaussian gradients are first summed over a lane's four pixels, then over the
+// wavefront with DPP adds, and lane 63 issues ONE set of hardware float atomics per
+// (tile, entry).  Compared with four wavefronts of one pixel per lane this does one
+// cross-lane reduction per entry instead of four and needs no LDS accumulators or barriers.
+__global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const int32_t* __restrict__ ranges, const int32_t* __restrict__ ids, const float4* __restrict__ splats,
     const float* __restrict__ final_T, const int32_t* __restrict__ final_idx, const float* __restrict__ v_image,
     const float* __restrict__ bg, float* grads, int W, int H, int ntx)
 {
-    __shared__ float4 s_a[kTilePixels]; // pixel x, pixel y, conic a, conic b
-    __shared__ float4 s_b[kTilePixels]; // conic c, opacity, red, green
-    __shared__ float s_c[kTilePixels];  // blue
-    __shared__ int s_id[kTilePixels];
-    __shared__ float s_acc[kTilePixels * kGradVals]; // per-entry sums over the four wavefronts
-    __shared__ int s_wave_max[4];
+    __shared__ float4 s_a[kBwdBatch]; // pixel x, pixel y, conic a, conic b
+    __shared__ float4 s_b[kBwdBatch]; // conic c, opacity, red, green
+    __shared__ float s_c[kBwdBatch];  // blue
+    __shared__ int s_id[kBwdBatch];
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int lane = threadIdx.x;
     const int tile = blockIdx.x;
     const int tx = tile % ntx;
     const int ty = tile / ntx;
-    const int x = tx * kTile + (tid & 15);
-    const int y = ty * kTile + (tid >> 4);
-    const bool inside = x < W && y < H;
+    const int x = tx * kTile + (lane & 15);
+    const int y0 = ty * kTile + (lane >> 4);
     const float pxf = (float)x + 0.5f;
-    const float pyf = (float)y + 0.5f;
-    const int64_t pix = inside ? (int64_t)y * W + x : 0;
+    const float bg0 = bg[0], bg1 = bg[1], bg2 = bg[2];
 
-    const float T_final = inside ? final_T[pix] : 0.0f;
-    const int bin_final = inside ? final_idx[pix] : -1;
-    float vo0 = 0.f, vo1 = 0.f, vo2 = 0.f;
-    if(inside)
+    // bterm = -T_final * (bg . v_out) - sum over the entries behind of (rgb . v_out) * alpha * T:
+    // the three per-channel colour buffers of cpp/gsplat/backward.cu:156-168 only ever appear
+    // dotted with v_out, so one scalar carries them
+    float pyf[kBwdPix], T[kBwdPix], vo0[kBwdPix], vo1[kBwdPix], vo2[kBwdPix], bterm[kBwdPix];
+    int bin_final[kBwdPix];
+    int m = -1;
+#pragma unroll
+    for(int p = 0; p < kBwdPix; ++p)
     {
-        vo0 = v_image[3 * pix];
-        vo1 = v_image[3 * pix + 1];
-        vo2 = v_image[3 * pix + 2];
+        const int y = y0 + 4 * p;
+        const bool inside = x < W && y < H;
+        const int64_t pix = inside ? (int64_t)y * W + x : 0;
+        pyf[p] = (float)y + 0.5f;
+        const float Tf = inside ? final_T[pix] : 0.0f;
+        T[p] = Tf;
+        bin_final[p] = inside ? final_idx[pix] : -1;
+        vo0[p] = inside ? v_image[3 * pix] : 0.f;
+        vo1[p] = inside ? v_image[3 * pix + 1] : 0.f;
+        vo2[p] = inside ? v_image[3 * pix + 2] : 0.f;
+        bterm[p] = -Tf * (bg0 * vo0[p] + bg1 * vo1[p] + bg2 * vo2[p]);
+        m = max(m, bin_final[p]);
     }
-    // -T_final * bg . v_out  (background term of cpp/gsplat/backward.cu:160-164, times ra later)
-    const float bg_term = -T_final * (bg[0] * vo0 + bg[1] * vo1 + bg[2] * vo2);
 
     const int start = ranges[tile];
     const int end = ranges[tile + 1];
 
-    // last entry any pixel of this wavefront / of this tile blended
-    int m = bin_final;
+    // last entry any pixel of this tile blended
 #pragma unroll
     for(int o = 32; o > 0; o >>= 1)
         m = max(m, __shfl_xor(m, o, DSX_WAVE));
-    if(lane == 0)
-        s_wave_max[wave] = m;
-    __syncthreads();
-    const int wave_last = m;
-    const int tile_last = max(max(s_wave_max[0], s_wave_max[1]), max(s_wave_max[2], s_wave_max[3]));
-    const int hi = min(end - 1, tile_last);
+    const int hi = min(end - 1, m);
 
-    float T = T_final;
-    float buf0 = 0.f, buf1 = 0.f, buf2 = 0.f;
-
-    for(int top = hi; top >= start; top -= kTilePixels)
+    for(int top = hi; top >= start; top -= kBwdBatch)
     {
-        __syncthreads(); // previous batch fully consumed (staging and accumulators)
-        const int e = top - tid;
-        if(e >= start)
-        {
-            const int g = ids[e];
-            const float4* rec = splats + 3 * (int64_t)g;
-            const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
-            s_a[tid] = make_float4(q0.x, q0.y, q1.x, q1.y);
-            s_b[tid] = make_float4(q1.z, q1.w, q2.x, q2.y);
-            s_c[tid] = q2.z;
-            s_id[tid] = g;
-        }
+        __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
 #pragma unroll
-        for(int j = 0; j < kGradVals; ++j)
-            s_acc[j * kTilePixels + tid] = 0.f;
+        for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
+        {
+            const int slot = h * DSX_WAVE + lane;
+            const int e = top - slot;
+            if(e >= start)
+            {
+                const int g = ids[e];
+                const float4* rec = splats + 3 * (int64_t)g;
+                const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
+                s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
+                s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
+                s_c[slot] = q2.z;
+                s_id[slot] = g;
+            }
+        }
         __syncthreads();
-        const int cnt = min(kTilePixels, top - start + 1);
-        // entries beyond what any lane of this wavefront blended are skipped outright
-        for(int t = max(0, top - wave_last); t < cnt; ++t)
+        const int cnt = min(kBwdBatch, top - start + 1);
+        for(int t = 0; t < cnt; ++t)
         {
             const int idx = top - t;
-            bool valid = idx <= bin_final;
-            float alpha = 0.f, vis = 0.f, dx = 0.f, dy = 0.f;
             const float4 A = s_a[t];
             const float4 B = s_b[t];
-            if(valid)
-            {
-                dx = A.x - pxf;
-                dy = A.y - pyf;
-                const float sigma = 0.5f * (A.z * dx * dx + B.x * dy * dy) + A.w * dx * dy;
-                vis = fast_exp(-sigma);
-                alpha = fminf(0.99f, B.y * vis);
-                if(sigma < 0.0f || alpha < kAlphaThreshold)
-                    valid = false;
-            }
-            if(__ballot(valid) == 0)
-                continue;
-            float g[kGradVals] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            if(valid)
-            {
-                const float ra = __builtin_amdgcn_rcpf(1.0f - alpha);
-                T *= ra;
-                const float fac = alpha * T;
-                g[6] = fac * vo0;
-                g[7] = fac * vo1;
-                g[8] = fac * vo2;
-                const float blue = s_c[t];
-                float v_alpha = (B.z * T - buf0 * ra) * vo0;
-                v_alpha += (B.w * T - buf1 * ra) * vo1;
-                v_alpha += (blue * T - buf2 * ra) * vo2;
-                v_alpha += bg_term * ra;
-                buf0 += B.z * fac;
-                buf1 += B.w * fac;
-                buf2 += blue * fac;
-                const float v_sigma = -B.y * vis * v_alpha;
-                g[0] = v_sigma * (A.z * dx + A.w * dy);
-                g[1] = v_sigma * (A.w * dx + B.x * dy);
-                g[2] = 0.5f * v_sigma * dx * dx;
-                g[3] = v_sigma * dx * dy;
-                g[4] = 0.5f * v_sigma * dy * dy;
-                g[5] = vis * v_alpha;
-            }
-#pragma unroll
-            for(int j = 0; j < kGradVals; ++j)
-                g[j] = wave_sum_to_lane63(g[j]);
-            if(lane == 63)
-            {
-#pragma unroll
-                for(int j = 0; j < kGradVals; ++j)
-                    atomicAdd(&s_acc[j * kTilePixels + t], g[j]);
-            }
-        }
-        __syncthreads();
-        // one set of global atomics per (tile, entry): thread t flushes entry t
-        if(tid < cnt)
-        {
-            float v[kGradVals];
+            const float dx = A.x - pxf;
+            const float adx2 = A.z * dx * dx;
+            const float bdx = A.w * dx;
+            float alpha[kBwdPix], vis[kBwdPix], dy[kBwdPix];
+            bool valid[kBwdPix];
             bool any = false;
 #pragma unroll
-            for(int j = 0; j < kGradVals; ++j)
+            for(int p = 0; p < kBwdPix; ++p)
             {
-                v[j] = s_acc[j * kTilePixels + tid];
-                any = any || v[j] != 0.f;
+                dy[p] = A.y - pyf[p];
+                const float sigma = 0.5f * (adx2 + B.x * dy[p] * dy[p]) + bdx * dy[p];
+                vis[p] = fast_exp(-sigma);
+                alpha[p] = fminf(0.99f, B.y * vis[p]);
+                valid[p] = idx <= bin_final[p] && !(sigma < 0.0f) && !(alpha[p] < kAlphaThreshold);
+                any = any || valid[p];
             }
-            if(any)
-            {
-                float* dst = grads + (int64_t)s_id[tid] * DSX_GRAD_FLOATS;
+            if(__ballot(any) == 0)
+                continue;
+            const float blue = s_c[t];
+            const float hdx2 = 0.5f * dx * dx;
+            const float adx = A.z * dx;
+            float g[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; // v_x, v_y, v_conic a b c, v_opacity, v_red, v_green
+            float g_blue = 0.f;
 #pragma unroll
-                for(int j = 0; j < kGradVals; ++j)
-                    unsafeAtomicAdd(dst + j, v[j]);
+            for(int p = 0; p < kBwdPix; ++p)
+            {
+                if(valid[p])
+                {
+                    const float ra = __builtin_amdgcn_rcpf(1.0f - alpha[p]);
+                    T[p] *= ra;
+                    const float fac = alpha[p] * T[p];
+                    g[6] += fac * vo0[p];
+                    g[7] += fac * vo1[p];
+                    g_blue += fac * vo2[p];
+                    const float rv = B.z * vo0[p] + B.w * vo1[p] + blue * vo2[p];
+                    const float v_alpha = rv * T[p] + bterm[p] * ra;
+                    bterm[p] -= rv * fac;
+                    const float v_sigma = -B.y * vis[p] * v_alpha;
+                    g[0] += v_sigma * (adx + A.w * dy[p]);
+                    g[1] += v_sigma * (bdx + B.x * dy[p]);
+                    g[2] += v_sigma * hdx2;
+                    g[3] += v_sigma * dx * dy[p];
+                    g[4] += 0.5f * v_sigma * dy[p] * dy[p];
+                    g[5] += vis[p] * v_alpha;
+                }
+            }
+            float s0, s1;
+            wave_sum8_to_last_quad(g, lane, s0, s1);
+            g_blue = wave_sum_to_lane63(g_blue);
+            if(lane >= 60)
+            {
+                // lane 60 + q holds the totals of g[4*(q&1) + 2*(q>>1)] and of the next index
+                const int q = lane - 60;
+                float* dst = grads + (int64_t)s_id[t] * DSX_GRAD_FLOATS + 4 * (q & 1) + 2 * (q >> 1);
+                unsafeAtomicAdd(dst, s0);
+                unsafeAtomicAdd(dst + 1, s1);
+                if(lane == 63)
+                    unsafeAtomicAdd(grads + (int64_t)s_id[t] * DSX_GRAD_FLOATS + 8, g_blue);
             }
         }
     }
@@ -310,7 +382,7 @@ int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, co
         return DSX_OK;
     {
         DSX_TIMED("blend_bwd_kernel", stream);
-        hipLaunchKernelGGL(blend_bwd_kernel, dim3(ntx * nty), dim3(kTilePixels), 0, stream, ranges, sorted_ids,
+        hipLaunchKernelGGL(blend_bwd_kernel, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
                            reinterpret_cast<const float4*>(splats), final_T, final_idx, v_image, cam.bg, grads,
                            cam.image_width, cam.image_height, ntx);
     }
