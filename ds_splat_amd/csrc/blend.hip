@@ -14,6 +14,34 @@ __device__ __forceinline__ float fast_exp(float x)
     return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
 }
 
+// Can this entry reach alpha >= 1/255 at ANY pixel of the tile?  The exponent's quadratic form
+// q(d) = 1/2 (a dx^2 + c dy^2) + b dx dy is convex, so its minimum over the box of pixel
+// centres is 0 if the centre lies inside and otherwise sits on one of the four edges, where it
+// is a clamped one-dimensional parabola.  An entry is dropped only if opacity * exp(-qmin)
+// stays below 0.99/255 (one percent of slack against rounding); whatever fails a comparison
+// (NaN, degenerate conic) is kept.  The reference's tile rectangle is the bounding square of a
+// 3-sigma circle, so about half of the (tile, entry) pairs a tile walks touch none of its pixels.
+__device__ __forceinline__ float edge_min(float a, float b, float c, float u, float v0, float v1)
+{
+    // minimum over v in [v0, v1] of 1/2 (a u^2 + c v^2) + b u v   (u fixed, c > 0)
+    const float v = fminf(v1, fmaxf(v0, -b * u * __builtin_amdgcn_rcpf(c)));
+    return 0.5f * (a * u * u + c * v * v) + b * u * v;
+}
+
+__device__ __forceinline__ bool entry_reaches_tile(float mx, float my, float a, float b, float c, float opacity,
+                                                   float box_x0, float box_y0)
+{
+    const float dx0 = box_x0 - mx, dx1 = box_x0 + 15.0f - mx;
+    const float dy0 = box_y0 - my, dy1 = box_y0 + 15.0f - my;
+    const bool inside = dx0 <= 0.0f && dx1 >= 0.0f && dy0 <= 0.0f && dy1 >= 0.0f;
+    float qmin = fminf(fminf(edge_min(a, b, c, dx0, dy0, dy1), edge_min(a, b, c, dx1, dy0, dy1)),
+                       fminf(edge_min(c, b, a, dy0, dx0, dx1), edge_min(c, b, a, dy1, dx0, dx1)));
+    qmin = inside ? 0.0f : qmin;
+    const bool well_formed = a > 0.0f && c > 0.0f;
+    const float limit = __logf(opacity * (255.0f / 0.99f)); // ln(opacity / (0.99/255))
+    return !(well_formed && qmin > limit);
+}
+
 // -----------------------------------------------------------------------------------------
 // forward: cpp/rasterizer_kernels.cu:341-431
 // -----------------------------------------------------------------------------------------
@@ -41,6 +69,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_fwd_kernel(const int32_t* __re
     const int x = tx * kTile + (lane & 15);
     const int y0 = ty * kTile + (lane >> 4);
     const float pxf = (float)x + 0.5f;
+    const float box_x0 = (float)(tx * kTile) + 0.5f, box_y0 = (float)(ty * kTile) + 0.5f; // first pixel centre
 
     const int start = ranges[tile];
     const int end = ranges[tile + 1];
@@ -64,11 +93,13 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_fwd_kernel(const int32_t* __re
         if(__ballot(!(done[0] && done[1] && done[2] && done[3])) == 0)
             break;
         __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
+        uint64_t todo[kFwdBatch / DSX_WAVE]; // entries of this round that can touch the tile
 #pragma unroll
         for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
         {
             const int slot = h * DSX_WAVE + lane;
             const int e = b + slot;
+            bool useful = false;
             if(e < end)
             {
                 const int g = ids[e];
@@ -77,21 +108,24 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_fwd_kernel(const int32_t* __re
                 s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
                 s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
+                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0);
             }
+            todo[h] = __ballot(useful);
         }
         __syncthreads();
-        const int cnt = min(kFwdBatch, end - b);
-        for(int i0 = 0; i0 < cnt; i0 += 2)
-        {
-            if(__ballot(!(done[0] && done[1] && done[2] && done[3])) == 0)
-                break;
 #pragma unroll
-            for(int u = 0; u < 2; ++u)
+        for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
+        {
+            uint64_t mask = todo[h];
+            while(mask != 0)
             {
-                const int i = i0 + u; // an entry past cnt holds stale data and is masked off
-                const float4 A = s_a[i & (kFwdBatch - 1)];
-                const float4 B = s_b[i & (kFwdBatch - 1)];
-                const float C = s_c[i & (kFwdBatch - 1)];
+                if(__ballot(!(done[0] && done[1] && done[2] && done[3])) == 0)
+                    break;
+                const int i = h * DSX_WAVE + __builtin_ctzll(mask);
+                mask &= mask - 1;
+                const float4 A = s_a[i];
+                const float4 B = s_b[i];
+                const float C = s_c[i];
                 const float dx = pxf - A.x;
                 const float bx = A.w * dx;           // conic b * dx
                 const float ax = -0.5f * A.z * dx * dx; // -1/2 conic a * dx^2
@@ -101,7 +135,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_fwd_kernel(const int32_t* __re
                     const float dy = pyf[p] - A.y;
                     const float power = ax - (0.5f * B.x * dy + bx) * dy;
                     const float alpha = fminf(0.999f, B.y * fast_exp(power));
-                    const bool pass = i < cnt && !done[p] && power < 0.0f && alpha >= kAlphaThreshold;
+                    const bool pass = !done[p] && power < 0.0f && alpha >= kAlphaThreshold;
                     const float Tn = (1.0f - alpha) * T[p];
                     const bool stop = pass && Tn < 0.0001f;
                     const bool apply = pass && !stop;
@@ -247,6 +281,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const int x = tx * kTile + (lane & 15);
     const int y0 = ty * kTile + (lane >> 4);
     const float pxf = (float)x + 0.5f;
+    const float box_x0 = (float)(tx * kTile) + 0.5f, box_y0 = (float)(ty * kTile) + 0.5f; // first pixel centre
     const float bg0 = bg[0], bg1 = bg[1], bg2 = bg[2];
 
     // bterm = -T_final * (bg . v_out) - sum over the entries behind of (rgb . v_out) * alpha * T:
@@ -284,11 +319,13 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     for(int top = hi; top >= start; top -= kBwdBatch)
     {
         __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
+        uint64_t todo[kBwdBatch / DSX_WAVE]; // entries of this round that can touch the tile
 #pragma unroll
         for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
         {
             const int slot = h * DSX_WAVE + lane;
             const int e = top - slot;
+            bool useful = false;
             if(e >= start)
             {
                 const int g = ids[e];
@@ -298,12 +335,16 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
                 s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
                 s_id[slot] = g;
+                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0);
             }
+            todo[h] = __ballot(useful);
         }
         __syncthreads();
-        const int cnt = min(kBwdBatch, top - start + 1);
-        for(int t = 0; t < cnt; ++t)
+#pragma unroll
+        for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
+        for(uint64_t mask = todo[h]; mask != 0; mask &= mask - 1)
         {
+            const int t = h * DSX_WAVE + __builtin_ctzll(mask);
             const int idx = top - t;
             const float4 A = s_a[t];
             const float4 B = s_b[t];

@@ -36,18 +36,22 @@ __device__ __forceinline__ int wave_incl_max_i32(int v, int lane)
     return v;
 }
 
-// lanes of the wavefront that hold the same (up to 9-bit) digit and are valid; call in uniform flow
+// lanes of the wavefront that hold the same (up to 9-bit) digit and are valid; call in uniform
+// flow.  Per digit bit: one sign-extending bit extract, one compare (the ballot) and, for each
+// half of the lane mask, one three-input boolean op  mask & ~(ballot ^ bit).
 __device__ __forceinline__ uint64_t match_digit(uint32_t d, bool valid)
 {
-    uint64_t mask = __ballot(valid);
+    const uint64_t v = __ballot(valid);
+    uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
 #pragma unroll
     for(int b = 0; b < kRadixBitsMax; ++b)
     {
-        const bool bit = (d >> b) & 1u;
-        const uint64_t m = __ballot(bit);
-        mask &= bit ? m : ~m;
+        const uint32_t x = (uint32_t)(((int32_t)(d << (31 - b))) >> 31); // all ones where bit b is set
+        const uint64_t m = __ballot(x != 0);
+        lo &= ~((uint32_t)m ^ x);
+        hi &= ~((uint32_t)(m >> 32) ^ x);
     }
-    return mask;
+    return ((uint64_t)hi << 32) | lo;
 }
 
 __device__ __forceinline__ uint64_t lanemask_lt(int lane)
@@ -387,7 +391,10 @@ constexpr uint32_t kFlagInclusive = 2u << 30;
 constexpr uint32_t kFlagMask = 3u << 30;
 constexpr uint32_t kValueMask = ~kFlagMask;
 constexpr int kSpinLimit = 1 << 18; // bounded wait: a stuck predecessor ends in an error flag, not a hang
-constexpr int kLookBatch = 4;       // predecessor statuses fetched per round trip
+#ifndef DSX_LOOK_BATCH
+#define DSX_LOOK_BATCH 4
+#endif
+constexpr int kLookBatch = DSX_LOOK_BATCH; // predecessor statuses fetched per round trip
 constexpr int kSortWaves = kSortThreads / DSX_WAVE;
 
 // One digit pass.  Tile = kSortTile consecutive keys, taken in arrival order through a dynamic
@@ -430,6 +437,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
     int64_t key[kSortItems];
     int32_t val[kSortItems];
     uint32_t pos[kSortItems];
+    uint32_t dig[kSortItems];
 #pragma unroll
     for(int it = 0; it < kSortItems; ++it)
     {
@@ -456,6 +464,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
         const int local = wave * (kSortItems * 64) + it * 64 + lane;
         const bool valid = local < tile_n;
         const uint32_t d = (uint32_t)(sortable(key[it]) >> shift) & mask;
+        dig[it] = d;
         const uint64_t m = match_digit(d, valid);
         const uint32_t below = (uint32_t)__popcll(m & lanemask_lt(lane));
         const uint32_t old = wh[d];
@@ -506,7 +515,7 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
         const int local = wave * (kSortItems * 64) + it * 64 + lane;
         if(local < tile_n)
         {
-            const uint32_t d = (uint32_t)(sortable(key[it]) >> shift) & mask;
+            const uint32_t d = dig[it];
             pos[it] += s_digit_start[d] + s_whist[wave][d];
             s_keys[pos[it]] = key[it];
         }
@@ -526,9 +535,11 @@ __global__ __launch_bounds__(kSortThreads) void radix_onesweep_kernel(
                 uint32_t v[kLookBatch];
 #pragma unroll
                 for(int b = 0; b < kLookBatch; ++b)
-                    v[b] = (t - b >= 0) ? __hip_atomic_load(status + (t - b) * kRadix + tid, __ATOMIC_RELAXED,
-                                                            __HIP_MEMORY_SCOPE_AGENT)
-                                        : kFlagInclusive;
+                {
+                    // rows below tile 0 are read as tile 0, whose status is inclusive from the start
+                    const int64_t row = t - b > 0 ? t - b : 0;
+                    v[b] = __hip_atomic_load(status + row * kRadix + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
 #pragma unroll
                 for(int b = 0; b < kLookBatch; ++b)
                 {
