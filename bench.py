@@ -39,8 +39,6 @@ def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, passes, counters):
         return "hbm", 24 * k, "B"
     if kernel == "radix_hist_kernel":
         return "hbm", 8 * k, "B"
-    if kernel == "ranges_boundaries_kernel":
-        return "hbm", 8 * k + 4 * (tiles + 1), "B"
     if kernel == "blend_fwd_kernel" and counters is not None:
         rej = counters.pairs_fwd - counters.pairs_fwd_applied
         return "valu", counters.pairs_fwd_applied * FWD_PAIR_FLOPS + rej * FWD_REJECT_FLOPS, "FLOP"

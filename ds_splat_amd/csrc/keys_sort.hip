@@ -24,18 +24,6 @@ __device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t v, int lane)
     return v;
 }
 
-__device__ __forceinline__ int wave_incl_max_i32(int v, int lane)
-{
-#pragma unroll
-    for(int o = 1; o < DSX_WAVE; o <<= 1)
-    {
-        const int t = __shfl_up(v, o, DSX_WAVE);
-        if(lane >= o)
-            v = max(v, t);
-    }
-    return v;
-}
-
 // lanes of the wavefront that hold the same (up to 9-bit) digit and are valid; call in uniform
 // flow.  Per digit bit: one sign-extending bit extract, one compare (the ballot) and, for each
 // half of the lane mask, one three-input boolean op  mask & ~(ballot ^ bit).
@@ -677,83 +665,45 @@ int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values
 // tile ranges
 // ---------------------------------------------------------------------------------------
 
-__global__ __launch_bounds__(256) void ranges_init_kernel(int32_t* ranges, int num_tiles, int32_t k)
+// ranges[j] = number of keys whose tile is below j, by binary search in the sorted keys: one
+// thread per tile, about log2(K) dependent loads each, instead of a pass over all K keys.
+// Two rules of the reference are kept (cpp/rasterizer_kernels.cu:313-322,
+// cpp/rasterizer_torch.cu:31-39): the boundary after the LAST run is never recorded, so tiles
+// above the highest occupied tile inherit the START of that run, and ranges[num_tiles] = K.
+// Keys with a negative depth carry tile -1 and sort first; ranges[0] skips them.
+__global__ __launch_bounds__(256) void ranges_search_kernel(const int64_t* __restrict__ keys, int64_t k,
+                                                            int num_tiles, int32_t* __restrict__ ranges)
 {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if(i < num_tiles)
-        ranges[i] = 0;
-    else if(i == num_tiles)
-        ranges[i] = k;
-}
-
-// where the tile field changes between neighbours, the next index starts the following tile
-__global__ __launch_bounds__(256) void ranges_boundaries_kernel(const int64_t* __restrict__ keys, int64_t k,
-                                                                int32_t* ranges)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if(i + 1 < k)
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if(j > num_tiles)
+        return;
+    if(j == num_tiles || k == 0)
     {
-        const int32_t cur = (int32_t)(keys[i] >> 32);
-        const int32_t nxt = (int32_t)(keys[i + 1] >> 32);
-        if(cur != nxt)
-            ranges[cur + 1] = (int32_t)(i + 1);
+        ranges[j] = j == num_tiles ? (int32_t)k : 0;
+        return;
     }
-}
-
-// inclusive running maximum over num_tiles+1 entries (one workgroup): empty tiles inherit the
-// end of the previous run
-__global__ __launch_bounds__(1024) void ranges_maxscan_kernel(int32_t* ranges, int count)
-{
-    __shared__ int wave_max[16];
-    __shared__ int carry_s;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    if(tid == 0)
-        carry_s = INT32_MIN;
-    __syncthreads();
-    for(int base = 0; base < count; base += 1024)
+    const int64_t last_tile = keys[k - 1] >> 32; // arithmetic shift: -1 for negative keys
+    const int64_t target_tile = j < last_tile ? j : last_tile;
+    const int64_t target = (int64_t)((uint64_t)target_tile << 32);
+    int64_t lo = 0, hi = k; // first index with keys[i] >= target
+    while(lo < hi)
     {
-        const int i = base + tid;
-        const int v = i < count ? ranges[i] : INT32_MIN;
-        int incl = wave_incl_max_i32(v, lane);
-        if(lane == 63)
-            wave_max[wave] = incl;
-        __syncthreads();
-        int prev = carry_s;
-        for(int w = 0; w < wave; ++w)
-            prev = max(prev, wave_max[w]);
-        incl = max(incl, prev);
-        if(i < count)
-            ranges[i] = incl;
-        __syncthreads();
-        if(tid == 1023)
-            carry_s = incl;
-        __syncthreads();
+        const int64_t mid = (lo + hi) >> 1;
+        if(keys[mid] < target)
+            lo = mid + 1;
+        else
+            hi = mid;
     }
+    ranges[j] = (int32_t)lo;
 }
 
 int launch_tile_ranges(int64_t k, const int64_t* sorted_keys, int num_tiles, int32_t* ranges, hipStream_t stream)
 {
     const int count = num_tiles + 1;
     {
-        DSX_TIMED("ranges_init_kernel", stream);
-        hipLaunchKernelGGL(ranges_init_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, ranges, num_tiles,
-                           (int32_t)k);
-    }
-    DSX_LAUNCH_CHECK();
-    if(k > 1)
-    {
-        {
-            DSX_TIMED("ranges_boundaries_kernel", stream);
-            hipLaunchKernelGGL(ranges_boundaries_kernel, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, stream,
-                               sorted_keys, k, ranges);
-        }
-        DSX_LAUNCH_CHECK();
-    }
-    {
-        DSX_TIMED("ranges_maxscan_kernel", stream);
-        hipLaunchKernelGGL(ranges_maxscan_kernel, dim3(1), dim3(1024), 0, stream, ranges, count);
+        DSX_TIMED("ranges_search_kernel", stream);
+        hipLaunchKernelGGL(ranges_search_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, sorted_keys, k,
+                           num_tiles, ranges);
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
