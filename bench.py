@@ -27,6 +27,19 @@ FWD_PAIR_FLOPS, FWD_REJECT_FLOPS = 25, 15
 BWD_PAIR_FLOPS, BWD_REJECT_FLOPS = 72, 15
 
 
+# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counters (two rocprofv3 --pmc runs of this
+# script with --copy-probe, each counter scaled by its reading for the 1 GiB copy; summary in
+# profiles/cfg2_hbm_traffic_per_kernel.md).  Counters cannot be read from inside this process, so
+# the figures are quoted here and only reported when workload and key count are the profiled ones.
+MEASURED_TRAFFIC = {
+    ("cfg2", 32604809): {
+        "project_fwd_kernel": 936.5e6, "emit_keys_kernel": 536.9e6, "radix_hist_kernel": 275.4e6,
+        "radix_onesweep_kernel": 908.5e6, "gaussian_bwd_kernel": 1333.2e6,
+        "blend_fwd_kernel": 78.5e6, "blend_bwd_kernel": 194.1e6,
+    },
+}
+
+
 def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, passes, counters):
     """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch."""
     if kernel == "project_fwd_kernel":
@@ -57,6 +70,8 @@ def main():
     ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--verbose", action="store_true", help="per-kernel table on stderr")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one 1 GiB device copy (a kernel of known traffic that scales HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding "
@@ -100,6 +115,12 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if args.copy_probe:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     _native.trace_enable(True)
     _native.trace_read()
@@ -180,6 +201,9 @@ def main():
                         "unit": "TFLOP/s", "frac": round(achieved / VALU_PEAK_TFLOPS, 4), "traffic": None,
                         "avg_launch_ms": round(avg, 4), "launches_per_step": lps,
                         "algorithmic_flop_per_launch": int(work)}
+        if args.n is None:
+            traffic = MEASURED_TRAFFIC.get((spec.name, int(k)), {}).get(name)
+            roofline["traffic"] = int(traffic) if traffic else None
         break
     if args.verbose:
         for ms_step, name, avg, lps, bound, work, unit in table:

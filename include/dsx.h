@@ -5,8 +5,10 @@
  * is marked "host".  `stream` is a hipStream_t passed as void* (NULL = the null stream).
  * The library allocates nothing on the device: outputs and workspace are the caller's.
  * All functions return 0 on success or a negative dsx_status; dsx_error_string() explains it.
- * Functions are re-entrant: no global mutable state, so different streams / devices may be
- * driven concurrently by different host threads (each call uses the current HIP device).
+ * Functions are re-entrant: the compute path keeps no global mutable state, so different
+ * streams / devices may be driven concurrently by different host threads (each call uses the
+ * current HIP device).  The one exception is the optional per-kernel timing trace
+ * (dsx_trace_enable / dsx_trace_read), a process-wide list behind a mutex, off by default.
  *
  * What each entry point replaces in the reference (deepsense-ai/ds-splat) is cited as
  * file:line next to it.  Matrices are row-major, math convention (translation in elements
