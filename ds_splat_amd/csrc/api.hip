@@ -139,13 +139,48 @@ extern "C" int32_t dsx_sort_passes(int32_t num_tiles)
 extern "C" size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height)
 {
     (void)n;
-    return forward_workspace(k < 0 ? 0 : k, dsx_num_tiles(width, height)).bytes;
+    return lists_workspace(k < 0 ? 0 : k, dsx_num_tiles(width, height)).bytes;
+}
+
+extern "C" size_t dsx_sort_workspace_bytes(int64_t k, int32_t num_tiles)
+{
+    return sort_workspace(k < 0 ? 0 : k, num_tiles < 0 ? 0 : num_tiles).bytes;
+}
+
+extern "C" size_t dsx_order_bytes(int64_t n)
+{
+    return order_layout(n < 0 ? 0 : n).bytes;
+}
+
+namespace
+{
+// keys_alt | values_alt | Sort32Workspace
+struct SortU32Layout
+{
+    size_t keys_alt, values_alt, sort, bytes;
+};
+SortU32Layout sort_u32_layout(int64_t count, int key_bits)
+{
+    auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    SortU32Layout l;
+    l.keys_alt = 0;
+    l.values_alt = align((size_t)count * 4);
+    l.sort = align(l.values_alt + (size_t)count * 4);
+    l.bytes = l.sort + sort32_workspace(count, key_bits).bytes;
+    return l;
+}
+} // namespace
+
+extern "C" size_t dsx_sort_u32_workspace_bytes(int64_t count, int32_t key_bits)
+{
+    return sort_u32_layout(count < 0 ? 0 : count, key_bits).bytes;
 }
 
 extern "C" int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
                                const float* quats, const float* opacities, const float* shs,
                                const float* cov3d_precomp, const float* colors_precomp, float* splats,
-                               int32_t* radii, float* cov3d, uint32_t* block_sums, void* stream)
+                               int32_t* radii, float* cov3d, uint32_t* block_sums, void* order, size_t order_bytes,
+                               void* stream)
 {
     if(int rc = check_camera(cam))
         return rc;
@@ -155,12 +190,22 @@ extern "C" int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* me
         return DSX_OK;
     if(!means3d || !opacities || !splats || !radii || !cov3d || !block_sums)
         return DSX_ERR_BAD_ARG;
+    uint32_t* depth_keys = nullptr;
+    uint2* rects = nullptr;
+    if(order)
+    {
+        const OrderLayout o = order_layout(n);
+        if(order_bytes < o.bytes)
+            return DSX_ERR_WORKSPACE;
+        depth_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(order) + o.depth_keys);
+        rects = reinterpret_cast<uint2*>(static_cast<char*>(order) + o.rects);
+    }
     if(!cov3d_precomp && (!scales || !quats))
         return DSX_ERR_BAD_ARG;
     if(!colors_precomp && !shs)
         return DSX_ERR_BAD_ARG;
     return launch_project_fwd(*cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp, splats,
-                              radii, cov3d, block_sums, as_stream(stream));
+                              radii, cov3d, block_sums, depth_keys, rects, as_stream(stream));
 }
 
 extern "C" int dsx_scan_u32(int64_t count, uint32_t* data, uint32_t* total, void* stream)
@@ -225,6 +270,81 @@ extern "C" int dsx_tile_ranges(int64_t k, const int64_t* sorted_keys, int32_t nu
     return launch_tile_ranges(k, sorted_keys, num_tiles, ranges, as_stream(stream));
 }
 
+extern "C" int dsx_sort_pairs_u32(int64_t count, int32_t key_bits, uint32_t* keys, uint32_t* values, void* workspace,
+                                  size_t workspace_bytes, void* stream)
+{
+    if(count < 0 || key_bits < 1 || key_bits > 32)
+        return DSX_ERR_BAD_ARG;
+    if(count <= 1)
+        return DSX_OK;
+    if(!keys || !values || !workspace)
+        return DSX_ERR_BAD_ARG;
+    if(count >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
+    const SortU32Layout l = sort_u32_layout(count, key_bits);
+    if(workspace_bytes < l.bytes)
+        return DSX_ERR_WORKSPACE;
+    char* base = static_cast<char*>(workspace);
+    uint32_t *ko, *vo;
+    int rc = launch_sort32(count, key_bits, keys, values, reinterpret_cast<uint32_t*>(base + l.keys_alt),
+                           reinterpret_cast<uint32_t*>(base + l.values_alt), false, true, base + l.sort,
+                           as_stream(stream), &ko, &vo);
+    if(rc)
+        return rc;
+    if(ko != keys)
+    {
+        if(hipMemcpyAsync(keys, ko, (size_t)count * 4, hipMemcpyDeviceToDevice, as_stream(stream)) != hipSuccess ||
+           hipMemcpyAsync(values, vo, (size_t)count * 4, hipMemcpyDeviceToDevice, as_stream(stream)) != hipSuccess)
+            return DSX_ERR_RUNTIME;
+    }
+    return DSX_OK;
+}
+
+extern "C" int dsx_depth_order(int64_t n, void* order, size_t order_bytes, void* stream)
+{
+    if(n < 0)
+        return DSX_ERR_BAD_ARG;
+    if(n == 0)
+        return DSX_OK;
+    if(!order)
+        return DSX_ERR_BAD_ARG;
+    if(order_bytes < order_layout(n).bytes)
+        return DSX_ERR_WORKSPACE;
+    return launch_depth_order(n, order, as_stream(stream));
+}
+
+extern "C" int dsx_order_view(int64_t n, const void* order, const uint32_t** depth_order,
+                              const uint32_t** block_offsets)
+{
+    if(n < 0 || !order)
+        return DSX_ERR_BAD_ARG;
+    const OrderLayout o = order_layout(n);
+    if(depth_order)
+        *depth_order = reinterpret_cast<const uint32_t*>(static_cast<const char*>(order) + o.ids_a);
+    if(block_offsets)
+        *block_offsets = reinterpret_cast<const uint32_t*>(static_cast<const char*>(order) + o.block_sums);
+    return DSX_OK;
+}
+
+extern "C" int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
+                              int32_t* ranges, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if(int rc = check_camera(cam))
+        return rc;
+    if(n < 0 || k < 0 || !ranges)
+        return DSX_ERR_BAD_ARG;
+    if(k >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
+    if(k > 0 && n > 0)
+    {
+        if(!order || !sorted_ids || !workspace)
+            return DSX_ERR_BAD_ARG;
+        if(workspace_bytes < lists_workspace(k, dsx_num_tiles(cam->image_width, cam->image_height)).bytes)
+            return DSX_ERR_WORKSPACE;
+    }
+    return launch_tile_lists(*cam, n, k, order, sorted_ids, ranges, workspace, as_stream(stream));
+}
+
 extern "C" int dsx_blend_fwd(const dsx_camera* cam, const int32_t* ranges, const int32_t* sorted_ids,
                              const float* splats, float* image, float* final_T, int32_t* final_idx, void* stream)
 {
@@ -277,77 +397,50 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
                                    const float* quats, const float* opacities, const float* shs,
                                    const float* cov3d_precomp, const float* colors_precomp, float* splats,
                                    int32_t* radii, float* cov3d, uint32_t* block_sums, uint32_t* k_scratch,
-                                   int64_t* num_keys, void* stream)
+                                   void* order, size_t order_bytes, int64_t* num_keys, void* stream)
 {
-    if(!num_keys || !k_scratch)
+    if(!num_keys || !k_scratch || (n > 0 && !order))
         return DSX_ERR_BAD_ARG;
     *num_keys = 0;
+    hipStream_t s = as_stream(stream);
     int rc = dsx_project_fwd(cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp, splats,
-                             radii, cov3d, block_sums, stream);
+                             radii, cov3d, block_sums, order, order_bytes, stream);
     if(rc || n == 0)
         return rc;
-    rc = launch_scan_u32(dsx_num_blocks(n), block_sums, k_scratch, as_stream(stream));
+    rc = launch_scan_u32(dsx_num_blocks(n), block_sums, k_scratch, s);
     if(rc)
         return rc;
-    uint32_t k_host = 0;
-    if(hipMemcpyAsync(&k_host, k_scratch, sizeof(uint32_t), hipMemcpyDeviceToHost, as_stream(stream)) != hipSuccess)
+    // K travels to the host while the depth order is computed: the wait below is for the copy
+    // only (it overlaps when *num_keys is pinned host memory; with pageable memory the copy is
+    // synchronous and nothing is lost)
+    hipEvent_t copied;
+    if(hipEventCreateWithFlags(&copied, hipEventDisableTiming) != hipSuccess)
         return DSX_ERR_RUNTIME;
-    if(hipStreamSynchronize(as_stream(stream)) != hipSuccess)
+    bool ok = hipMemcpyAsync(num_keys, k_scratch, sizeof(uint32_t), hipMemcpyDeviceToHost, s) == hipSuccess &&
+              hipEventRecord(copied, s) == hipSuccess;
+    if(ok)
+        rc = launch_depth_order(n, order, s);
+    ok = ok && hipEventSynchronize(copied) == hipSuccess;
+    (void)hipEventDestroy(copied);
+    if(!ok)
         return DSX_ERR_RUNTIME;
-    *num_keys = (int64_t)k_host;
-    return k_host >= (1u << 30) ? DSX_ERR_TOO_LARGE : DSX_OK;
+    if(rc)
+        return rc;
+    *num_keys &= 0xffffffffll; // four bytes were copied into the low half (little endian)
+    return *num_keys >= (1ll << 30) ? DSX_ERR_TOO_LARGE : DSX_OK;
 }
 
 extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
-                                  const uint32_t* block_offsets, int32_t* sorted_ids, int32_t* ranges,
-                                  float* image, float* final_T, int32_t* final_idx, void* workspace,
-                                  size_t workspace_bytes, void* stream)
+                                  const void* order, int32_t* sorted_ids, int32_t* ranges, float* image,
+                                  float* final_T, int32_t* final_idx, void* workspace, size_t workspace_bytes,
+                                  void* stream)
 {
-    if(int rc = check_camera(cam))
-        return rc;
-    if(n < 0 || k < 0 || !ranges || !image || !final_T || !final_idx)
+    if(!image || !final_T || !final_idx)
         return DSX_ERR_BAD_ARG;
-    if(k >= (1ll << 30))
-        return DSX_ERR_TOO_LARGE;
-    hipStream_t s = as_stream(stream);
-    const int num_tiles = dsx_num_tiles(cam->image_width, cam->image_height);
-    const int64_t* sorted_keys = nullptr;
-    if(k > 0)
-    {
-        if(!splats || !block_offsets || !sorted_ids || !workspace)
-            return DSX_ERR_BAD_ARG;
-        const ForwardWorkspace fw = forward_workspace(k, num_tiles);
-        if(workspace_bytes < fw.bytes)
-            return DSX_ERR_WORKSPACE;
-        const SortWorkspace sw = sort_workspace(k, num_tiles);
-        char* base = static_cast<char*>(workspace);
-        char* sbase = base + fw.sort;
-        // ping-pong parity: start so that the last pass lands the ids in the caller's buffer
-        int64_t* keys_x = reinterpret_cast<int64_t*>(base + fw.keys);
-        int64_t* keys_y = reinterpret_cast<int64_t*>(sbase + sw.keys_alt);
-        int32_t* vals_final = sorted_ids;
-        int32_t* vals_other = reinterpret_cast<int32_t*>(sbase + sw.values_alt);
-        const bool even = (sw.passes % 2) == 0 || k <= 1;
-        int64_t* keys_a = keys_x;
-        int64_t* keys_b = keys_y;
-        int32_t* vals_a = even ? vals_final : vals_other;
-        int32_t* vals_b = even ? vals_other : vals_final;
-        int rc = launch_emit_keys(*cam, n, k, splats, block_offsets, keys_a, vals_a, s);
-        if(rc)
-            return rc;
-        int64_t* ko;
-        int32_t* vo;
-        rc = launch_sort_pairs(k, num_tiles, keys_a, vals_a, keys_b, vals_b, sbase, s, &ko, &vo);
-        if(rc)
-            return rc;
-        if(vo != sorted_ids)
-            return DSX_ERR_RUNTIME;
-        sorted_keys = ko;
-    }
-    int rc = launch_tile_ranges(k, sorted_keys, num_tiles, ranges, s);
+    int rc = dsx_tile_lists(cam, n, k, order, sorted_ids, ranges, workspace, workspace_bytes, stream);
     if(rc)
         return rc;
-    return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, s);
+    return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream));
 }
 
 extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
@@ -392,7 +485,7 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     const int64_t nb = dsx_num_blocks(n);
 
     auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
-    size_t o_splats = 0, o_radii, o_cov3d, o_bs, o_k, o_ranges, o_T, o_idx, stage1;
+    size_t o_splats = 0, o_radii, o_cov3d, o_bs, o_k, o_ranges, o_T, o_idx, o_order, stage1;
     o_radii = align(o_splats + (size_t)n * 48);
     o_cov3d = align(o_radii + (size_t)n * 4);
     o_bs = align(o_cov3d + (size_t)n * 24);
@@ -400,7 +493,9 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     o_ranges = align(o_k + 4);
     o_T = align(o_ranges + (size_t)(num_tiles + 1) * 4);
     o_idx = align(o_T + (size_t)P * 4);
-    stage1 = align(o_idx + (size_t)P * 4);
+    o_order = align(o_idx + (size_t)P * 4);
+    const size_t order_bytes = order_layout(n).bytes;
+    stage1 = align(o_order + order_bytes);
     char* buf = nullptr;
     if(hipMallocAsync(reinterpret_cast<void**>(&buf), stage1 + 256, s) != hipSuccess)
         return DSX_ERR_RUNTIME;
@@ -408,17 +503,17 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     int rc = dsx_forward_project(&cam, n, means3d, scales, quats, opacities, shs, nullptr, nullptr,
                                  reinterpret_cast<float*>(buf + o_splats), reinterpret_cast<int32_t*>(buf + o_radii),
                                  reinterpret_cast<float*>(buf + o_cov3d), reinterpret_cast<uint32_t*>(buf + o_bs),
-                                 reinterpret_cast<uint32_t*>(buf + o_k), &k, stream);
+                                 reinterpret_cast<uint32_t*>(buf + o_k), buf + o_order, order_bytes, &k, stream);
     char* buf2 = nullptr;
     if(rc == DSX_OK)
     {
-        const size_t ws = forward_workspace(k, num_tiles).bytes;
+        const size_t ws = lists_workspace(k, num_tiles).bytes;
         const size_t o_ids = align(ws);
         if(hipMallocAsync(reinterpret_cast<void**>(&buf2), o_ids + (size_t)k * 4 + 256, s) != hipSuccess)
             rc = DSX_ERR_RUNTIME;
         else
-            rc = dsx_forward_finish(&cam, n, k, reinterpret_cast<float*>(buf + o_splats),
-                                    reinterpret_cast<uint32_t*>(buf + o_bs), reinterpret_cast<int32_t*>(buf2 + o_ids),
+            rc = dsx_forward_finish(&cam, n, k, reinterpret_cast<float*>(buf + o_splats), buf + o_order,
+                                    reinterpret_cast<int32_t*>(buf2 + o_ids),
                                     reinterpret_cast<int32_t*>(buf + o_ranges), image,
                                     reinterpret_cast<float*>(buf + o_T), reinterpret_cast<int32_t*>(buf + o_idx),
                                     buf2, ws, stream);

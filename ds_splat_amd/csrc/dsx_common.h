@@ -104,11 +104,106 @@ struct ForwardWorkspace
 };
 ForwardWorkspace forward_workspace(int64_t k, int num_tiles);
 
+// ---- 32-bit radix sort (depth order of the Gaussians, tile partition of the tile lists) ----
+constexpr int kBits32 = 8;
+constexpr int kBins32 = 1 << kBits32;
+#ifndef DSX_SORT32_THREADS
+#define DSX_SORT32_THREADS 512
+#endif
+#ifndef DSX_SORT32_ITEMS
+#define DSX_SORT32_ITEMS 16
+#endif
+constexpr int kSort32Threads = DSX_SORT32_THREADS;
+constexpr int kSort32Items = DSX_SORT32_ITEMS;
+constexpr int kSort32Tile = kSort32Threads * kSort32Items;
+constexpr int kMaxPasses32 = 4;
+
+// Digits of a key whose low `key_bits` bits are significant: fewest passes with digits of at
+// most 8 bits, bits spread evenly.
+struct Digits32
+{
+    int passes;
+    int shift[kMaxPasses32];
+    uint32_t mask[kMaxPasses32];
+};
+inline Digits32 digits32(int key_bits)
+{
+    Digits32 d;
+    if(key_bits < 1)
+        key_bits = 1;
+    if(key_bits > 32)
+        key_bits = 32;
+    d.passes = (key_bits + kBits32 - 1) / kBits32;
+    const int base = key_bits / d.passes, rem = key_bits % d.passes;
+    int shift = 0;
+    for(int p = 0; p < kMaxPasses32; ++p)
+    {
+        const int bits = p < d.passes ? base + (p < rem ? 1 : 0) : 0;
+        d.shift[p] = shift;
+        d.mask[p] = bits ? (1u << bits) - 1u : 0u;
+        shift += bits;
+    }
+    return d;
+}
+// bits needed for tile slots 0..num_tiles (slot 0 = keys with a negative depth, slot t+1 = tile t)
+inline int slot_bits(int num_tiles)
+{
+    int b = 1;
+    while((1ll << b) < (long long)num_tiles + 1)
+        ++b;
+    return b;
+}
+
+// Workspace of one 32-bit sort of `count` pairs (offsets relative to its base, 256-byte aligned).
+struct Sort32Workspace
+{
+    size_t hist;     // uint32[passes * 256]
+    size_t counters; // uint32[passes + 1]: dynamic tile ids per pass, [passes] = error flag
+    size_t status;   // uint32[passes * tiles * 256]
+    size_t bytes;
+    int passes;
+    int64_t tiles;
+};
+Sort32Workspace sort32_workspace(int64_t count, int key_bits);
+
+// Per-Gaussian buffer that carries the depth order from the projection to the tile lists.
+struct OrderLayout
+{
+    size_t depth_keys; // uint32[n]  depth bits (written by the projection)
+    size_t keys_alt;   // uint32[n]
+    size_t ids_a;      // uint32[n]  the depth order ends here
+    size_t ids_b;      // uint32[n]
+    size_t rects;      // uint2[n]   packed tile rectangle (written by the projection)
+    size_t block_sums; // uint32[blocks + 1] tile counts of 256 consecutive Gaussians IN DEPTH ORDER, scanned
+    size_t sort;       // Sort32Workspace
+    size_t bytes;
+};
+OrderLayout order_layout(int64_t n);
+
+// Workspace of the tile lists for k keys.
+struct ListsWorkspace
+{
+    size_t slots_a; // uint32[k]
+    size_t slots_b; // uint32[k]
+    size_t ids_alt; // int32[k]
+    size_t sort;    // Sort32Workspace
+    size_t bytes;
+    int passes;
+};
+ListsWorkspace lists_workspace(int64_t k, int num_tiles);
+
 // launchers (each returns a dsx_status)
+int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
+                  uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
+                  uint32_t** keys_out, uint32_t** vals_out);
+int launch_depth_order(int64_t n, void* order, hipStream_t stream);
+int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
+                      int32_t* ranges, void* workspace, hipStream_t stream);
 int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, const float* scales,
                        const float* quats, const float* opacities, const float* shs,
                        const float* cov3d_precomp, const float* colors_precomp, float* splats,
-                       int32_t* radii, float* cov3d, uint32_t* block_sums, hipStream_t stream);
+                       int32_t* radii, float* cov3d, uint32_t* block_sums, uint32_t* depth_keys,
+                       uint2* rects, hipStream_t stream);
 int launch_scan_u32(int64_t count, uint32_t* data, uint32_t* total, hipStream_t stream);
 int launch_emit_keys(const dsx_camera& cam, int64_t n, int64_t k, const float* splats,
                      const uint32_t* block_offsets, int64_t* keys, int32_t* values,

@@ -37,6 +37,8 @@ struct ProjectParams
     int32_t* radii;
     float* cov3d;
     uint32_t* block_sums;
+    uint32_t* depth_keys; // optional: depth bits per Gaussian, the key of the depth order
+    uint2* rects;         // optional: packed tile rectangle per Gaussian (zero when it emits nothing)
     float focal_x, focal_y, tanfovx, tanfovy, c_x, c_y, scale_modifier;
     int sh_degree, sh_stride; // active degree; floats per shs row
     int ntx, nty;
@@ -316,6 +318,16 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
 
         // the last Gaussian never emits keys (cpp/rasterizer_torch.cu:99-104)
         count = (i == p.n - 1) ? 0u : (uint32_t)tiles;
+        if(p.depth_keys)
+        {
+            // x = sx | sy << 16, y = width | height << 16 | (depth sign) << 31
+            const uint32_t depth_bits = __float_as_uint(vz);
+            p.depth_keys[i] = depth_bits;
+            p.rects[i] = count ? make_uint2((uint32_t)r.sx | ((uint32_t)r.sy << 16),
+                                            (uint32_t)(r.ex - r.sx) | ((uint32_t)(r.ey - r.sy) << 16) |
+                                                (depth_bits & 0x80000000u))
+                               : make_uint2(0u, 0u);
+        }
     }
 
     const uint32_t ws = wave_sum_u32(count);
@@ -329,7 +341,7 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
 int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, const float* scales,
                        const float* quats, const float* opacities, const float* shs,
                        const float* cov3d_precomp, const float* colors_precomp, float* splats, int32_t* radii,
-                       float* cov3d, uint32_t* block_sums, hipStream_t stream)
+                       float* cov3d, uint32_t* block_sums, uint32_t* depth_keys, uint2* rects, hipStream_t stream)
 {
     if(n == 0)
         return DSX_OK;
@@ -349,6 +361,8 @@ int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, c
     p.radii = radii;
     p.cov3d = cov3d;
     p.block_sums = block_sums;
+    p.depth_keys = depth_keys;
+    p.rects = depth_keys ? rects : nullptr;
     // cpp/rasterizer_torch.cu:144-147
     p.focal_y = cam.image_height / (2 * cam.tanfovy);
     p.focal_x = cam.image_width / (2 * cam.tanfovx);

@@ -1,0 +1,674 @@
+// Per-tile depth-ordered Gaussian lists without a 64-bit sort of all K keys.
+//
+// The order the blend kernels need is (tile, depth bits, Gaussian index): the order a stable
+// sort of the (tile << 32 | depth) keys produces, because keys are emitted by ascending Gaussian
+// index and a Gaussian touches a tile at most once.  The same order falls out of
+//   1. a stable sort of the N Gaussians by their 32 depth bits (N is ~10x smaller than K),
+//   2. emitting (tile slot, Gaussian) pairs in that depth order,
+//   3. a STABLE partition of the K pairs by tile slot alone (2 passes of <= 8 bits).
+// Keys with a negative depth carry tile field -1 in the 64-bit scheme and sort first by their
+// unsigned depth bits; here they take slot 0 and real tiles move up by one, and the unsigned
+// depth order of step 1 keeps their relative order.  HBM traffic: 8 bytes per pair written
+// once and moved twice, instead of 12 bytes moved five times.
+#include "dsx_common.h"
+
+namespace dsx
+{
+
+__device__ __forceinline__ uint32_t wave_incl_scan32(uint32_t v, int lane)
+{
+#pragma unroll
+    for(int o = 1; o < DSX_WAVE; o <<= 1)
+    {
+        const uint32_t t = __shfl_up(v, o, DSX_WAVE);
+        if(lane >= o)
+            v += t;
+    }
+    return v;
+}
+
+// lanes of the wavefront that hold the same (up to 8-bit) digit and are valid; uniform flow only
+__device__ __forceinline__ uint64_t match_digit8(uint32_t d, bool valid)
+{
+    const uint64_t v = __ballot(valid);
+    uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+#pragma unroll
+    for(int b = 0; b < kBits32; ++b)
+    {
+        const uint32_t x = (uint32_t)(((int32_t)(d << (31 - b))) >> 31); // all ones where bit b is set
+        const uint64_t m = __ballot(x != 0);
+        lo &= ~((uint32_t)m ^ x);
+        hi &= ~((uint32_t)(m >> 32) ^ x);
+    }
+    return ((uint64_t)hi << 32) | lo;
+}
+
+__device__ __forceinline__ uint32_t lane_below32(uint32_t v, uint32_t first)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)first, (int)v, 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+}
+
+// ---------------------------------------------------------------------------------------
+// histograms of every digit in one read (run-length merged: neighbouring keys often share a digit)
+// ---------------------------------------------------------------------------------------
+constexpr int kHist32Threads = 256;
+constexpr int kHist32Items = 8;
+
+__global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const uint32_t* __restrict__ keys, int64_t count,
+                                                                const Digits32 plan,
+                                                                uint32_t* __restrict__ global_hist)
+{
+    __shared__ uint32_t hist[kMaxPasses32 * kBins32];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    for(int j = tid; j < plan.passes * kBins32; j += kHist32Threads)
+        hist[j] = 0;
+    __syncthreads();
+    const int64_t chunk = (int64_t)kHist32Threads * kHist32Items;
+    const int64_t chunks = (count + chunk - 1) / chunk;
+    for(int64_t c = blockIdx.x; c < chunks; c += gridDim.x)
+    {
+        uint32_t s[kHist32Items];
+        bool valid[kHist32Items];
+#pragma unroll
+        for(int it = 0; it < kHist32Items; ++it)
+        {
+            const int64_t i = c * chunk + it * kHist32Threads + tid;
+            valid[it] = i < count;
+            s[it] = valid[it] ? __builtin_nontemporal_load(keys + i) : 0u;
+        }
+#pragma unroll
+        for(int it = 0; it < kHist32Items; ++it)
+        {
+            const uint64_t vmask = __ballot(valid[it]); // valid lanes are a prefix of the wavefront
+            const int nvalid = __popcll(vmask);
+            for(int p = 0; p < plan.passes; ++p)
+            {
+                const uint32_t d = (s[it] >> plan.shift[p]) & plan.mask[p];
+                const uint32_t below = lane_below32(d, ~d);
+                const bool head = valid[it] && (lane == 0 || below != d);
+                const uint64_t heads = __ballot(head);
+                if(head)
+                {
+                    const uint64_t above = lane == 63 ? 0ull : (heads >> (lane + 1));
+                    const int run = above ? __ffsll((unsigned long long)above) : nvalid - lane;
+                    atomicAdd(&hist[p * kBins32 + d], (uint32_t)run);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for(int j = tid; j < plan.passes * kBins32; j += kHist32Threads)
+        if(hist[j])
+            atomicAdd(&global_hist[j], hist[j]);
+}
+
+// exclusive scan of each pass's 256 bins (one workgroup per pass)
+__global__ __launch_bounds__(kBins32) void hist32_scan_kernel(uint32_t* global_hist)
+{
+    __shared__ uint32_t wave_tot[kBins32 / DSX_WAVE];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    uint32_t* h = global_hist + blockIdx.x * kBins32;
+    const uint32_t v = h[tid];
+    const uint32_t incl = wave_incl_scan32(v, lane);
+    if(lane == 63)
+        wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t prefix = 0;
+    for(int w = 0; w < wave; ++w)
+        prefix += wave_tot[w];
+    h[tid] = prefix + incl - v;
+}
+
+// ---------------------------------------------------------------------------------------
+// one digit pass (chained scan over tiles, decoupled look-back) for (uint32 key, uint32 value)
+// ---------------------------------------------------------------------------------------
+constexpr uint32_t kFlagAggregate32 = 1u << 30;
+constexpr uint32_t kFlagInclusive32 = 2u << 30;
+constexpr uint32_t kFlagMask32 = 3u << 30;
+constexpr uint32_t kValueMask32 = ~kFlagMask32;
+constexpr int kSpinLimit32 = 1 << 18; // bounded wait: a stuck predecessor ends in an error flag, not a hang
+constexpr int kLookBatch32 = 4;
+constexpr int kSort32Waves = kSort32Threads / DSX_WAVE;
+
+static_assert(kSort32Threads >= kBins32, "one thread per digit");
+static_assert(kSort32Tile <= 65535, "u16 ranks");
+
+// vals_in == nullptr: the values are the input positions (iota).  keys_out == nullptr: the
+// keys are not needed after this pass.
+__global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
+    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ keys_out,
+    uint32_t* __restrict__ vals_out, int64_t count, int shift, uint32_t mask, const uint32_t* __restrict__ hist_excl,
+    uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag)
+{
+    __shared__ uint32_t s_keys[kSort32Tile]; // reused for the values in the second round
+    __shared__ uint16_t s_whist[kSort32Waves][kBins32];
+    __shared__ uint32_t s_digit_start[kBins32];
+    __shared__ uint32_t s_gbase[kBins32];
+    __shared__ uint32_t s_wave_tot[kBins32 / DSX_WAVE];
+    __shared__ uint32_t s_tile;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+
+    if(tid == 0)
+        s_tile = atomicAdd(tile_counter, 1u);
+    for(int j = tid; j < kSort32Waves * kBins32; j += kSort32Threads)
+        (&s_whist[0][0])[j] = 0;
+    __syncthreads();
+    const int64_t tile = s_tile;
+    const int64_t tile_base = tile * kSort32Tile;
+    const int tile_n = (int)min((int64_t)kSort32Tile, count - tile_base);
+
+    // ---- load (striped inside each wavefront: coalesced, order = (item, lane)) -------------
+    uint32_t key[kSort32Items];
+    uint32_t val[kSort32Items];
+    uint32_t pos[kSort32Items];
+#pragma unroll
+    for(int it = 0; it < kSort32Items; ++it)
+    {
+        const int local = wave * (kSort32Items * 64) + it * 64 + lane;
+        key[it] = 0;
+        val[it] = 0;
+        if(local < tile_n)
+        {
+            key[it] = __builtin_nontemporal_load(keys_in + tile_base + local);
+            val[it] = vals_in ? __builtin_nontemporal_load(vals_in + tile_base + local) : (uint32_t)(tile_base + local);
+        }
+    }
+
+    // ---- wave-local stable rank ------------------------------------------------------------
+    uint16_t* wh = s_whist[wave];
+#pragma unroll
+    for(int it = 0; it < kSort32Items; ++it)
+    {
+        const int local = wave * (kSort32Items * 64) + it * 64 + lane;
+        const bool valid = local < tile_n;
+        const uint32_t d = (key[it] >> shift) & mask;
+        const uint64_t m = match_digit8(d, valid);
+        const uint32_t below = (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+        const uint32_t old = wh[d];
+        __builtin_amdgcn_wave_barrier();
+        if(valid && below == 0)
+            wh[d] = (uint16_t)(old + (uint32_t)__popcll(m));
+        __builtin_amdgcn_wave_barrier();
+        pos[it] = old + below;
+    }
+    __syncthreads();
+
+    // ---- per-digit totals of the tile (thread d <-> digit d), wave offsets, digit starts ----
+    const bool digit_thread = tid < kBins32;
+    uint32_t total = 0;
+    uint32_t* my_status = status + tile * kBins32 + (digit_thread ? tid : 0);
+    if(digit_thread)
+    {
+#pragma unroll
+        for(int w = 0; w < kSort32Waves; ++w)
+        {
+            const uint32_t c = s_whist[w][tid];
+            s_whist[w][tid] = (uint16_t)total;
+            total += c;
+        }
+        __hip_atomic_store(my_status, total | (tile == 0 ? kFlagInclusive32 : kFlagAggregate32), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t incl = wave_incl_scan32(total, lane);
+        if(lane == 63)
+            s_wave_tot[wave] = incl;
+        s_gbase[tid] = incl - total; // wave-local exclusive prefix, completed after the barrier
+    }
+    __syncthreads();
+    if(digit_thread)
+    {
+        uint32_t prefix = 0;
+        for(int w = 0; w < wave; ++w)
+            prefix += s_wave_tot[w];
+        s_digit_start[tid] = prefix + s_gbase[tid];
+    }
+    __syncthreads();
+
+    // ---- keys into LDS in tile-sorted order ----------------------------------------------
+#pragma unroll
+    for(int it = 0; it < kSort32Items; ++it)
+    {
+        const int local = wave * (kSort32Items * 64) + it * 64 + lane;
+        if(local < tile_n)
+        {
+            const uint32_t d = (key[it] >> shift) & mask;
+            pos[it] += s_digit_start[d] + s_whist[wave][d];
+            s_keys[pos[it]] = key[it];
+        }
+    }
+
+    // ---- chained scan over earlier tiles (decoupled look-back), one thread per digit -------
+    if(digit_thread)
+    {
+        uint32_t excl = 0;
+        if(tile > 0)
+        {
+            int64_t t = tile - 1; // next predecessor to account for
+            int spins = 0;
+            bool done = false;
+            while(!done)
+            {
+                uint32_t v[kLookBatch32];
+#pragma unroll
+                for(int b = 0; b < kLookBatch32; ++b)
+                {
+                    // rows below tile 0 are read as tile 0, whose status is inclusive from the start
+                    const int64_t row = t - b > 0 ? t - b : 0;
+                    v[b] = __hip_atomic_load(status + row * kBins32 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for(int b = 0; b < kLookBatch32; ++b)
+                {
+                    if(done)
+                        break;
+                    if((v[b] & kFlagMask32) == 0)
+                    {
+                        if(++spins > kSpinLimit32)
+                        {
+                            *error_flag = 1u;
+                            done = true;
+                        }
+                        else
+                            __builtin_amdgcn_s_sleep(1);
+                        break;
+                    }
+                    excl += v[b] & kValueMask32;
+                    --t;
+                    if(v[b] & kFlagInclusive32)
+                        done = true;
+                }
+            }
+            __hip_atomic_store(my_status, ((excl + total) & kValueMask32) | kFlagInclusive32, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        s_gbase[tid] = hist_excl[tid] + excl - s_digit_start[tid];
+    }
+    __syncthreads();
+
+    // ---- scatter keys: consecutive threads -> consecutive addresses inside a digit's run ----
+    uint32_t out[kSort32Items];
+#pragma unroll
+    for(int it = 0; it < kSort32Items; ++it)
+    {
+        const int j = it * kSort32Threads + tid;
+        out[it] = 0;
+        if(j < tile_n)
+        {
+            const uint32_t kk = s_keys[j];
+            out[it] = s_gbase[(kk >> shift) & mask] + (uint32_t)j;
+            if(keys_out)
+                keys_out[out[it]] = kk;
+        }
+    }
+    __syncthreads();
+
+    // ---- values through the same buffer, same positions ------------------------------------
+#pragma unroll
+    for(int it = 0; it < kSort32Items; ++it)
+    {
+        const int local = wave * (kSort32Items * 64) + it * 64 + lane;
+        if(local < tile_n)
+            s_keys[pos[it]] = val[it];
+    }
+    __syncthreads();
+#pragma unroll
+    for(int it = 0; it < kSort32Items; ++it)
+    {
+        const int j = it * kSort32Threads + tid;
+        if(j < tile_n)
+            vals_out[out[it]] = s_keys[j];
+    }
+}
+
+Sort32Workspace sort32_workspace(int64_t count, int key_bits)
+{
+    auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    Sort32Workspace w;
+    w.passes = digits32(key_bits).passes;
+    w.tiles = (count + kSort32Tile - 1) / kSort32Tile;
+    size_t off = 0;
+    w.hist = off;
+    off = align(off + (size_t)w.passes * kBins32 * 4);
+    w.counters = off;
+    off = align(off + (size_t)(w.passes + 1) * 4);
+    w.status = off;
+    off = align(off + (size_t)w.passes * (size_t)w.tiles * kBins32 * 4);
+    w.bytes = off;
+    return w;
+}
+
+// Stable ascending sort of `count` (key, value) pairs by the low key_bits bits of the key.
+// Ping-pong between (keys_a, vals_a) and (keys_b, vals_b); *keys_out / *vals_out say where the
+// result is (keys only when keep_keys).
+int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
+                  uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
+                  uint32_t** keys_out, uint32_t** vals_out)
+{
+    *keys_out = keys_a;
+    *vals_out = vals_a;
+    if(count <= 0)
+        return DSX_OK;
+    if(count >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
+    const Sort32Workspace w = sort32_workspace(count, key_bits);
+    const Digits32 plan = digits32(key_bits);
+    char* base = static_cast<char*>(sort_ws);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(base + w.hist);
+    uint32_t* counters = reinterpret_cast<uint32_t*>(base + w.counters);
+    uint32_t* status = reinterpret_cast<uint32_t*>(base + w.status);
+    int rc = launch_fill_u32(hist, (int64_t)(w.bytes / 4), 0u, stream);
+    if(rc)
+        return rc;
+    const int64_t chunks = (count + kHist32Threads * kHist32Items - 1) / (kHist32Threads * kHist32Items);
+    {
+        DSX_TIMED("hist32_kernel", stream);
+        hipLaunchKernelGGL(hist32_kernel, dim3((unsigned)min((int64_t)2048, chunks)), dim3(kHist32Threads), 0, stream,
+                           keys_a, count, plan, hist);
+    }
+    DSX_LAUNCH_CHECK();
+    {
+        DSX_TIMED("hist32_scan_kernel", stream);
+        hipLaunchKernelGGL(hist32_scan_kernel, dim3(w.passes), dim3(kBins32), 0, stream, hist);
+    }
+    DSX_LAUNCH_CHECK();
+    uint32_t* kin = keys_a;
+    uint32_t* vin = vals_a;
+    uint32_t* kout = keys_b;
+    uint32_t* vout = vals_b;
+    for(int p = 0; p < w.passes; ++p)
+    {
+        const bool last = p == w.passes - 1;
+        {
+            DSX_TIMED("onesweep32_kernel", stream);
+            hipLaunchKernelGGL(onesweep32_kernel, dim3((unsigned)w.tiles), dim3(kSort32Threads), 0, stream, kin,
+                               (p == 0 && iota_values) ? nullptr : vin, (last && !keep_keys) ? nullptr : kout, vout,
+                               count, plan.shift[p], plan.mask[p], hist + p * kBins32,
+                               status + (size_t)p * w.tiles * kBins32, counters + p, counters + w.passes);
+        }
+        DSX_LAUNCH_CHECK();
+        uint32_t* tk = kin;
+        kin = kout;
+        kout = tk;
+        uint32_t* tv = vin;
+        vin = vout;
+        vout = tv;
+    }
+    *keys_out = kin;
+    *vals_out = vin;
+    return DSX_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// depth order of the Gaussians and the scanned tile counts in that order
+// ---------------------------------------------------------------------------------------
+
+OrderLayout order_layout(int64_t n)
+{
+    auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    OrderLayout o;
+    size_t off = 0;
+    o.depth_keys = off;
+    off = align(off + (size_t)n * 4);
+    o.keys_alt = off;
+    off = align(off + (size_t)n * 4);
+    o.ids_a = off;
+    off = align(off + (size_t)n * 4);
+    o.ids_b = off;
+    off = align(off + (size_t)n * 4);
+    o.rects = off;
+    off = align(off + (size_t)n * 8);
+    o.block_sums = off;
+    off = align(off + (size_t)((n + kProjBlock - 1) / kProjBlock + 1) * 4);
+    o.sort = off;
+    off += sort32_workspace(n, 32).bytes;
+    o.bytes = align(off);
+    return o;
+}
+
+__device__ __forceinline__ uint32_t rect_count(uint2 r)
+{
+    return (r.y & 0xffffu) * ((r.y >> 16) & 0x7fffu);
+}
+
+// tile count of each run of 256 Gaussians taken in depth order
+__global__ __launch_bounds__(kProjBlock) void ordered_block_sums_kernel(const uint32_t* __restrict__ order,
+                                                                       const uint2* __restrict__ rects, int64_t n,
+                                                                       uint32_t* __restrict__ block_sums)
+{
+    __shared__ uint32_t wave_sums[kProjBlock / DSX_WAVE];
+    const int tid = threadIdx.x;
+    const int64_t p = (int64_t)blockIdx.x * kProjBlock + tid;
+    uint32_t count = 0;
+    if(p < n)
+        count = rect_count(rects[order[p]]);
+    const uint32_t ws = wave_sum_u32(count);
+    if((tid & 63) == 0)
+        wave_sums[tid >> 6] = ws;
+    __syncthreads();
+    if(tid == 0)
+        block_sums[blockIdx.x] = wave_sums[0] + wave_sums[1] + wave_sums[2] + wave_sums[3];
+}
+
+// order: the buffer of order_layout(n) whose depth_keys and rects the projection has written
+int launch_depth_order(int64_t n, void* order, hipStream_t stream)
+{
+    if(n <= 0)
+        return DSX_OK;
+    const OrderLayout o = order_layout(n);
+    char* base = static_cast<char*>(order);
+    uint32_t* keys_a = reinterpret_cast<uint32_t*>(base + o.depth_keys);
+    uint32_t* keys_b = reinterpret_cast<uint32_t*>(base + o.keys_alt);
+    uint32_t* ids_a = reinterpret_cast<uint32_t*>(base + o.ids_a);
+    uint32_t* ids_b = reinterpret_cast<uint32_t*>(base + o.ids_b);
+    uint32_t* block_sums = reinterpret_cast<uint32_t*>(base + o.block_sums);
+    uint32_t *ko, *vo;
+    // 32 key bits = 4 passes: the values (iota in pass 0) go b, a, b, a and end in ids_a
+    int rc = launch_sort32(n, 32, keys_a, ids_a, keys_b, ids_b, true, false, base + o.sort, stream, &ko, &vo);
+    if(rc)
+        return rc;
+    if(vo != ids_a)
+        return DSX_ERR_RUNTIME;
+    const uint32_t* perm = vo;
+    const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
+    {
+        DSX_TIMED("ordered_block_sums_kernel", stream);
+        hipLaunchKernelGGL(ordered_block_sums_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, perm,
+                           reinterpret_cast<const uint2*>(base + o.rects), n, block_sums);
+    }
+    DSX_LAUNCH_CHECK();
+    return launch_scan_u32(blocks, block_sums, block_sums + blocks, stream);
+}
+
+// ---------------------------------------------------------------------------------------
+// emission in depth order: one workgroup per 256 Gaussians of the depth order, one thread per
+// OUTPUT pair, so stores are contiguous however uneven the per-Gaussian tile counts are
+// ---------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t* __restrict__ order,
+                                                                  const uint2* __restrict__ rects,
+                                                                  const uint32_t* __restrict__ block_offsets,
+                                                                  int64_t n, int64_t k, int ntx,
+                                                                  uint32_t* __restrict__ slots,
+                                                                  int32_t* __restrict__ ids)
+{
+    __shared__ uint32_t s_off[kProjBlock + 1];
+    __shared__ uint32_t s_origin[kProjBlock]; // slot of the rectangle's first tile (0 for negative depths)
+    __shared__ uint32_t s_w[kProjBlock];      // width; 0 marks a negative depth (every pair goes to slot 0)
+    __shared__ float s_winv[kProjBlock];
+    __shared__ uint32_t s_id[kProjBlock];
+    __shared__ uint32_t wave_tot[kProjBlock / DSX_WAVE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int64_t p = (int64_t)blockIdx.x * kProjBlock + tid;
+
+    uint32_t count = 0;
+    if(p < n)
+    {
+        const uint32_t g = order[p];
+        const uint2 r = rects[g];
+        count = rect_count(r);
+        const uint32_t w = r.y & 0xffffu;
+        const bool negative = (r.y >> 31) != 0;
+        s_origin[tid] = negative ? 0u : (r.x >> 16) * (uint32_t)ntx + (r.x & 0xffffu) + 1u;
+        s_w[tid] = negative ? 0u : w;
+        s_winv[tid] = 1.0f / (float)(w ? w : 1u);
+        s_id[tid] = g;
+    }
+    const uint32_t incl = wave_incl_scan32(count, lane);
+    if(lane == 63)
+        wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t prefix = 0;
+    for(int w = 0; w < wave; ++w)
+        prefix += wave_tot[w];
+    s_off[tid] = prefix + incl - count;
+    if(tid == kProjBlock - 1)
+        s_off[kProjBlock] = prefix + incl;
+    __syncthreads();
+
+    const uint32_t total = s_off[kProjBlock];
+    const int64_t base = block_offsets[blockIdx.x];
+    for(uint32_t j = tid; j < total; j += kProjBlock)
+    {
+        // largest g with s_off[g] <= j
+        int lo = 0, hi = kProjBlock;
+        while(hi - lo > 1)
+        {
+            const int mid = (lo + hi) >> 1;
+            if(s_off[mid] <= j)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        const uint32_t r = j - s_off[lo];
+        const uint32_t w = s_w[lo];
+        uint32_t slot = 0;
+        if(w)
+        {
+            // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
+            uint32_t ry = (uint32_t)((float)r * s_winv[lo]);
+            if(ry * w > r)
+                --ry;
+            else if((ry + 1) * w <= r)
+                ++ry;
+            const uint32_t rx = r - ry * w;
+            slot = s_origin[lo] + ry * (uint32_t)ntx + rx;
+        }
+        const int64_t out = base + j;
+        if(out < k)
+        {
+            slots[out] = slot;
+            ids[out] = (int32_t)s_id[lo];
+        }
+    }
+}
+
+// ranges[j] = number of pairs whose tile is below j, by binary search in the sorted slots.
+// Two rules of the reference are kept (cpp/rasterizer_kernels.cu:313-322,
+// cpp/rasterizer_torch.cu:31-39): the boundary after the LAST run is never recorded, so tiles
+// above the highest occupied tile inherit the START of that run, and ranges[num_tiles] = K.
+// Slot 0 (negative depths) is skipped by ranges[0].
+__global__ __launch_bounds__(256) void ranges_slots_kernel(const uint32_t* __restrict__ slots, int64_t k,
+                                                           int num_tiles, int32_t* __restrict__ ranges)
+{
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if(j > num_tiles)
+        return;
+    if(j == num_tiles || k == 0)
+    {
+        ranges[j] = j == num_tiles ? (int32_t)k : 0;
+        return;
+    }
+    const uint32_t last_slot = slots[k - 1];
+    const uint32_t target = (uint32_t)(j + 1) < last_slot ? (uint32_t)(j + 1) : last_slot;
+    int64_t lo = 0, hi = k; // first index with slots[i] >= target
+    while(lo < hi)
+    {
+        const int64_t mid = (lo + hi) >> 1;
+        if(slots[mid] < target)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    ranges[j] = (int32_t)lo;
+}
+
+ListsWorkspace lists_workspace(int64_t k, int num_tiles)
+{
+    auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    ListsWorkspace w;
+    w.passes = digits32(slot_bits(num_tiles)).passes;
+    size_t off = 0;
+    w.slots_a = off;
+    off = align(off + (size_t)k * 4);
+    w.slots_b = off;
+    off = align(off + (size_t)k * 4);
+    w.ids_alt = off;
+    off = align(off + (size_t)k * 4);
+    w.sort = off;
+    off += sort32_workspace(k, slot_bits(num_tiles)).bytes;
+    w.bytes = align(off);
+    return w;
+}
+
+// order: buffer of order_layout(n) after launch_depth_order.  Writes sorted_ids[k], ranges[T+1].
+int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
+                      int32_t* ranges, void* workspace, hipStream_t stream)
+{
+    const int num_tiles = tiles_x(cam.image_width) * tiles_y(cam.image_height);
+    const uint32_t* sorted_slots = nullptr;
+    if(k > 0 && n > 0)
+    {
+        if(k >= (1ll << 30))
+            return DSX_ERR_TOO_LARGE;
+        const OrderLayout o = order_layout(n);
+        const ListsWorkspace w = lists_workspace(k, num_tiles);
+        const char* obase = static_cast<const char*>(order);
+        char* base = static_cast<char*>(workspace);
+        uint32_t* slots_a = reinterpret_cast<uint32_t*>(base + w.slots_a);
+        uint32_t* slots_b = reinterpret_cast<uint32_t*>(base + w.slots_b);
+        uint32_t* ids_final = reinterpret_cast<uint32_t*>(sorted_ids);
+        uint32_t* ids_other = reinterpret_cast<uint32_t*>(base + w.ids_alt);
+        // ping-pong parity: start so that the last pass lands the ids in the caller's buffer
+        const bool even = (w.passes % 2) == 0;
+        uint32_t* vals_a = even ? ids_final : ids_other;
+        uint32_t* vals_b = even ? ids_other : ids_final;
+        const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
+        {
+            DSX_TIMED("emit_ordered_kernel", stream);
+            hipLaunchKernelGGL(emit_ordered_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
+                               reinterpret_cast<const uint32_t*>(obase + o.ids_a),
+                               reinterpret_cast<const uint2*>(obase + o.rects),
+                               reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k,
+                               tiles_x(cam.image_width), slots_a, reinterpret_cast<int32_t*>(vals_a));
+        }
+        DSX_LAUNCH_CHECK();
+        uint32_t *ko, *vo;
+        int rc = launch_sort32(k, slot_bits(num_tiles), slots_a, vals_a, slots_b, vals_b, false, true, base + w.sort,
+                               stream, &ko, &vo);
+        if(rc)
+            return rc;
+        if(vo != ids_final)
+            return DSX_ERR_RUNTIME;
+        sorted_slots = ko;
+    }
+    else
+        k = 0;
+    const int count = num_tiles + 1;
+    {
+        DSX_TIMED("ranges_slots_kernel", stream);
+        hipLaunchKernelGGL(ranges_slots_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, sorted_slots, k,
+                           num_tiles, ranges);
+    }
+    DSX_LAUNCH_CHECK();
+    return DSX_OK;
+}
+
+} // namespace dsx

@@ -5,6 +5,7 @@ launches on torch's current stream of the tensors' device and allocates its outp
 torch (the native library allocates nothing).
 """
 import ctypes as C
+import threading
 
 import torch
 
@@ -67,7 +68,8 @@ def camera_from_scene(sc, device, bg=None, sh_degree=None, scale_modifier=None):
                       sc["sh_degree"] if sh_degree is None else sh_degree, 3, sc["campos"].to(device))
 
 
-def project_fwd(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, colors_precomp=None):
+def project_fwd(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, colors_precomp=None, order=None):
+    """order: optional uint8 buffer of new_order(n) that also receives depth bits and tile rectangles."""
     lib = N.load()
     n = means3d.shape[0]
     dev = means3d.device
@@ -77,8 +79,49 @@ def project_fwd(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None,
     block_sums = torch.empty((int(lib.dsx_num_blocks(n)),), dtype=torch.int32, device=dev)
     N.check(lib.dsx_project_fwd(cam.ref, n, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(opacities), _ptr(shs),
                                 _ptr(cov3d_precomp), _ptr(colors_precomp), _ptr(splats), _ptr(radii), _ptr(cov3d),
-                                _ptr(block_sums), _stream()))
+                                _ptr(block_sums), _ptr(order), 0 if order is None else order.numel(), _stream()))
     return splats, radii, cov3d, block_sums
+
+
+def new_order(n, device):
+    """The per-Gaussian buffer that carries the depth order from the projection to the tile lists."""
+    return torch.empty((max(int(N.load().dsx_order_bytes(n)), 1),), dtype=torch.uint8, device=device)
+
+
+def depth_order(n, order):
+    """Sorts the Gaussians of a projected `order` buffer by depth bits (stable).  Returns views
+    (depth order int32[n], scanned tile counts of its 256-Gaussian blocks int32[blocks + 1])."""
+    lib = N.load()
+    N.check(lib.dsx_depth_order(n, _ptr(order), order.numel(), _stream()))
+    p_order, p_off = C.c_void_p(), C.c_void_p()
+    N.check(lib.dsx_order_view(n, _ptr(order), C.byref(p_order), C.byref(p_off)))
+    base = order.data_ptr()
+    as_i32 = order.view(torch.int32)
+    o0 = (p_order.value - base) // 4
+    o1 = (p_off.value - base) // 4
+    return as_i32[o0:o0 + n], as_i32[o1:o1 + int(lib.dsx_num_blocks(n)) + 1]
+
+
+def tile_lists(cam, n, k, order):
+    """(sorted_ids[k], ranges[T+1]) from a depth-ordered `order` buffer."""
+    lib = N.load()
+    dev = order.device
+    sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
+    ranges = torch.empty((cam.num_tiles + 1,), dtype=torch.int32, device=dev)
+    nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height))
+    ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
+    N.check(lib.dsx_tile_lists(cam.ref, n, k, _ptr(order), _ptr(sorted_ids), _ptr(ranges), _ptr(ws), nbytes, _stream()))
+    return sorted_ids, ranges
+
+
+def sort_pairs_u32(keys, values, key_bits=32):
+    """Stable ascending sort of (uint32 key, uint32 value) pairs held in int32 tensors, in place."""
+    lib = N.load()
+    count = keys.numel()
+    nbytes = int(lib.dsx_sort_u32_workspace_bytes(count, key_bits))
+    ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=keys.device)
+    N.check(lib.dsx_sort_pairs_u32(count, key_bits, _ptr(keys), _ptr(values), _ptr(ws), nbytes, _stream()))
+    return keys, values
 
 
 def scan_u32(data):
@@ -101,7 +144,7 @@ def sort_pairs(keys, values, num_tiles, width=None, height=None):
     """Sorts in place."""
     lib = N.load()
     k = keys.numel()
-    nbytes = int(lib.dsx_workspace_bytes(0, k, 16 * max(num_tiles, 1), 16))
+    nbytes = int(lib.dsx_sort_workspace_bytes(k, num_tiles))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=keys.device)
     N.check(lib.dsx_sort_pairs(k, num_tiles, _ptr(keys), _ptr(values), _ptr(ws), nbytes, _stream()))
     return keys, values
@@ -150,6 +193,18 @@ def gaussian_bwd(cam, num_bases, means3d, scales, quats, splats, cov3d, radii, g
     return o
 
 
+_pinned = threading.local()
+
+
+def _pinned_i64():
+    """One pinned int64 per host thread: the landing place of the key count."""
+    t = getattr(_pinned, "slot", None)
+    if t is None:
+        t = torch.zeros((1,), dtype=torch.int64, pin_memory=True)
+        _pinned.slot = t
+    return t
+
+
 class ForwardState:
     """What the forward keeps for the backward (the reference saves the analogous tensors
     on the autograd context, ds_splat/rasterizer.py:47-64)."""
@@ -167,12 +222,14 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     st.cov3d = torch.empty((n, 6), dtype=torch.float32, device=dev)
     block_sums = torch.empty((int(lib.dsx_num_blocks(n)) + 1,), dtype=torch.int32, device=dev)
     k_scratch = block_sums[-1:]
-    k = C.c_int64(0)
+    order = new_order(n, dev)
+    k_host = _pinned_i64()
     stream = _stream()
     N.check(lib.dsx_forward_project(cam.ref, n, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(opacities), _ptr(shs),
                                     _ptr(cov3d_precomp), _ptr(colors_precomp), _ptr(st.splats), _ptr(st.radii),
-                                    _ptr(st.cov3d), _ptr(block_sums), _ptr(k_scratch), C.byref(k), stream))
-    k = int(k.value)
+                                    _ptr(st.cov3d), _ptr(block_sums), _ptr(k_scratch), _ptr(order), order.numel(),
+                                    _ptr(k_host), stream))
+    k = int(k_host.item())
     st.num_keys = k
     st.sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
     st.ranges = torch.empty((cam.num_tiles + 1,), dtype=torch.int32, device=dev)
@@ -181,7 +238,7 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     st.final_idx = torch.empty((cam.height, cam.width), dtype=torch.int32, device=dev)
     nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
-    N.check(lib.dsx_forward_finish(cam.ref, n, k, _ptr(st.splats), _ptr(block_sums), _ptr(st.sorted_ids),
+    N.check(lib.dsx_forward_finish(cam.ref, n, k, _ptr(st.splats), _ptr(order), _ptr(st.sorted_ids),
                                    _ptr(st.ranges), _ptr(image), _ptr(st.final_T), _ptr(st.final_idx), _ptr(ws),
                                    nbytes, stream))
     return image, st

@@ -77,8 +77,14 @@ int64_t dsx_num_blocks(int64_t n);
 /* tiles of an image, and radix passes the sort runs for that many tiles */
 int32_t dsx_num_tiles(int32_t width, int32_t height);
 int32_t dsx_sort_passes(int32_t num_tiles);
-/* bytes of `workspace` dsx_forward_finish / dsx_sort_pairs need for k keys */
+/* bytes of `workspace` dsx_forward_finish / dsx_tile_lists need for k keys */
 size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height);
+/* bytes of `workspace` dsx_sort_pairs needs for k keys, and dsx_sort_pairs_u32 for count pairs */
+size_t dsx_sort_workspace_bytes(int64_t k, int32_t num_tiles);
+size_t dsx_sort_u32_workspace_bytes(int64_t count, int32_t key_bits);
+/* bytes of the per-Gaussian `order` buffer that carries the depth order from the projection
+ * (dsx_project_fwd / dsx_forward_project) to the tile lists (dsx_tile_lists / dsx_forward_finish) */
+size_t dsx_order_bytes(int64_t n);
 
 /* ------------------------------------------------------------------------------------ */
 /* Per-stage entry points (each one individually parity-tested and timed)                */
@@ -89,11 +95,13 @@ size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height);
  * and block_sums[dsx_num_blocks(n)] (tile count of each 256-Gaussian block; the last
  * Gaussian counts as zero, cpp/rasterizer_torch.cu:99-104).  shs may be NULL iff
  * colors_precomp is given; scales/quats may be NULL iff cov3d_precomp is given (then cov3d
- * receives a copy). */
+ * receives a copy).  order (may be NULL): buffer of dsx_order_bytes(n) that also receives each
+ * Gaussian's depth bits and packed tile rectangle, the input of dsx_depth_order. */
 int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
                     const float* quats, const float* opacities, const float* shs,
                     const float* cov3d_precomp, const float* colors_precomp, float* splats,
-                    int32_t* radii, float* cov3d, uint32_t* block_sums, void* stream);
+                    int32_t* radii, float* cov3d, uint32_t* block_sums, void* order,
+                    size_t order_bytes, void* stream);
 
 /* Exclusive prefix of `count` uint32 values in place, total written to *total (device).
  * Replaces the in-block Hillis-Steele scan of cpp/rasterizer_kernels.cu:131-142 together
@@ -109,7 +117,7 @@ int dsx_emit_keys(const dsx_camera* cam, int64_t n, int64_t k, const float* spla
 /* Stage 2b — replaces thrust::sort_by_key, cpp/rasterizer_torch.cu:70-76: stable ascending
  * sort of (int64 key, int32 value) pairs where every key is (tile << 32 | depth bits) with
  * tile in [0, num_tiles) or a negative key (tile field all ones).  keys/values are sorted
- * in place; workspace needs dsx_workspace_bytes(0, k, ...) bytes. */
+ * in place; workspace needs dsx_sort_workspace_bytes(k, num_tiles) bytes. */
 int dsx_sort_pairs(int64_t k, int32_t num_tiles, int64_t* keys, int32_t* values, void* workspace,
                    size_t workspace_bytes, void* stream);
 
@@ -118,6 +126,29 @@ int dsx_sort_pairs(int64_t k, int32_t num_tiles, int64_t* keys, int32_t* values,
  * ranges has num_tiles+1 entries. */
 int dsx_tile_ranges(int64_t k, const int64_t* sorted_keys, int32_t num_tiles, int32_t* ranges,
                     void* stream);
+
+/* Stages 2+3, fast route — the same sorted_ids[k] and ranges[T+1] as dsx_emit_keys +
+ * dsx_sort_pairs + dsx_tile_ranges (i.e. as calculate_keys_and_indices_kernel, thrust::sort_by_key
+ * and identify_tile_ranges, cpp/rasterizer_torch.cu:70-104) without sorting K 64-bit keys: the
+ * order (tile, depth bits, Gaussian index) is produced by (1) a stable sort of the n Gaussians by
+ * their 32 depth bits, (2) emission of (tile slot, Gaussian) pairs in that order, (3) a stable
+ * partition of the k pairs by tile slot.
+ *
+ * dsx_sort_pairs_u32: stable ascending sort of (uint32 key, uint32 value) pairs by the low
+ * key_bits bits of the key, in place (the building block of both (1) and (3)).
+ * dsx_depth_order: step (1) on an `order` buffer the projection has filled; it also leaves the
+ * scanned tile counts of the depth-ordered 256-Gaussian blocks in the buffer.
+ * dsx_order_view: device pointers into the buffer (depth order uint32[n], block offsets
+ * uint32[dsx_num_blocks(n)+1] whose last entry is K), for inspection.
+ * dsx_tile_lists: steps (2) and (3) and the ranges. */
+int dsx_sort_pairs_u32(int64_t count, int32_t key_bits, uint32_t* keys, uint32_t* values,
+                       void* workspace, size_t workspace_bytes, void* stream);
+int dsx_depth_order(int64_t n, void* order, size_t order_bytes, void* stream);
+int dsx_order_view(int64_t n, const void* order, const uint32_t** depth_order,
+                   const uint32_t** block_offsets);
+int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const void* order,
+                   int32_t* sorted_ids, int32_t* ranges, void* workspace, size_t workspace_bytes,
+                   void* stream);
 
 /* Stage 4 — replaces rasterizer_cuda_forward + render_image_kernel,
  * cpp/rasterizer_torch.cu:44-68, cpp/rasterizer_kernels.cu:341-431.
@@ -151,20 +182,23 @@ int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const 
 /* ------------------------------------------------------------------------------------ */
 
 /* First half of rasterizer_forward_deepsense (cpp/rasterizer_torch.cu:170-208): projection,
- * block scan and the read-back of K (the one host synchronisation of the forward, in place of
- * the reference's two at cpp/rasterizer_torch.cu:103-104).  block_sums is scanned in place.
- * k_scratch: device uint32[1]; *num_keys (host) receives K. */
+ * block scan, the read-back of K (the one host wait of the forward, in place of the reference's
+ * two device drains at cpp/rasterizer_torch.cu:103-104) and, overlapping that read-back, the
+ * depth order.  block_sums is scanned in place.  k_scratch: device uint32[1].  order: device
+ * buffer of dsx_order_bytes(n).  *num_keys (host; pinned memory lets the copy overlap)
+ * receives K. */
 int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
                         const float* scales, const float* quats, const float* opacities,
                         const float* shs, const float* cov3d_precomp, const float* colors_precomp,
                         float* splats, int32_t* radii, float* cov3d, uint32_t* block_sums,
-                        uint32_t* k_scratch, int64_t* num_keys /* host */, void* stream);
+                        uint32_t* k_scratch, void* order, size_t order_bytes,
+                        int64_t* num_keys /* host */, void* stream);
 
-/* Second half: key emission, sort, tile ranges, blend.  sorted_ids[k] and ranges[T+1] are
+/* Second half: tile lists (dsx_tile_lists) and blend.  sorted_ids[k] and ranges[T+1] are
  * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H). */
 int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
-                       const uint32_t* block_offsets, int32_t* sorted_ids, int32_t* ranges,
-                       float* image, float* final_T, int32_t* final_idx, void* workspace,
+                       const void* order, int32_t* sorted_ids, int32_t* ranges, float* image,
+                       float* final_T, int32_t* final_idx, void* workspace,
                        size_t workspace_bytes, void* stream);
 
 /* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316. grads is scratch [n*12]. */

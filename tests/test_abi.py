@@ -36,7 +36,12 @@ def test_host_helpers():
     # 32 depth bits + bits for tile ids 0..T (slot 0 = negative keys), at most 9 bits a pass
     assert lib.dsx_sort_passes(8160) == 5 and lib.dsx_sort_passes(255) == 5 and lib.dsx_sort_passes(32400) == 6
     assert lib.dsx_workspace_bytes(0, 0, 64, 64) >= 0
-    assert lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080) > (1 << 20) * 24
+    # tile lists: two uint32 slot buffers and one id buffer; 64-bit sort: key and value copies
+    assert (1 << 20) * 12 < lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080) < (1 << 20) * 14
+    assert lib.dsx_sort_workspace_bytes(1 << 20, 8160) > (1 << 20) * 12
+    assert lib.dsx_sort_u32_workspace_bytes(1 << 20, 32) > (1 << 20) * 8
+    # order buffer: 4 uint32 arrays and one uint2 array per Gaussian
+    assert lib.dsx_order_bytes(1 << 20) > (1 << 20) * 24
     assert b"workspace" in lib.dsx_error_string(-5)
     assert lib.dsx_error_string(0) == b"ok"
 
@@ -48,7 +53,11 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.dsx_sort_pairs(-5, 10, None, None, None, 0, None) == -1
     assert lib.dsx_sort_pairs(1 << 31, 10, 1, 1, 1, 0, None) == -4
     assert lib.dsx_tile_ranges(10, None, 4, None, None) == -1
-    assert lib.dsx_project_fwd(None, 10, *([None] * 12)) == -1
+    assert lib.dsx_project_fwd(None, 10, *([None] * 12), 0, None) == -1
+    assert lib.dsx_sort_pairs_u32(10, 33, 1, 1, 1, 0, None) == -1
+    assert lib.dsx_sort_pairs_u32(10, 32, 1, 1, 1, 0, None) == -5
+    assert lib.dsx_depth_order(10, None, 0, None) == -1
+    assert lib.dsx_depth_order(10, 1, 16, None) == -5
 
 
 def test_python_api_surface():

@@ -166,8 +166,9 @@ def test_full_size_properties_cfg2():
     n = sc["n"]
     cam = stages.camera_from_scene(sc, DEV)
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    order = stages.new_order(n, DEV)
     splats, radii, cov3d, block_sums = stages.project_fwd(cam, t["means_3d"], t["scales"], t["rotations"],
-                                                          t["opacities"], t["shs"])
+                                                          t["opacities"], t["shs"], order=order)
     tiles = splats[:, 11].view(torch.int32).to(torch.int64)
     tiles_eff = tiles.clone()
     tiles_eff[-1] = 0
@@ -190,6 +191,15 @@ def test_full_size_properties_cfg2():
     assert torch.equal(keys & 0xFFFFFFFF, depth_bits[vals.to(torch.int64)])                # pairs stay together
     ranges = stages.tile_ranges(keys, cam.num_tiles)
     assert (ranges[1:] >= ranges[:-1]).all() and int(ranges[-1]) == k and int(ranges[0]) == 0
+    # the fast route (depth order of the Gaussians, ordered emission, tile partition) gives the
+    # same lists as the 64-bit sort of all keys
+    perm, offsets = stages.depth_order(n, order)
+    assert int(offsets[-1]) == k
+    d_sorted = (depth_bits & 0xFFFFFFFF)[perm.to(torch.int64)]       # unsigned order of the depth bits
+    assert (d_sorted[1:] >= d_sorted[:-1]).all()
+    ids_fast, ranges_fast = stages.tile_lists(cam, n, k, order)
+    assert torch.equal(ids_fast, vals) and torch.equal(ranges_fast, ranges)
+    del ids_fast, ranges_fast, perm, offsets, d_sorted
     tile_of = (keys >> 32).to(torch.int64)
     r = ranges.to(torch.int64)
     t_last = int(tile_of[-1])

@@ -188,6 +188,85 @@ def test_sort_pairs_vs_oracle_on_emitted_keys(oracle):
     assert (dv.cpu().numpy() == S["sorted_ids"]).all()
 
 
+# ------------------------------------------------------------------------------- stages 2+3, fast route
+@pytest.mark.parametrize("count,key_bits,ties", [(2, 32, False), (1000, 32, False), (8192, 8, True), (8193, 13, False),
+                                                 (70_000, 15, True), (1_000_003, 32, False), (300_001, 32, True),
+                                                 (200_000, 1, True), (123_457, 17, False)])
+def test_sort_pairs_u32_matches_stable_sort(count, key_bits, ties):
+    """Stable ascending unsigned sort of keys that use their low key_bits bits."""
+    st_ = _stages()
+    rng = np.random.default_rng(count + key_bits)
+    if ties:
+        pool = rng.integers(0, 1 << key_bits, 37, dtype=np.uint64)
+        keys = rng.choice(pool, count).astype(np.uint32)
+    else:
+        keys = rng.integers(0, 1 << key_bits, count, dtype=np.uint64).astype(np.uint32)
+    vals = np.arange(count, dtype=np.uint32)
+    rng.shuffle(vals)
+    dk, dv = dev(keys.view(np.int32)), dev(vals.view(np.int32))
+    st_.sort_pairs_u32(dk, dv, key_bits)
+    torch.cuda.synchronize()
+    order = np.argsort(keys, kind="stable")                  # unsigned order
+    assert (dk.cpu().numpy().view(np.uint32) == keys[order]).all()
+    assert (dv.cpu().numpy().view(np.uint32) == vals[order]).all()
+
+
+def test_sort_pairs_u32_orders_depth_bits_like_the_64_bit_keys():
+    """Unsigned order of float bits: positive depths ascending, then negative depths by
+    ascending magnitude: the order the sign-extended 64-bit keys have inside one tile
+    (negative keys first there, which the tile slot 0 of the fast route reproduces)."""
+    st_ = _stages()
+    rng = np.random.default_rng(5)
+    depth = np.concatenate([rng.uniform(0.01, 90, 5000), -rng.uniform(0.01, 90, 700), [0.0, -0.0]]).astype(np.float32)
+    rng.shuffle(depth)
+    bits = depth.view(np.uint32)
+    dk, dv = dev(bits.view(np.int32)), dev(np.arange(len(bits), dtype=np.int32))
+    st_.sort_pairs_u32(dk, dv, 32)
+    got = dv.cpu().numpy()
+    keys64 = depth.view(np.int32).astype(np.int64)          # sign-extended, tile 0
+    neg = keys64 < 0
+    want = np.concatenate([np.argsort(np.where(neg, np.iinfo(np.int64).max, keys64), kind="stable")[:(~neg).sum()],
+                           np.argsort(np.where(neg, keys64, np.iinfo(np.int64).max), kind="stable")[:neg.sum()]])
+    assert (got == want).all()
+
+
+@pytest.mark.parametrize("n,W,H,scale_mul,flip", [(20000, 256, 256, 2.0, 0), (3000, 200, 120, 12.0, 0),
+                                                  (500, 64, 48, 3.0, 120), (1, 32, 32, 1.0, 0), (2, 32, 32, 1.0, 0),
+                                                  (60000, 512, 384, 3.0, 500), (4000, 40, 30, 8.0, 50),
+                                                  (30000, 3840, 2160, 6.0, 300)])
+def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip):
+    """Depth order + ordered emission + tile partition give the oracle's sorted ids and ranges
+    (the result of the stable 64-bit sort of the emitted keys) bit for bit, including keys with
+    negative depths, the last Gaussian that never emits, 1-pass (<= 255 tiles) and 4K plans."""
+    st_ = _stages()
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=11 + n, scale_mul=scale_mul,
+                                               flip_behind=flip)
+    oracle.free(st)
+    k = S["num_keys"]
+    cam = st_.camera_from_scene(sc, DEV)
+    order = st_.new_order(n, DEV)
+    splats, radii_g, cov3d, block_sums = st_.project_fwd(cam, dev(A["means_3d"]), dev(A["scales"]),
+                                                         dev(A["rotations"]), dev(A["opacities"]), dev(A["shs"]),
+                                                         order=order)
+    perm, offsets = st_.depth_order(n, order)
+    torch.cuda.synchronize()
+    depth_bits = splats[:, 2].contiguous().view(torch.int32).cpu().numpy().view(np.uint32)
+    assert (perm.cpu().numpy() == np.argsort(depth_bits, kind="stable")).all()
+    tt = S["tiles_touched"].astype(np.int64).copy()
+    tt[-1] = 0
+    tt_sorted = tt[perm.cpu().numpy()]
+    pad = np.zeros((-n) % 256, np.int64)
+    sums = np.concatenate([tt_sorted, pad]).reshape(-1, 256).sum(1)
+    assert (offsets.cpu().numpy().astype(np.int64) == np.concatenate([[0], np.cumsum(sums)])).all()
+    assert int(offsets[-1]) == k
+    ids, ranges = st_.tile_lists(cam, n, k, order)
+    torch.cuda.synchronize()
+    assert (ids.cpu().numpy() == S["sorted_ids"]).all()
+    assert (ranges.cpu().numpy() == S["ranges"]).all()
+    if flip:
+        assert (S["sorted_keys"] < 0).any() and S["ranges"][0] > 0
+
+
 # ------------------------------------------------------------------------------- stage 3
 def test_tile_ranges_reference_kats():
     import json
