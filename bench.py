@@ -32,26 +32,27 @@ BWD_PAIR_FLOPS, BWD_REJECT_FLOPS = 72, 15
 # profiles/cfg2_hbm_traffic_per_kernel.md).  Counters cannot be read from inside this process, so
 # the figures are quoted here and only reported when workload and key count are the profiled ones.
 MEASURED_TRAFFIC = {
-    ("cfg2", 32604809): {
-        "project_fwd_kernel": 936.5e6, "emit_keys_kernel": 536.9e6, "radix_hist_kernel": 275.4e6,
-        "radix_onesweep_kernel": 908.5e6, "gaussian_bwd_kernel": 1333.2e6,
-        "blend_fwd_kernel": 78.5e6, "blend_bwd_kernel": 194.1e6,
-    },
 }
 
 
-def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, passes, counters):
+def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, counters):
     """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch."""
+    slot_bytes = 2 if tiles + 1 <= 65535 else 4
     if kernel == "project_fwd_kernel":
-        return "hbm", n * (44 + 12 * coeffs + 8 + 64), "B"
+        # inputs 44 + 12c bytes, outputs radii + cov3d + splat record + depth key + tile rectangle
+        return "hbm", n * (44 + 12 * coeffs + 4 + 24 + 48 + 4 + 8), "B"
     if kernel == "gaussian_bwd_kernel":
         return "hbm", n * (112 + 76 + 12 * coeffs), "B"
-    if kernel == "emit_keys_kernel":
-        return "hbm", 20 * n + 12 * k, "B"
-    if kernel == "radix_onesweep_kernel":
-        return "hbm", 24 * k, "B"
-    if kernel == "radix_hist_kernel":
-        return "hbm", 8 * k, "B"
+    if kernel == "hist32_kernel":
+        return "hbm", 4 * n, "B"
+    if kernel == "onesweep32_kernel<sort>":                  # depth sort of the Gaussians: key + id, in and out
+        return "hbm", 16 * n, "B"
+    if kernel == "ordered_block_sums_kernel":
+        return "hbm", 12 * n, "B"
+    if kernel == "emit_ordered_kernel":
+        return "hbm", 12 * n + (slot_bytes + 4) * k, "B"
+    if kernel == "onesweep32_kernel<tile partition>":        # tile partition: slot + id, in and out
+        return "hbm", 2 * (slot_bytes + 4) * k, "B"
     if kernel == "blend_fwd_kernel" and counters is not None:
         rej = counters.pairs_fwd - counters.pairs_fwd_applied
         return "valu", counters.pairs_fwd_applied * FWD_PAIR_FLOPS + rej * FWD_REJECT_FLOPS, "FLOP"
@@ -59,6 +60,18 @@ def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, passes, counters):
         rej = counters.pairs_bwd - counters.pairs_bwd_valid
         return "valu", counters.pairs_bwd_valid * BWD_PAIR_FLOPS + rej * BWD_REJECT_FLOPS, "FLOP"
     return None, 0, ""
+
+
+def roofline_entry(name, avg, lps, bound, work, traffic):
+    if bound == "hbm":
+        achieved = work / (avg * 1e-3) / 1e9
+        return {"kernel": name, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "avg_launch_ms": round(avg, 4),
+                "launches_per_step": lps, "algorithmic_bytes_per_launch": int(work)}
+    achieved = work / (avg * 1e-3) / 1e12
+    return {"kernel": name, "bound": "valu", "achieved": round(achieved, 2), "peak": VALU_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": round(achieved / VALU_PEAK_TFLOPS, 4), "traffic": traffic,
+            "avg_launch_ms": round(avg, 4), "launches_per_step": lps, "algorithmic_flop_per_launch": int(work)}
 
 
 def main():
@@ -146,7 +159,6 @@ def main():
     torch.cuda.synchronize()
     k = st.num_keys
     tiles = cam.num_tiles
-    passes = int(_native.load().dsx_sort_passes(tiles))
 
     # ---- CPU baseline: the oracle's OpenMP build on the host cores, same inputs -----------------
     cpu_baseline = None
@@ -177,34 +189,28 @@ def main():
             "keys_match_gpu": bool(k_cpu == k),
         }
 
-    # ---- roofline of the dominant kernel --------------------------------------------------------
+    # ---- roofline of the dominant kernel (and of the dominant HBM-bound one, if that is another) ----
     table = []
     for name, (tot, cnt) in per_kernel.items():
         launches_per_step = cnt / args.steps
         avg = tot / cnt
-        bound, work, unit = algorithmic_work(name, n, k, W * H, tiles, coeffs, passes, counters)
+        bound, work, unit = algorithmic_work(name, n, k, W * H, tiles, coeffs, counters)
         table.append((tot / args.steps, name, avg, launches_per_step, bound, work, unit))
     table.sort(reverse=True)
+    measured = MEASURED_TRAFFIC.get((spec.name, int(k)), {}) if args.n is None else {}
     roofline = None
+    roofline_hbm = None
     for ms_step, name, avg, lps, bound, work, unit in table:
         if bound is None:
             continue
-        if bound == "hbm":
-            achieved = work / (avg * 1e-3) / 1e9
-            roofline = {"kernel": name, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                        "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                        "avg_launch_ms": round(avg, 4), "launches_per_step": lps,
-                        "algorithmic_bytes_per_launch": int(work)}
-        else:
-            achieved = work / (avg * 1e-3) / 1e12
-            roofline = {"kernel": name, "bound": "valu", "achieved": round(achieved, 2), "peak": VALU_PEAK_TFLOPS,
-                        "unit": "TFLOP/s", "frac": round(achieved / VALU_PEAK_TFLOPS, 4), "traffic": None,
-                        "avg_launch_ms": round(avg, 4), "launches_per_step": lps,
-                        "algorithmic_flop_per_launch": int(work)}
-        if args.n is None:
-            traffic = MEASURED_TRAFFIC.get((spec.name, int(k)), {}).get(name)
-            roofline["traffic"] = int(traffic) if traffic else None
-        break
+        traffic = measured.get(name)
+        entry = roofline_entry(name, avg, lps, bound, work, int(traffic) if traffic else None)
+        if roofline is None:
+            roofline = entry
+        if roofline_hbm is None and bound == "hbm":
+            roofline_hbm = entry
+        if roofline is not None and roofline_hbm is not None:
+            break
     if args.verbose:
         for ms_step, name, avg, lps, bound, work, unit in table:
             extra = ""
@@ -226,10 +232,11 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: %d Gaussians, %dx%d, SH degree %d, %s" %
                                (spec.name, n, W, H, sc["sh_degree"], "forward+backward" if do_backward else "forward"),
-                   "num_keys": int(k), "tiles": int(tiles), "radix_passes": passes},
+                   "num_keys": int(k), "tiles": int(tiles)},
         "mpix_per_s": round(W * H / (ms_per_step * 1e-3) / 1e6, 1),
         "kernels_ms_per_step": {name: round(ms_step, 4) for ms_step, name, *_ in table},
         "roofline": roofline,
+        "roofline_hbm": roofline_hbm,
         "cpu_baseline": cpu_baseline,
     }
     print(json.dumps(out))

@@ -166,7 +166,7 @@ SortU32Layout sort_u32_layout(int64_t count, int key_bits)
     l.keys_alt = 0;
     l.values_alt = align((size_t)count * 4);
     l.sort = align(l.values_alt + (size_t)count * 4);
-    l.bytes = l.sort + sort32_workspace(count, key_bits).bytes;
+    l.bytes = l.sort + sort32_workspace(count, key_bits, kDepthSortTile).bytes;
     return l;
 }
 } // namespace

@@ -107,15 +107,27 @@ ForwardWorkspace forward_workspace(int64_t k, int num_tiles);
 // ---- 32-bit radix sort (depth order of the Gaussians, tile partition of the tile lists) ----
 constexpr int kBits32 = 8;
 constexpr int kBins32 = 1 << kBits32;
-#ifndef DSX_SORT32_THREADS
-#define DSX_SORT32_THREADS 512
+// Two geometries of the same pass kernel: the depth sort of the N Gaussians (few keys: small
+// tiles so that the launch fills the chip) and the partition of the K pairs (large tiles: the
+// look-back traffic falls with the number of tiles).
+#ifndef DSX_NSORT_THREADS
+#define DSX_NSORT_THREADS 512
 #endif
-#ifndef DSX_SORT32_ITEMS
-#define DSX_SORT32_ITEMS 16
+#ifndef DSX_NSORT_ITEMS
+#define DSX_NSORT_ITEMS 16
 #endif
-constexpr int kSort32Threads = DSX_SORT32_THREADS;
-constexpr int kSort32Items = DSX_SORT32_ITEMS;
-constexpr int kSort32Tile = kSort32Threads * kSort32Items;
+#ifndef DSX_KSORT_THREADS
+#define DSX_KSORT_THREADS 512
+#endif
+#ifndef DSX_KSORT_ITEMS
+#define DSX_KSORT_ITEMS 16
+#endif
+constexpr int kDepthSortThreads = DSX_NSORT_THREADS;
+constexpr int kDepthSortItems = DSX_NSORT_ITEMS;
+constexpr int kDepthSortTile = kDepthSortThreads * kDepthSortItems;
+constexpr int kListSortThreads = DSX_KSORT_THREADS;
+constexpr int kListSortItems = DSX_KSORT_ITEMS;
+constexpr int kListSortTile = kListSortThreads * kListSortItems;
 constexpr int kMaxPasses32 = 4;
 
 // Digits of a key whose low `key_bits` bits are significant: fewest passes with digits of at
@@ -164,7 +176,7 @@ struct Sort32Workspace
     int passes;
     int64_t tiles;
 };
-Sort32Workspace sort32_workspace(int64_t count, int key_bits);
+Sort32Workspace sort32_workspace(int64_t count, int key_bits, int tile_keys);
 
 // Per-Gaussian buffer that carries the depth order from the projection to the tile lists.
 struct OrderLayout
@@ -174,6 +186,7 @@ struct OrderLayout
     size_t ids_a;      // uint32[n]  the depth order ends here
     size_t ids_b;      // uint32[n]
     size_t rects;      // uint2[n]   packed tile rectangle (written by the projection)
+    size_t rects_sorted; // uint2[n] the same in depth order
     size_t block_sums; // uint32[blocks + 1] tile counts of 256 consecutive Gaussians IN DEPTH ORDER, scanned
     size_t sort;       // Sort32Workspace
     size_t bytes;

@@ -28,13 +28,15 @@ __device__ __forceinline__ uint32_t wave_incl_scan32(uint32_t v, int lane)
 }
 
 // lanes of the wavefront that hold the same (up to 8-bit) digit and are valid; uniform flow only
-__device__ __forceinline__ uint64_t match_digit8(uint32_t d, bool valid)
+__device__ __forceinline__ uint64_t match_digit8(uint32_t d, bool valid, int bits)
 {
     const uint64_t v = __ballot(valid);
     uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
 #pragma unroll
     for(int b = 0; b < kBits32; ++b)
     {
+        if(b >= bits) // uniform: digits narrower than 8 bits need fewer rounds
+            break;
         const uint32_t x = (uint32_t)(((int32_t)(d << (31 - b))) >> 31); // all ones where bit b is set
         const uint64_t m = __ballot(x != 0);
         lo &= ~((uint32_t)m ^ x);
@@ -51,10 +53,17 @@ __device__ __forceinline__ uint32_t lane_below32(uint32_t v, uint32_t first)
 // ---------------------------------------------------------------------------------------
 // histograms of every digit in one read (run-length merged: neighbouring keys often share a digit)
 // ---------------------------------------------------------------------------------------
+#ifndef DSX_HIST_BLOCKS
+#define DSX_HIST_BLOCKS 512 // few workgroups: each ends with one global atomic per bin, which serialise per address
+#endif
+#ifndef DSX_EMIT_BLOCKS
+#define DSX_EMIT_BLOCKS 2048
+#endif
 constexpr int kHist32Threads = 256;
 constexpr int kHist32Items = 8;
 
-__global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const uint32_t* __restrict__ keys, int64_t count,
+template <typename KeyT>
+__global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const KeyT* __restrict__ keys, int64_t count,
                                                                 const Digits32 plan,
                                                                 uint32_t* __restrict__ global_hist)
 {
@@ -75,7 +84,7 @@ __global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const uint32_t* 
         {
             const int64_t i = c * chunk + it * kHist32Threads + tid;
             valid[it] = i < count;
-            s[it] = valid[it] ? __builtin_nontemporal_load(keys + i) : 0u;
+            s[it] = valid[it] ? (uint32_t)__builtin_nontemporal_load(keys + i) : 0u;
         }
 #pragma unroll
         for(int it = 0; it < kHist32Items; ++it)
@@ -130,19 +139,24 @@ constexpr uint32_t kFlagInclusive32 = 2u << 30;
 constexpr uint32_t kFlagMask32 = 3u << 30;
 constexpr uint32_t kValueMask32 = ~kFlagMask32;
 constexpr int kSpinLimit32 = 1 << 18; // bounded wait: a stuck predecessor ends in an error flag, not a hang
-constexpr int kLookBatch32 = 4;
-constexpr int kSort32Waves = kSort32Threads / DSX_WAVE;
+#ifndef DSX_LOOK32
+#define DSX_LOOK32 4
+#endif
+constexpr int kLookBatch32 = DSX_LOOK32;
 
-static_assert(kSort32Threads >= kBins32, "one thread per digit");
-static_assert(kSort32Tile <= 65535, "u16 ranks");
+static_assert(kDepthSortThreads >= kBins32 && kListSortThreads >= kBins32, "one thread per digit");
+static_assert(kDepthSortTile <= 65535 && kListSortTile <= 65535, "u16 ranks");
 
 // vals_in == nullptr: the values are the input positions (iota).  keys_out == nullptr: the
-// keys are not needed after this pass.
+// keys are not needed after this pass.  KeyT: uint32_t, or uint16_t for tile slots that fit.
+template <typename KeyT, int kSort32Threads, int kSort32Items>
 __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
-    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ keys_out,
+    const KeyT* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, KeyT* __restrict__ keys_out,
     uint32_t* __restrict__ vals_out, int64_t count, int shift, uint32_t mask, const uint32_t* __restrict__ hist_excl,
     uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag)
 {
+    constexpr int kSort32Tile = kSort32Threads * kSort32Items;
+    constexpr int kSort32Waves = kSort32Threads / DSX_WAVE;
     __shared__ uint32_t s_keys[kSort32Tile]; // reused for the values in the second round
     __shared__ uint16_t s_whist[kSort32Waves][kBins32];
     __shared__ uint32_t s_digit_start[kBins32];
@@ -162,6 +176,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     const int64_t tile = s_tile;
     const int64_t tile_base = tile * kSort32Tile;
     const int tile_n = (int)min((int64_t)kSort32Tile, count - tile_base);
+    const int bits = 32 - __builtin_clz(mask); // mask = 2^bits - 1, bits >= 1
 
     // ---- load (striped inside each wavefront: coalesced, order = (item, lane)) -------------
     uint32_t key[kSort32Items];
@@ -175,7 +190,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
         val[it] = 0;
         if(local < tile_n)
         {
-            key[it] = __builtin_nontemporal_load(keys_in + tile_base + local);
+            key[it] = (uint32_t)__builtin_nontemporal_load(keys_in + tile_base + local);
             val[it] = vals_in ? __builtin_nontemporal_load(vals_in + tile_base + local) : (uint32_t)(tile_base + local);
         }
     }
@@ -188,7 +203,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
         const int local = wave * (kSort32Items * 64) + it * 64 + lane;
         const bool valid = local < tile_n;
         const uint32_t d = (key[it] >> shift) & mask;
-        const uint64_t m = match_digit8(d, valid);
+        const uint64_t m = match_digit8(d, valid, bits);
         const uint32_t below = (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
         const uint32_t old = wh[d];
         __builtin_amdgcn_wave_barrier();
@@ -200,7 +215,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     __syncthreads();
 
     // ---- per-digit totals of the tile (thread d <-> digit d), wave offsets, digit starts ----
-    const bool digit_thread = tid < kBins32;
+    const bool digit_thread = tid < kBins32; // thread d owns digit d (bins above the mask stay empty)
     uint32_t total = 0;
     uint32_t* my_status = status + tile * kBins32 + (digit_thread ? tid : 0);
     if(digit_thread)
@@ -246,7 +261,11 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     if(digit_thread)
     {
         uint32_t excl = 0;
-        if(tile > 0)
+#ifdef EXP_NOLOOK
+        if(false)
+#else
+        if(tile > 0 && (uint32_t)tid <= mask) // bins above the mask are empty in every tile
+#endif
         {
             int64_t t = tile - 1; // next predecessor to account for
             int spins = 0;
@@ -302,7 +321,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
             const uint32_t kk = s_keys[j];
             out[it] = s_gbase[(kk >> shift) & mask] + (uint32_t)j;
             if(keys_out)
-                keys_out[out[it]] = kk;
+                keys_out[out[it]] = (KeyT)kk;
         }
     }
     __syncthreads();
@@ -325,12 +344,12 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     }
 }
 
-Sort32Workspace sort32_workspace(int64_t count, int key_bits)
+Sort32Workspace sort32_workspace(int64_t count, int key_bits, int tile_keys)
 {
     auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
     Sort32Workspace w;
     w.passes = digits32(key_bits).passes;
-    w.tiles = (count + kSort32Tile - 1) / kSort32Tile;
+    w.tiles = (count + tile_keys - 1) / tile_keys;
     size_t off = 0;
     w.hist = off;
     off = align(off + (size_t)w.passes * kBins32 * 4);
@@ -342,9 +361,62 @@ Sort32Workspace sort32_workspace(int64_t count, int key_bits)
     return w;
 }
 
-// Stable ascending sort of `count` (key, value) pairs by the low key_bits bits of the key.
+// zeroes histograms, tile counters and look-back statuses of one sort
+static int sort32_clear(int64_t count, int key_bits, int tile_keys, void* sort_ws, hipStream_t stream)
+{
+    const Sort32Workspace w = sort32_workspace(count, key_bits, tile_keys);
+    return launch_fill_u32(reinterpret_cast<uint32_t*>(static_cast<char*>(sort_ws) + w.hist), (int64_t)(w.bytes / 4), 0u,
+                           stream);
+}
+
+// The digit passes of a sort whose raw digit histograms are already in the workspace.
 // Ping-pong between (keys_a, vals_a) and (keys_b, vals_b); *keys_out / *vals_out say where the
 // result is (keys only when keep_keys).
+template <typename KeyT, int kThreads, int kItems>
+static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* vals_a, KeyT* keys_b, uint32_t* vals_b,
+                         bool iota_values, bool keep_keys, void* sort_ws, const char* label, hipStream_t stream,
+                         KeyT** keys_out, uint32_t** vals_out)
+{
+    const Sort32Workspace w = sort32_workspace(count, key_bits, kThreads * kItems);
+    const Digits32 plan = digits32(key_bits);
+    char* base = static_cast<char*>(sort_ws);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(base + w.hist);
+    uint32_t* counters = reinterpret_cast<uint32_t*>(base + w.counters);
+    uint32_t* status = reinterpret_cast<uint32_t*>(base + w.status);
+    {
+        DSX_TIMED("hist32_scan_kernel", stream);
+        hipLaunchKernelGGL(hist32_scan_kernel, dim3(w.passes), dim3(kBins32), 0, stream, hist);
+    }
+    DSX_LAUNCH_CHECK();
+    KeyT* kin = keys_a;
+    uint32_t* vin = vals_a;
+    KeyT* kout = keys_b;
+    uint32_t* vout = vals_b;
+    for(int p = 0; p < w.passes; ++p)
+    {
+        const bool last = p == w.passes - 1;
+        {
+            DSX_TIMED(label, stream);
+            hipLaunchKernelGGL((onesweep32_kernel<KeyT, kThreads, kItems>), dim3((unsigned)w.tiles), dim3(kThreads), 0, stream,
+                               (const KeyT*)kin, (const uint32_t*)((p == 0 && iota_values) ? nullptr : vin),
+                               (last && !keep_keys) ? (KeyT*)nullptr : kout, vout, count, plan.shift[p], plan.mask[p],
+                               (const uint32_t*)(hist + p * kBins32), status + (size_t)p * w.tiles * kBins32,
+                               counters + p, counters + w.passes);
+        }
+        DSX_LAUNCH_CHECK();
+        KeyT* tk = kin;
+        kin = kout;
+        kout = tk;
+        uint32_t* tv = vin;
+        vin = vout;
+        vout = tv;
+    }
+    *keys_out = kin;
+    *vals_out = vin;
+    return DSX_OK;
+}
+
+// Stable ascending sort of `count` (key, value) pairs by the low key_bits bits of the key.
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
                   uint32_t** keys_out, uint32_t** vals_out)
@@ -355,52 +427,20 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
         return DSX_OK;
     if(count >= (1ll << 30))
         return DSX_ERR_TOO_LARGE;
-    const Sort32Workspace w = sort32_workspace(count, key_bits);
-    const Digits32 plan = digits32(key_bits);
-    char* base = static_cast<char*>(sort_ws);
-    uint32_t* hist = reinterpret_cast<uint32_t*>(base + w.hist);
-    uint32_t* counters = reinterpret_cast<uint32_t*>(base + w.counters);
-    uint32_t* status = reinterpret_cast<uint32_t*>(base + w.status);
-    int rc = launch_fill_u32(hist, (int64_t)(w.bytes / 4), 0u, stream);
+    int rc = sort32_clear(count, key_bits, kDepthSortTile, sort_ws, stream);
     if(rc)
         return rc;
+    const Sort32Workspace w = sort32_workspace(count, key_bits, kDepthSortTile);
     const int64_t chunks = (count + kHist32Threads * kHist32Items - 1) / (kHist32Threads * kHist32Items);
     {
         DSX_TIMED("hist32_kernel", stream);
-        hipLaunchKernelGGL(hist32_kernel, dim3((unsigned)min((int64_t)2048, chunks)), dim3(kHist32Threads), 0, stream,
-                           keys_a, count, plan, hist);
+        hipLaunchKernelGGL(hist32_kernel<uint32_t>, dim3((unsigned)min((int64_t)DSX_HIST_BLOCKS, chunks)), dim3(kHist32Threads), 0,
+                           stream, (const uint32_t*)keys_a, count, digits32(key_bits),
+                           reinterpret_cast<uint32_t*>(static_cast<char*>(sort_ws) + w.hist));
     }
     DSX_LAUNCH_CHECK();
-    {
-        DSX_TIMED("hist32_scan_kernel", stream);
-        hipLaunchKernelGGL(hist32_scan_kernel, dim3(w.passes), dim3(kBins32), 0, stream, hist);
-    }
-    DSX_LAUNCH_CHECK();
-    uint32_t* kin = keys_a;
-    uint32_t* vin = vals_a;
-    uint32_t* kout = keys_b;
-    uint32_t* vout = vals_b;
-    for(int p = 0; p < w.passes; ++p)
-    {
-        const bool last = p == w.passes - 1;
-        {
-            DSX_TIMED("onesweep32_kernel", stream);
-            hipLaunchKernelGGL(onesweep32_kernel, dim3((unsigned)w.tiles), dim3(kSort32Threads), 0, stream, kin,
-                               (p == 0 && iota_values) ? nullptr : vin, (last && !keep_keys) ? nullptr : kout, vout,
-                               count, plan.shift[p], plan.mask[p], hist + p * kBins32,
-                               status + (size_t)p * w.tiles * kBins32, counters + p, counters + w.passes);
-        }
-        DSX_LAUNCH_CHECK();
-        uint32_t* tk = kin;
-        kin = kout;
-        kout = tk;
-        uint32_t* tv = vin;
-        vin = vout;
-        vout = tv;
-    }
-    *keys_out = kin;
-    *vals_out = vin;
-    return DSX_OK;
+    return sort32_passes<uint32_t, kDepthSortThreads, kDepthSortItems>(count, key_bits, keys_a, vals_a, keys_b, vals_b, iota_values, keep_keys, sort_ws,
+                                   "onesweep32_kernel<sort>", stream, keys_out, vals_out);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -422,10 +462,12 @@ OrderLayout order_layout(int64_t n)
     off = align(off + (size_t)n * 4);
     o.rects = off;
     off = align(off + (size_t)n * 8);
+    o.rects_sorted = off;
+    off = align(off + (size_t)n * 8);
     o.block_sums = off;
     off = align(off + (size_t)((n + kProjBlock - 1) / kProjBlock + 1) * 4);
     o.sort = off;
-    off += sort32_workspace(n, 32).bytes;
+    off += sort32_workspace(n, 32, kDepthSortTile).bytes;
     o.bytes = align(off);
     return o;
 }
@@ -435,9 +477,12 @@ __device__ __forceinline__ uint32_t rect_count(uint2 r)
     return (r.y & 0xffffu) * ((r.y >> 16) & 0x7fffu);
 }
 
-// tile count of each run of 256 Gaussians taken in depth order
+// Tile count of each run of 256 Gaussians taken in depth order.  This is the one random
+// gather of the per-Gaussian rectangles; they are stored again in depth order so that the
+// emission reads them in sequence.
 __global__ __launch_bounds__(kProjBlock) void ordered_block_sums_kernel(const uint32_t* __restrict__ order,
                                                                        const uint2* __restrict__ rects, int64_t n,
+                                                                       uint2* __restrict__ rects_sorted,
                                                                        uint32_t* __restrict__ block_sums)
 {
     __shared__ uint32_t wave_sums[kProjBlock / DSX_WAVE];
@@ -445,7 +490,11 @@ __global__ __launch_bounds__(kProjBlock) void ordered_block_sums_kernel(const ui
     const int64_t p = (int64_t)blockIdx.x * kProjBlock + tid;
     uint32_t count = 0;
     if(p < n)
-        count = rect_count(rects[order[p]]);
+    {
+        const uint2 r = rects[order[p]];
+        rects_sorted[p] = r;
+        count = rect_count(r);
+    }
     const uint32_t ws = wave_sum_u32(count);
     if((tid & 63) == 0)
         wave_sums[tid >> 6] = ws;
@@ -478,7 +527,8 @@ int launch_depth_order(int64_t n, void* order, hipStream_t stream)
     {
         DSX_TIMED("ordered_block_sums_kernel", stream);
         hipLaunchKernelGGL(ordered_block_sums_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, perm,
-                           reinterpret_cast<const uint2*>(base + o.rects), n, block_sums);
+                           reinterpret_cast<const uint2*>(base + o.rects), n,
+                           reinterpret_cast<uint2*>(base + o.rects_sorted), block_sums);
     }
     DSX_LAUNCH_CHECK();
     return launch_scan_u32(blocks, block_sums, block_sums + blocks, stream);
@@ -489,12 +539,13 @@ int launch_depth_order(int64_t n, void* order, hipStream_t stream)
 // OUTPUT pair, so stores are contiguous however uneven the per-Gaussian tile counts are
 // ---------------------------------------------------------------------------------------
 
+template <typename SlotT>
 __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t* __restrict__ order,
-                                                                  const uint2* __restrict__ rects,
+                                                                  const uint2* __restrict__ rects_sorted,
                                                                   const uint32_t* __restrict__ block_offsets,
-                                                                  int64_t n, int64_t k, int ntx,
-                                                                  uint32_t* __restrict__ slots,
-                                                                  int32_t* __restrict__ ids)
+                                                                  int64_t n, int64_t k, int ntx, const Digits32 plan,
+                                                                  SlotT* __restrict__ slots, int32_t* __restrict__ ids,
+                                                                  uint32_t* __restrict__ global_hist)
 {
     __shared__ uint32_t s_off[kProjBlock + 1];
     __shared__ uint32_t s_origin[kProjBlock]; // slot of the rectangle's first tile (0 for negative depths)
@@ -502,72 +553,103 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     __shared__ float s_winv[kProjBlock];
     __shared__ uint32_t s_id[kProjBlock];
     __shared__ uint32_t wave_tot[kProjBlock / DSX_WAVE];
+    __shared__ uint32_t hist[kMaxPasses32 * kBins32]; // digit histograms of the partition that follows
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int64_t p = (int64_t)blockIdx.x * kProjBlock + tid;
+    for(int j = tid; j < plan.passes * kBins32; j += kProjBlock)
+        hist[j] = 0;
 
-    uint32_t count = 0;
-    if(p < n)
+    const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
+    for(int64_t blk = blockIdx.x; blk < blocks; blk += gridDim.x)
     {
-        const uint32_t g = order[p];
-        const uint2 r = rects[g];
-        count = rect_count(r);
-        const uint32_t w = r.y & 0xffffu;
-        const bool negative = (r.y >> 31) != 0;
-        s_origin[tid] = negative ? 0u : (r.x >> 16) * (uint32_t)ntx + (r.x & 0xffffu) + 1u;
-        s_w[tid] = negative ? 0u : w;
-        s_winv[tid] = 1.0f / (float)(w ? w : 1u);
-        s_id[tid] = g;
-    }
-    const uint32_t incl = wave_incl_scan32(count, lane);
-    if(lane == 63)
-        wave_tot[wave] = incl;
-    __syncthreads();
-    uint32_t prefix = 0;
-    for(int w = 0; w < wave; ++w)
-        prefix += wave_tot[w];
-    s_off[tid] = prefix + incl - count;
-    if(tid == kProjBlock - 1)
-        s_off[kProjBlock] = prefix + incl;
-    __syncthreads();
+        __syncthreads(); // the previous round has finished with the LDS arrays
+        const int64_t p = blk * kProjBlock + tid;
+        uint32_t count = 0;
+        if(p < n)
+        {
+            const uint32_t g = order[p];
+            const uint2 r = rects_sorted[p];
+            count = rect_count(r);
+            const uint32_t w = r.y & 0xffffu;
+            const bool negative = (r.y >> 31) != 0;
+            s_origin[tid] = negative ? 0u : (r.x >> 16) * (uint32_t)ntx + (r.x & 0xffffu) + 1u;
+            s_w[tid] = negative ? 0u : w;
+            s_winv[tid] = 1.0f / (float)(w ? w : 1u);
+            s_id[tid] = g;
+        }
+        const uint32_t incl = wave_incl_scan32(count, lane);
+        if(lane == 63)
+            wave_tot[wave] = incl;
+        __syncthreads();
+        uint32_t prefix = 0;
+        for(int w = 0; w < wave; ++w)
+            prefix += wave_tot[w];
+        s_off[tid] = prefix + incl - count;
+        if(tid == kProjBlock - 1)
+            s_off[kProjBlock] = prefix + incl;
+        __syncthreads();
 
-    const uint32_t total = s_off[kProjBlock];
-    const int64_t base = block_offsets[blockIdx.x];
-    for(uint32_t j = tid; j < total; j += kProjBlock)
-    {
-        // largest g with s_off[g] <= j
-        int lo = 0, hi = kProjBlock;
-        while(hi - lo > 1)
+        const uint32_t total = s_off[kProjBlock];
+        const int64_t base = block_offsets[blk];
+        for(uint32_t j0 = 0; j0 < total; j0 += kProjBlock) // uniform trip count: ballots below
         {
-            const int mid = (lo + hi) >> 1;
-            if(s_off[mid] <= j)
-                lo = mid;
-            else
-                hi = mid;
-        }
-        const uint32_t r = j - s_off[lo];
-        const uint32_t w = s_w[lo];
-        uint32_t slot = 0;
-        if(w)
-        {
-            // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
-            uint32_t ry = (uint32_t)((float)r * s_winv[lo]);
-            if(ry * w > r)
-                --ry;
-            else if((ry + 1) * w <= r)
-                ++ry;
-            const uint32_t rx = r - ry * w;
-            slot = s_origin[lo] + ry * (uint32_t)ntx + rx;
-        }
-        const int64_t out = base + j;
-        if(out < k)
-        {
-            slots[out] = slot;
-            ids[out] = (int32_t)s_id[lo];
+            const uint32_t j = j0 + tid;
+            const bool valid = j < total && base + j < k;
+            uint32_t slot = 0;
+            uint32_t id = 0;
+            if(valid)
+            {
+                // largest g with s_off[g] <= j
+                int lo = 0, hi = kProjBlock;
+                while(hi - lo > 1)
+                {
+                    const int mid = (lo + hi) >> 1;
+                    if(s_off[mid] <= j)
+                        lo = mid;
+                    else
+                        hi = mid;
+                }
+                const uint32_t r = j - s_off[lo];
+                const uint32_t w = s_w[lo];
+                if(w)
+                {
+                    // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
+                    uint32_t ry = (uint32_t)((float)r * s_winv[lo]);
+                    if(ry * w > r)
+                        --ry;
+                    else if((ry + 1) * w <= r)
+                        ++ry;
+                    const uint32_t rx = r - ry * w;
+                    slot = s_origin[lo] + ry * (uint32_t)ntx + rx;
+                }
+                id = s_id[lo];
+                slots[base + j] = (SlotT)slot;
+                ids[base + j] = (int32_t)id;
+            }
+            // digit histograms: a run of equal digits in neighbouring lanes is added by its first lane
+            const uint64_t vmask = __ballot(valid); // valid lanes are a prefix of the wavefront
+            const int nvalid = __popcll(vmask);
+            for(int ps = 0; ps < plan.passes; ++ps)
+            {
+                const uint32_t d = (slot >> plan.shift[ps]) & plan.mask[ps];
+                const uint32_t below = lane_below32(d, ~d);
+                const bool head = valid && (lane == 0 || below != d);
+                const uint64_t heads = __ballot(head);
+                if(head)
+                {
+                    const uint64_t above = lane == 63 ? 0ull : (heads >> (lane + 1));
+                    const int run = above ? __ffsll((unsigned long long)above) : nvalid - lane;
+                    atomicAdd(&hist[ps * kBins32 + d], (uint32_t)run);
+                }
+            }
         }
     }
+    __syncthreads();
+    for(int j = tid; j < plan.passes * kBins32; j += kProjBlock)
+        if(hist[j])
+            atomicAdd(&global_hist[j], hist[j]);
 }
 
 // ranges[j] = number of pairs whose tile is below j, by binary search in the sorted slots.
@@ -575,7 +657,8 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
 // cpp/rasterizer_torch.cu:31-39): the boundary after the LAST run is never recorded, so tiles
 // above the highest occupied tile inherit the START of that run, and ranges[num_tiles] = K.
 // Slot 0 (negative depths) is skipped by ranges[0].
-__global__ __launch_bounds__(256) void ranges_slots_kernel(const uint32_t* __restrict__ slots, int64_t k,
+template <typename SlotT>
+__global__ __launch_bounds__(256) void ranges_slots_kernel(const SlotT* __restrict__ slots, int64_t k,
                                                            int num_tiles, int32_t* __restrict__ ranges)
 {
     const int j = blockIdx.x * 256 + threadIdx.x;
@@ -600,22 +683,83 @@ __global__ __launch_bounds__(256) void ranges_slots_kernel(const uint32_t* __res
     ranges[j] = (int32_t)lo;
 }
 
+// tile slots 0..num_tiles fit 16 bits for every image up to 65534 tiles (4K has 32400)
+static bool slots_are_u16(int num_tiles)
+{
+    return num_tiles + 1 <= 65535;
+}
+
 ListsWorkspace lists_workspace(int64_t k, int num_tiles)
 {
     auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
     ListsWorkspace w;
+    const size_t slot_bytes = slots_are_u16(num_tiles) ? 2 : 4;
     w.passes = digits32(slot_bits(num_tiles)).passes;
     size_t off = 0;
     w.slots_a = off;
-    off = align(off + (size_t)k * 4);
+    off = align(off + (size_t)k * slot_bytes);
     w.slots_b = off;
-    off = align(off + (size_t)k * 4);
+    off = align(off + (size_t)k * slot_bytes);
     w.ids_alt = off;
     off = align(off + (size_t)k * 4);
     w.sort = off;
-    off += sort32_workspace(k, slot_bits(num_tiles)).bytes;
+    off += sort32_workspace(k, slot_bits(num_tiles), kListSortTile).bytes;
     w.bytes = align(off);
     return w;
+}
+
+template <typename SlotT>
+static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_tiles, const void* order,
+                           int32_t* sorted_ids, int32_t* ranges, void* workspace, hipStream_t stream)
+{
+    const SlotT* sorted_slots = nullptr;
+    if(k > 0)
+    {
+        const OrderLayout o = order_layout(n);
+        const ListsWorkspace w = lists_workspace(k, num_tiles);
+        const int bits = slot_bits(num_tiles);
+        const char* obase = static_cast<const char*>(order);
+        char* base = static_cast<char*>(workspace);
+        SlotT* slots_a = reinterpret_cast<SlotT*>(base + w.slots_a);
+        SlotT* slots_b = reinterpret_cast<SlotT*>(base + w.slots_b);
+        uint32_t* ids_final = reinterpret_cast<uint32_t*>(sorted_ids);
+        uint32_t* ids_other = reinterpret_cast<uint32_t*>(base + w.ids_alt);
+        // ping-pong parity: start so that the last pass lands the ids in the caller's buffer
+        const bool even = (w.passes % 2) == 0;
+        uint32_t* vals_a = even ? ids_final : ids_other;
+        uint32_t* vals_b = even ? ids_other : ids_final;
+        int rc = sort32_clear(k, bits, kListSortTile, base + w.sort, stream);
+        if(rc)
+            return rc;
+        const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
+        {
+            DSX_TIMED("emit_ordered_kernel", stream);
+            hipLaunchKernelGGL(emit_ordered_kernel<SlotT>, dim3((unsigned)min(blocks, (int64_t)DSX_EMIT_BLOCKS)), dim3(kProjBlock),
+                               0, stream, reinterpret_cast<const uint32_t*>(obase + o.ids_a),
+                               reinterpret_cast<const uint2*>(obase + o.rects_sorted),
+                               reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k, tiles_x(cam.image_width),
+                               digits32(bits), slots_a, reinterpret_cast<int32_t*>(vals_a),
+                               reinterpret_cast<uint32_t*>(base + w.sort + sort32_workspace(k, bits, kListSortTile).hist));
+        }
+        DSX_LAUNCH_CHECK();
+        SlotT* ko;
+        uint32_t* vo;
+        rc = sort32_passes<SlotT, kListSortThreads, kListSortItems>(k, bits, slots_a, vals_a, slots_b, vals_b, false, true, base + w.sort,
+                                  "onesweep32_kernel<tile partition>", stream, &ko, &vo);
+        if(rc)
+            return rc;
+        if(vo != ids_final)
+            return DSX_ERR_RUNTIME;
+        sorted_slots = ko;
+    }
+    const int count = num_tiles + 1;
+    {
+        DSX_TIMED("ranges_slots_kernel", stream);
+        hipLaunchKernelGGL(ranges_slots_kernel<SlotT>, dim3((count + 255) / 256), dim3(256), 0, stream, sorted_slots, k,
+                           num_tiles, ranges);
+    }
+    DSX_LAUNCH_CHECK();
+    return DSX_OK;
 }
 
 // order: buffer of order_layout(n) after launch_depth_order.  Writes sorted_ids[k], ranges[T+1].
@@ -623,52 +767,13 @@ int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* o
                       int32_t* ranges, void* workspace, hipStream_t stream)
 {
     const int num_tiles = tiles_x(cam.image_width) * tiles_y(cam.image_height);
-    const uint32_t* sorted_slots = nullptr;
-    if(k > 0 && n > 0)
-    {
-        if(k >= (1ll << 30))
-            return DSX_ERR_TOO_LARGE;
-        const OrderLayout o = order_layout(n);
-        const ListsWorkspace w = lists_workspace(k, num_tiles);
-        const char* obase = static_cast<const char*>(order);
-        char* base = static_cast<char*>(workspace);
-        uint32_t* slots_a = reinterpret_cast<uint32_t*>(base + w.slots_a);
-        uint32_t* slots_b = reinterpret_cast<uint32_t*>(base + w.slots_b);
-        uint32_t* ids_final = reinterpret_cast<uint32_t*>(sorted_ids);
-        uint32_t* ids_other = reinterpret_cast<uint32_t*>(base + w.ids_alt);
-        // ping-pong parity: start so that the last pass lands the ids in the caller's buffer
-        const bool even = (w.passes % 2) == 0;
-        uint32_t* vals_a = even ? ids_final : ids_other;
-        uint32_t* vals_b = even ? ids_other : ids_final;
-        const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
-        {
-            DSX_TIMED("emit_ordered_kernel", stream);
-            hipLaunchKernelGGL(emit_ordered_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
-                               reinterpret_cast<const uint32_t*>(obase + o.ids_a),
-                               reinterpret_cast<const uint2*>(obase + o.rects),
-                               reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k,
-                               tiles_x(cam.image_width), slots_a, reinterpret_cast<int32_t*>(vals_a));
-        }
-        DSX_LAUNCH_CHECK();
-        uint32_t *ko, *vo;
-        int rc = launch_sort32(k, slot_bits(num_tiles), slots_a, vals_a, slots_b, vals_b, false, true, base + w.sort,
-                               stream, &ko, &vo);
-        if(rc)
-            return rc;
-        if(vo != ids_final)
-            return DSX_ERR_RUNTIME;
-        sorted_slots = ko;
-    }
-    else
+    if(k >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
+    if(n <= 0)
         k = 0;
-    const int count = num_tiles + 1;
-    {
-        DSX_TIMED("ranges_slots_kernel", stream);
-        hipLaunchKernelGGL(ranges_slots_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, sorted_slots, k,
-                           num_tiles, ranges);
-    }
-    DSX_LAUNCH_CHECK();
-    return DSX_OK;
+    if(slots_are_u16(num_tiles))
+        return tile_lists_impl<uint16_t>(cam, n, k, num_tiles, order, sorted_ids, ranges, workspace, stream);
+    return tile_lists_impl<uint32_t>(cam, n, k, num_tiles, order, sorted_ids, ranges, workspace, stream);
 }
 
 } // namespace dsx

@@ -36,12 +36,13 @@ def test_host_helpers():
     # 32 depth bits + bits for tile ids 0..T (slot 0 = negative keys), at most 9 bits a pass
     assert lib.dsx_sort_passes(8160) == 5 and lib.dsx_sort_passes(255) == 5 and lib.dsx_sort_passes(32400) == 6
     assert lib.dsx_workspace_bytes(0, 0, 64, 64) >= 0
-    # tile lists: two uint32 slot buffers and one id buffer; 64-bit sort: key and value copies
-    assert (1 << 20) * 12 < lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080) < (1 << 20) * 14
+    # tile lists: two slot buffers (16-bit slots up to 65534 tiles, else 32-bit) and one id buffer
+    assert (1 << 20) * 8 < lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080) < (1 << 20) * 9
+    assert (1 << 20) * 12 < lib.dsx_workspace_bytes(0, 1 << 20, 16400, 1040) < (1 << 20) * 13
     assert lib.dsx_sort_workspace_bytes(1 << 20, 8160) > (1 << 20) * 12
     assert lib.dsx_sort_u32_workspace_bytes(1 << 20, 32) > (1 << 20) * 8
-    # order buffer: 4 uint32 arrays and one uint2 array per Gaussian
-    assert lib.dsx_order_bytes(1 << 20) > (1 << 20) * 24
+    # order buffer: 4 uint32 arrays and two uint2 arrays per Gaussian
+    assert lib.dsx_order_bytes(1 << 20) > (1 << 20) * 32
     assert b"workspace" in lib.dsx_error_string(-5)
     assert lib.dsx_error_string(0) == b"ok"
 

@@ -233,11 +233,12 @@ def test_sort_pairs_u32_orders_depth_bits_like_the_64_bit_keys():
 @pytest.mark.parametrize("n,W,H,scale_mul,flip", [(20000, 256, 256, 2.0, 0), (3000, 200, 120, 12.0, 0),
                                                   (500, 64, 48, 3.0, 120), (1, 32, 32, 1.0, 0), (2, 32, 32, 1.0, 0),
                                                   (60000, 512, 384, 3.0, 500), (4000, 40, 30, 8.0, 50),
-                                                  (30000, 3840, 2160, 6.0, 300)])
+                                                  (30000, 3840, 2160, 6.0, 300), (20000, 16400, 1040, 8.0, 100)])
 def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip):
     """Depth order + ordered emission + tile partition give the oracle's sorted ids and ranges
     (the result of the stable 64-bit sort of the emitted keys) bit for bit, including keys with
-    negative depths, the last Gaussian that never emits, 1-pass (<= 255 tiles) and 4K plans."""
+    negative depths, the last Gaussian that never emits, 1-pass (<= 255 tiles) and 4K plans, and
+    an image of more than 65534 tiles (32-bit instead of 16-bit tile slots)."""
     st_ = _stages()
     sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=11 + n, scale_mul=scale_mul,
                                                flip_behind=flip)
