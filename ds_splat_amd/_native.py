@@ -99,6 +99,31 @@ def load():
     return lib
 
 
+_ext = None
+
+
+def load_torch_ext():
+    """Imports the C++ torch binding (ds_splat_amd/lib/_dsx_torch*.so, built from csrc/torch_ext.cpp
+    and linked against libdsx.so).  Raises if it is not built: there is no Python fallback."""
+    global _ext
+    if _ext is not None:
+        return _ext
+    import glob
+    import importlib.util
+    import torch  # noqa: F401  (the binding links against torch's libraries)
+    load()
+    found = sorted(glob.glob(os.path.join(_HERE, "lib", "_dsx_torch*.so")))
+    if not found:
+        raise RuntimeError(
+            "ds_splat_amd: the torch binding ds_splat_amd/lib/_dsx_torch*.so is missing — build it with "
+            "`python -c 'import __graft_entry__ as g; g.build()'` or `make -C ds_splat_amd/csrc`")
+    spec = importlib.util.spec_from_file_location("_dsx_torch", found[0])
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    _ext = mod
+    return mod
+
+
 def check(status):
     if status != 0:
         raise RuntimeError(load().dsx_error_string(status).decode())

@@ -1,0 +1,159 @@
+// Thin PyTorch binding over the C ABI of libdsx (include/dsx.h): it owns no kernels and no
+// HIP calls.  It plays the role of the reference's pybind module ds_splat_cuda
+// (cpp/rasterizer_python.cpp:3-23) and of the tensor plumbing in cpp/rasterizer_torch.cu:170-316:
+// allocate the outputs as torch tensors, hand raw device pointers and the caller's stream to
+// the library, return the tensors the autograd function keeps for the backward.
+#include <torch/extension.h>
+
+#include <c10/core/DeviceGuard.h>
+
+#include <stdexcept>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "dsx.h"
+
+namespace
+{
+
+void check(int status)
+{
+    if(status != DSX_OK)
+        throw std::runtime_error(dsx_error_string(status));
+}
+
+const float* fptr(const c10::optional<at::Tensor>& t)
+{
+    return (t.has_value() && t->defined() && t->numel() > 0) ? t->data_ptr<float>() : nullptr;
+}
+
+struct Camera
+{
+    at::Tensor view, proj, campos, bg; // float32, contiguous, on the device: kept alive for the call
+    dsx_camera c;
+};
+
+Camera make_camera(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
+                   int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view, const at::Tensor& proj,
+                   const at::Tensor& campos, const at::Tensor& bg, const at::Device& dev)
+{
+    Camera cam;
+    auto prep = [&](const at::Tensor& t) { return t.to(dev, at::kFloat).contiguous(); };
+    cam.view = prep(view);
+    cam.proj = prep(proj);
+    cam.campos = prep(campos);
+    cam.bg = prep(bg);
+    TORCH_CHECK(cam.view.numel() == 16 && cam.proj.numel() == 16 && cam.campos.numel() >= 3 && cam.bg.numel() >= 3,
+                "camera tensors must be 4x4, 4x4, [3], [3]");
+    cam.c.image_height = (int32_t)height;
+    cam.c.image_width = (int32_t)width;
+    cam.c.tanfovx = (float)tanfovx;
+    cam.c.tanfovy = (float)tanfovy;
+    cam.c.scale_modifier = (float)scale_modifier;
+    cam.c.sh_degree = (int32_t)sh_degree;
+    cam.c.max_sh_degree = (int32_t)max_sh_degree;
+    cam.c.view = cam.view.data_ptr<float>();
+    cam.c.proj = cam.proj.data_ptr<float>();
+    cam.c.campos = cam.campos.data_ptr<float>();
+    cam.c.bg = cam.bg.data_ptr<float>();
+    return cam;
+}
+
+at::Tensor& pinned_key_count()
+{
+    // one pinned int64 per host thread: the landing place of the key count
+    thread_local at::Tensor slot = at::zeros({1}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
+    return slot;
+}
+
+} // namespace
+
+// image[H,W,3], radii[N], splats[N,12], cov3d[N,6], sorted_ids[K], ranges[T+1], final_T[H,W], final_idx[H,W]
+std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
+                                int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view,
+                                const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
+                                const at::Tensor& means3d, const c10::optional<at::Tensor>& scales,
+                                const c10::optional<at::Tensor>& quats, const at::Tensor& opacities,
+                                const c10::optional<at::Tensor>& shs, const c10::optional<at::Tensor>& cov3d_precomp,
+                                const c10::optional<at::Tensor>& colors_precomp, int64_t stream)
+{
+    const at::Device dev = means3d.device();
+    c10::DeviceGuard guard(dev);
+    Camera cam = make_camera(height, width, tanfovx, tanfovy, scale_modifier, sh_degree, max_sh_degree, view, proj,
+                             campos, bg, dev);
+    const int64_t n = means3d.numel() / 3;
+    const auto f32 = at::TensorOptions().dtype(at::kFloat).device(dev);
+    const auto i32 = at::TensorOptions().dtype(at::kInt).device(dev);
+    const auto u8 = at::TensorOptions().dtype(at::kByte).device(dev);
+    void* s = reinterpret_cast<void*>(stream);
+
+    at::Tensor splats = at::empty({n, DSX_SPLAT_FLOATS}, f32);
+    at::Tensor radii = at::empty({n}, i32);
+    at::Tensor cov3d = at::empty({n, 6}, f32);
+    at::Tensor block_sums = at::empty({dsx_num_blocks(n) + 1}, i32);
+    const size_t order_bytes = dsx_order_bytes(n);
+    at::Tensor order = at::empty({(int64_t)std::max<size_t>(order_bytes, 1)}, u8);
+    at::Tensor& k_host = pinned_key_count();
+    uint32_t* bs = reinterpret_cast<uint32_t*>(block_sums.data_ptr<int32_t>());
+    check(dsx_forward_project(&cam.c, n, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
+                              opacities.data_ptr<float>(), fptr(shs), fptr(cov3d_precomp), fptr(colors_precomp),
+                              splats.data_ptr<float>(), radii.data_ptr<int32_t>(), cov3d.data_ptr<float>(), bs,
+                              bs + dsx_num_blocks(n), order.data_ptr(), order_bytes, k_host.data_ptr<int64_t>(), s));
+    const int64_t k = *k_host.data_ptr<int64_t>();
+    const int64_t tiles = dsx_num_tiles((int32_t)width, (int32_t)height);
+    at::Tensor sorted_ids = at::empty({k}, i32);
+    at::Tensor ranges = at::empty({tiles + 1}, i32);
+    at::Tensor image = at::empty({height, width, 3}, f32);
+    at::Tensor final_T = at::empty({height, width}, f32);
+    at::Tensor final_idx = at::empty({height, width}, i32);
+    const size_t ws_bytes = dsx_workspace_bytes(n, k, (int32_t)width, (int32_t)height);
+    at::Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 1)}, u8);
+    check(dsx_forward_finish(&cam.c, n, k, splats.data_ptr<float>(), order.data_ptr(), sorted_ids.data_ptr<int32_t>(),
+                             ranges.data_ptr<int32_t>(), image.data_ptr<float>(), final_T.data_ptr<float>(),
+                             final_idx.data_ptr<int32_t>(), ws.data_ptr(), ws_bytes, s));
+    return {image, radii, splats, cov3d, sorted_ids, ranges, final_T, final_idx};
+}
+
+// v_mean3d[N,3], v_means2d[N,3], v_shs[N,B,3] (undefined when num_bases == 0), v_colors[N,3],
+// v_opacity[N,1], v_scale[N,3], v_quat[N,4], v_cov3d[N,6]
+std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
+                                 int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view,
+                                 const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
+                                 int64_t num_bases, const at::Tensor& means3d, const c10::optional<at::Tensor>& scales,
+                                 const c10::optional<at::Tensor>& quats, const at::Tensor& splats,
+                                 const at::Tensor& cov3d, const at::Tensor& radii, const at::Tensor& ranges,
+                                 const at::Tensor& sorted_ids, const at::Tensor& final_T, const at::Tensor& final_idx,
+                                 const at::Tensor& v_image, int64_t stream)
+{
+    const at::Device dev = means3d.device();
+    c10::DeviceGuard guard(dev);
+    Camera cam = make_camera(height, width, tanfovx, tanfovy, scale_modifier, sh_degree, max_sh_degree, view, proj,
+                             campos, bg, dev);
+    const int64_t n = means3d.numel() / 3;
+    const auto f32 = at::TensorOptions().dtype(at::kFloat).device(dev);
+    TORCH_CHECK(v_image.is_contiguous() && v_image.scalar_type() == at::kFloat && v_image.numel() == height * width * 3,
+                "v_image must be a contiguous float32 [H, W, 3] tensor");
+    at::Tensor v_mean3d = at::empty({n, 3}, f32), v_means2d = at::empty({n, 3}, f32);
+    at::Tensor v_shs = num_bases > 0 ? at::empty({n, num_bases, 3}, f32) : at::Tensor();
+    at::Tensor v_colors = at::empty({n, 3}, f32), v_opacity = at::empty({n, 1}, f32);
+    at::Tensor v_scale = at::empty({n, 3}, f32), v_quat = at::empty({n, 4}, f32), v_cov3d = at::empty({n, 6}, f32);
+    at::Tensor grads = at::empty({n, DSX_GRAD_FLOATS}, f32);
+    check(dsx_backward(&cam.c, n, (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
+                       splats.data_ptr<float>(), cov3d.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                       ranges.data_ptr<int32_t>(), sorted_ids.numel() ? sorted_ids.data_ptr<int32_t>() : nullptr,
+                       final_T.data_ptr<float>(), final_idx.data_ptr<int32_t>(), v_image.data_ptr<float>(),
+                       grads.data_ptr<float>(), v_mean3d.data_ptr<float>(), v_means2d.data_ptr<float>(),
+                       num_bases > 0 ? v_shs.data_ptr<float>() : nullptr, v_colors.data_ptr<float>(),
+                       v_opacity.data_ptr<float>(), v_scale.data_ptr<float>(), v_quat.data_ptr<float>(),
+                       v_cov3d.data_ptr<float>(), reinterpret_cast<void*>(stream)));
+    return {v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d};
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.doc() = "torch binding of libdsx (gfx950 3D-Gaussian-Splatting rasterizer)";
+    m.def("forward", &forward, "projection, tile lists and blend; returns the tensors the backward needs");
+    m.def("backward", &backward, "blend backward and per-Gaussian backward");
+    m.def("version", []() { return dsx_version(); });
+}

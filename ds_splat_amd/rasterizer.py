@@ -14,6 +14,7 @@ from dataclasses import dataclass
 
 import torch
 
+from . import _native
 from . import stages
 
 
@@ -77,40 +78,45 @@ def _num_bases(shs):
 
 
 class DsRasterizerFunction(torch.autograd.Function):
+    """Forward and backward through the C++ torch binding (csrc/torch_ext.cpp), which allocates the
+    outputs and calls the C ABI of libdsx.so on the current stream."""
+
     @staticmethod
     def forward(ctx, means_3d, means_2d, shs, colors_precomp, opacities, scales, rotations, cov_3d_precomp,
                 raster_settings):
         s = raster_settings
         _validate(means_3d, means_2d, shs, colors_precomp, opacities, scales, rotations, cov_3d_precomp, s)
-        with torch.cuda.device(means_3d.device):
-            cam = stages.CameraArgs(s.image_height, s.image_width, s.tanfovx, s.tanfovy, s.bg, s.scale_modifier,
-                                    s.view_matrix, s.proj_matrix, s.sh_degree, s.max_sh_degree, s.campos)
-            opt = lambda t: t if t.numel() > 0 else None
-            image, st = stages.forward(cam, means_3d, opt(scales), opt(rotations), opacities, opt(shs),
-                                       opt(cov_3d_precomp), opt(colors_precomp))
+        ext = _native.load_torch_ext()
+        opt = lambda t: t if t.numel() > 0 else None
+        stream = torch.cuda.current_stream(means_3d.device).cuda_stream
+        cam = (int(s.image_height), int(s.image_width), float(s.tanfovx), float(s.tanfovy), float(s.scale_modifier),
+               int(s.sh_degree), int(s.max_sh_degree), s.view_matrix, s.proj_matrix, s.campos, s.bg)
+        image, radii, splats, cov3d, sorted_ids, ranges, final_T, final_idx = ext.forward(
+            *cam, means_3d, opt(scales), opt(rotations), opacities, opt(shs), opt(cov_3d_precomp), opt(colors_precomp),
+            stream)
         ctx.cam = cam
-        ctx.state = st
         ctx.num_bases = _num_bases(shs) if shs.numel() > 0 else 0
         ctx.opacity_shape = opacities.shape
-        ctx.save_for_backward(means_3d, scales, rotations)
-        ctx.mark_non_differentiable(st.radii)
-        return image, st.radii
+        ctx.num_keys = sorted_ids.numel()
+        ctx.save_for_backward(means_3d, scales, rotations, splats, cov3d, radii, ranges, sorted_ids, final_T, final_idx)
+        ctx.mark_non_differentiable(radii)
+        return image, radii
 
     @staticmethod
     def backward(ctx, rendered_img_grad, _):
-        means_3d, scales, rotations = ctx.saved_tensors
-        st, cam = ctx.state, ctx.cam
+        means_3d, scales, rotations, splats, cov3d, radii, ranges, sorted_ids, final_T, final_idx = ctx.saved_tensors
+        ext = _native.load_torch_ext()
         opt = lambda t: t if t.numel() > 0 else None
-        with torch.cuda.device(means_3d.device):
-            g = stages.backward(cam, st, ctx.num_bases, means_3d, opt(scales), opt(rotations),
-                                rendered_img_grad.contiguous())
-        v_opacity = g["v_opacity"]
+        stream = torch.cuda.current_stream(means_3d.device).cuda_stream
+        v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d = ext.backward(
+            *ctx.cam, ctx.num_bases, means_3d, opt(scales), opt(rotations), splats, cov3d, radii, ranges, sorted_ids,
+            final_T, final_idx, rendered_img_grad.contiguous(), stream)
         if tuple(ctx.opacity_shape) != tuple(v_opacity.shape):
             v_opacity = v_opacity.reshape(ctx.opacity_shape)
         needs = ctx.needs_input_grad
         pick = lambda i, t: t if needs[i] else None
-        return (pick(0, g["v_mean3d"]), pick(1, g["v_means2d"]), pick(2, g["v_shs"]), pick(3, g["v_colors"]),
-                pick(4, v_opacity), pick(5, g["v_scale"]), pick(6, g["v_quat"]), pick(7, g["v_cov3d"]), None)
+        return (pick(0, v_mean3d), pick(1, v_means2d), pick(2, v_shs), pick(3, v_colors), pick(4, v_opacity),
+                pick(5, v_scale), pick(6, v_quat), pick(7, v_cov3d), None)
 
 
 @dataclass
@@ -141,9 +147,23 @@ class GaussianRasterizer(torch.nn.Module):
     def __init__(self, raster_settings: GaussianRasterizationSettings):
         super().__init__()
         self._settings = raster_settings
+        self._native_cache = None
 
     @property
     def settings_for_cpp_code(self):
+        # the reference transposes both matrices on every call (ds_splat/rasterizer.py:147-148);
+        # the result is kept here for as long as the settings' tensors are the same, unmodified ones
+        rs = self._settings
+        key = (id(rs), id(rs.viewmatrix), rs.viewmatrix._version, id(rs.projmatrix), rs.projmatrix._version,
+               id(rs.bg), id(rs.campos), rs.image_height, rs.image_width, rs.tanfovx, rs.tanfovy, rs.scale_modifier,
+               rs.sh_degree, rs.max_sh_degree)
+        if self._native_cache is not None and self._native_cache[0] == key:
+            return self._native_cache[1]
+        s = self._build_native_settings()
+        self._native_cache = (key, s)
+        return s
+
+    def _build_native_settings(self):
         s = _NativeSettings()
         s.image_height = self._settings.image_height
         s.image_width = self._settings.image_width

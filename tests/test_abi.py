@@ -26,6 +26,13 @@ def test_library_exports_every_declared_symbol():
         assert getattr(lib, name) is not None
 
 
+def test_torch_binding_loads_and_links_the_library():
+    from ds_splat_amd import _native
+    ext = _native.load_torch_ext()
+    assert ext.version() == _native.load().dsx_version()
+    assert callable(ext.forward) and callable(ext.backward)
+
+
 def test_host_helpers():
     from ds_splat_amd import _native
     lib = _native.load()
