@@ -4,7 +4,9 @@
 // spherical-harmonics rows of its 64 Gaussians (a contiguous 12 KB span at degree 3) into LDS
 // with 16-byte coalesced loads and then every lane reads its own row back with an odd LDS
 // pitch (conflict free), so the 192-byte AoS rows never produce strided HBM traffic; only
-// the columns the active degree needs are fetched.
+// the columns the active degree needs are fetched, and only the rows of Gaussians whose centre
+// passes the frustum test.  The rows go through LDS in two parts (degrees 0-2, then degree 3)
+// so that a workgroup holds 30 KB instead of 50 KB and five workgroups fit a compute unit.
 //
 // This translation unit is compiled with floating-point contraction OFF and uses only
 // + - * / sqrt on binary32: radii, tile counts and depth keys are integers derived from these
@@ -18,7 +20,10 @@
 namespace dsx
 {
 
-constexpr int kShPitch = 49; // floats per row in LDS (48 coefficients, odd pitch)
+// Rows pass through LDS in two parts: floats 0..27 (degrees 0-2 need 0..26; float 27, the
+// first of degree 3, rides along because it shares a 16-byte chunk) and floats 28..47.
+constexpr int kShLowFloats = 28;
+constexpr int kShPitch = 29; // floats per row in LDS (odd pitch: conflict-free row reads)
 
 struct ProjectParams
 {
@@ -74,19 +79,34 @@ __device__ __forceinline__ void cov3d_from_scale_rot(const float* sc, float4 q, 
     out[5] = m20 * m20 + m21 * m21 + m22 * m22;
 }
 
-// SH degree 0..3 -> RGB (+0.5, clamped at 0); f = this Gaussian's coefficient row in LDS.
-// Term order as cpp/rasterizer_kernels.cu:433-554.
-__device__ __forceinline__ float3 sh_to_rgb(int deg, const float* f, float3 mean, float3 cam)
+// SH degree 0..3 -> RGB (+0.5, clamped at 0), term order as cpp/rasterizer_kernels.cu:433-554,
+// in two steps that add to the same accumulators in the reference's order: degrees 0-2 from
+// floats 0..26 of the row, then degree 3 from float 27 (f27) and floats 28..47 (g[0..19]).
+struct ShDir
+{
+    float vx, vy, vz;
+};
+
+__device__ __forceinline__ ShDir sh_direction(float3 mean, float3 cam)
+{
+    const float dx = mean.x - cam.x, dy = mean.y - cam.y, dz = mean.z - cam.z;
+    const float inv_norm = 1.0f / sqrtf(dx * dx + dy * dy + dz * dz);
+    ShDir d;
+    d.vx = dx * inv_norm;
+    d.vy = dy * inv_norm;
+    d.vz = dz * inv_norm;
+    return d;
+}
+
+__device__ __forceinline__ void sh_low(int deg, const float* f, ShDir d, float& rx, float& ry, float& rz)
 {
     const float C0 = 0.28209479177387814f;
-    float rx = 0.0f + C0 * f[0];
-    float ry = 0.0f + C0 * f[1];
-    float rz = 0.0f + C0 * f[2];
+    rx = 0.0f + C0 * f[0];
+    ry = 0.0f + C0 * f[1];
+    rz = 0.0f + C0 * f[2];
     if(deg >= 1)
     {
-        const float dx = mean.x - cam.x, dy = mean.y - cam.y, dz = mean.z - cam.z;
-        const float inv_norm = 1.0f / sqrtf(dx * dx + dy * dy + dz * dz);
-        const float vx = dx * inv_norm, vy = dy * inv_norm, vz = dz * inv_norm;
+        const float vx = d.vx, vy = d.vy, vz = d.vz;
         const float C1 = 0.4886025119029199f;
         rx += C1 * (-vy * f[3] + vz * f[6] - vx * f[9]);
         ry += C1 * (-vy * f[4] + vz * f[7] - vx * f[10]);
@@ -101,25 +121,88 @@ __device__ __forceinline__ float3 sh_to_rgb(int deg, const float* f, float3 mean
             rx += A0 * xy * f[12] + A1 * yz * f[15] + A2 * q2 * f[18] + A3 * xz * f[21] + A4 * q4 * f[24];
             ry += A0 * xy * f[13] + A1 * yz * f[16] + A2 * q2 * f[19] + A3 * xz * f[22] + A4 * q4 * f[25];
             rz += A0 * xy * f[14] + A1 * yz * f[17] + A2 * q2 * f[20] + A3 * xz * f[23] + A4 * q4 * f[26];
-            if(deg >= 3)
+        }
+    }
+}
+
+// g[j] = float 28 + j of the row
+__device__ __forceinline__ void sh_high(float f27, const float* g, ShDir d, float& rx, float& ry, float& rz)
+{
+    const float vx = d.vx, vy = d.vy, vz = d.vz;
+    const float xx = vx * vx, yy = vy * vy, zz = vz * vz;
+    const float xy = vx * vy;
+    const float B0 = -0.5900435899266435f, B1 = 2.890611442640554f, B2 = -0.4570457994644658f,
+                B3 = 0.3731763325901154f, B4 = -0.4570457994644658f, B5 = 1.445305721320277f,
+                B6 = -0.5900435899266435f;
+    const float t0 = B0 * vy * (3.0f * xx - yy);
+    const float t1 = B1 * xy * vz;
+    const float t2 = B2 * vy * (4.0f * zz - xx - yy);
+    const float t3 = B3 * vz * (2.0f * zz - 3.0f * xx - 3.0f * yy);
+    const float t4 = B4 * vx * (4.0f * zz - xx - yy);
+    const float t5 = B5 * vz * (xx - yy);
+    const float t6 = B6 * vx * (xx - 3.0f * yy);
+    rx += t0 * f27 + t1 * g[2] + t2 * g[5] + t3 * g[8] + t4 * g[11] + t5 * g[14] + t6 * g[17];
+    ry += t0 * g[0] + t1 * g[3] + t2 * g[6] + t3 * g[9] + t4 * g[12] + t5 * g[15] + t6 * g[18];
+    rz += t0 * g[1] + t1 * g[4] + t2 * g[7] + t3 * g[10] + t4 * g[13] + t5 * g[16] + t6 * g[19];
+}
+
+// Copies columns [c_begin, c_end) of the wavefront's wanted SH rows into LDS at dst[row * kShPitch
+// + (c - c_begin)].  Fast path: 16-byte chunks of 192-byte rows; c_begin and c_end are
+// multiples of 4 there.
+template <int kMaxChunksPerLane>
+__device__ __forceinline__ void stage_sh_columns(const ProjectParams& p, int64_t row0, int rows, uint64_t wanted_rows,
+                                                 int c_begin, int c_end, int lane, float* dst)
+{
+    if(c_end <= c_begin)
+        return;
+    if(p.sh_stride == 48 && ((uintptr_t)p.shs & 15) == 0)
+    {
+        const float4* src = reinterpret_cast<const float4*>(p.shs + row0 * 48);
+        const int q0 = c_begin >> 2;
+        const int per_row = ((c_end + 3) >> 2) - q0; // 16-byte chunks per row in this part
+        const int chunks = rows * per_row;
+        // all loads are issued before the first LDS write, so their latencies overlap
+        float4 v[kMaxChunksPerLane];
+        int at[kMaxChunksPerLane];
+#pragma unroll
+        for(int it = 0; it < kMaxChunksPerLane; ++it)
+        {
+            const int e = it * 64 + lane;
+            const int row = e / per_row;
+            const int c4 = e - row * per_row;
+            at[it] = -1;
+            if(e < chunks && ((wanted_rows >> row) & 1))
             {
-                const float B0 = -0.5900435899266435f, B1 = 2.890611442640554f, B2 = -0.4570457994644658f,
-                            B3 = 0.3731763325901154f, B4 = -0.4570457994644658f, B5 = 1.445305721320277f,
-                            B6 = -0.5900435899266435f;
-                const float t0 = B0 * vy * (3.0f * xx - yy);
-                const float t1 = B1 * xy * vz;
-                const float t2 = B2 * vy * (4.0f * zz - xx - yy);
-                const float t3 = B3 * vz * (2.0f * zz - 3.0f * xx - 3.0f * yy);
-                const float t4 = B4 * vx * (4.0f * zz - xx - yy);
-                const float t5 = B5 * vz * (xx - yy);
-                const float t6 = B6 * vx * (xx - 3.0f * yy);
-                rx += t0 * f[27] + t1 * f[30] + t2 * f[33] + t3 * f[36] + t4 * f[39] + t5 * f[42] + t6 * f[45];
-                ry += t0 * f[28] + t1 * f[31] + t2 * f[34] + t3 * f[37] + t4 * f[40] + t5 * f[43] + t6 * f[46];
-                rz += t0 * f[29] + t1 * f[32] + t2 * f[35] + t3 * f[38] + t4 * f[41] + t5 * f[44] + t6 * f[47];
+                v[it] = nt_load_f4(src + row * 12 + q0 + c4);
+                at[it] = row * kShPitch + c4 * 4;
+            }
+        }
+#pragma unroll
+        for(int it = 0; it < kMaxChunksPerLane; ++it)
+        {
+            if(at[it] >= 0)
+            {
+                float* d = dst + at[it];
+                d[0] = v[it].x;
+                d[1] = v[it].y;
+                d[2] = v[it].z;
+                d[3] = v[it].w;
             }
         }
     }
-    return make_float3(fmaxf(rx + 0.5f, 0.0f), fmaxf(ry + 0.5f, 0.0f), fmaxf(rz + 0.5f, 0.0f));
+    else
+    {
+        const float* src = p.shs + row0 * p.sh_stride;
+        const int width = c_end - c_begin;
+        const int total = rows * width;
+        for(int e = lane; e < total; e += 64)
+        {
+            const int row = e / width;
+            const int c = e - row * width;
+            if((wanted_rows >> row) & 1)
+                dst[row * kShPitch + c] = src[(int64_t)row * p.sh_stride + c_begin + c];
+        }
+    }
 }
 
 __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectParams p)
@@ -133,56 +216,77 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
     const int64_t i = (int64_t)blockIdx.x * kProjBlock + tid;
     const bool live = i < p.n;
 
-    // ---- stage this wavefront's SH rows through LDS (coalesced) -----------------------------
+    // frustum test on the centre: strict NDC box, z_ndc > 0.1 (cpp/rasterizer_kernels.cu:7-24).
+    // It comes first because a Gaussian that fails it is culled whatever its shape is, nothing
+    // downstream reads its colour, and so its SH row (the largest input) is never fetched.
+    float3 mean = make_float3(0.f, 0.f, 0.f);
+    bool in_frustum = false;
+    if(live)
+    {
+        mean = make_float3(p.means3d[3 * i], p.means3d[3 * i + 1], p.means3d[3 * i + 2]);
+        const float* P = p.proj;
+        const float inv_w = 1.0f / (P[12] * mean.x + P[13] * mean.y + P[14] * mean.z + P[15]);
+        const float nx = inv_w * (P[0] * mean.x + P[1] * mean.y + P[2] * mean.z + P[3]);
+        const float ny = inv_w * (P[4] * mean.x + P[5] * mean.y + P[6] * mean.z + P[7]);
+        const float nz = inv_w * (P[8] * mean.x + P[9] * mean.y + P[10] * mean.z + P[11]);
+        in_frustum = nx > -1.0f && nx < 1.0f && ny > -1.0f && ny < 1.0f && nz > 0.1f;
+    }
+    const uint64_t wanted_rows = __ballot(in_frustum); // bit r: lane r of this wavefront needs its SH row
+
+    // ---- colours: this wavefront's SH rows through LDS, degrees 0-2 first, then degree 3 -------
+    // (each wavefront owns its part of the LDS array, so wavefront-local ordering is enough)
     const bool use_sh = p.colors_precomp == nullptr;
+    float3 rgb = make_float3(0.f, 0.f, 0.f);
     if(use_sh)
     {
         const int64_t row0 = (int64_t)blockIdx.x * kProjBlock + wave * 64;
         const int rows = (int)max((int64_t)0, min((int64_t)64, p.n - row0));
         const int need = (p.sh_degree + 1) * (p.sh_degree + 1) * 3; // floats per row actually used
         float* dst = sh_lds[wave];
-        if(p.sh_stride == 48 && ((uintptr_t)p.shs & 15) == 0)
+        const float* row = dst + lane * kShPitch;
+        stage_sh_columns<7>(p, row0, rows, wanted_rows, 0, min(need, kShLowFloats), lane, dst);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        float rx = 0.f, ry = 0.f, rz = 0.f, f27 = 0.f;
+        ShDir dir = {0.f, 0.f, 0.f};
+        if(in_frustum)
         {
-            const float4* src = reinterpret_cast<const float4*>(p.shs + row0 * 48);
-            const int chunks = rows * 12;
-            const int need4 = (need + 3) >> 2;
+            float f[27];
+            const int low = min(need, 27);
 #pragma unroll
-            for(int j = 0; j < 12; ++j)
-            {
-                const int e = j * 64 + lane;
-                const int row = e / 12;
-                const int c4 = e - row * 12;
-                if(e < chunks && c4 < need4)
-                {
-                    const float4 v = nt_load_f4(src + e);
-                    float* d = dst + row * kShPitch + c4 * 4;
-                    d[0] = v.x;
-                    d[1] = v.y;
-                    d[2] = v.z;
-                    d[3] = v.w;
-                }
-            }
+            for(int j = 0; j < 27; ++j)
+                f[j] = j < low ? row[j] : 0.0f;
+            f27 = row[27];
+            if(p.sh_degree >= 1)
+                dir = sh_direction(mean, make_float3(p.campos[0], p.campos[1], p.campos[2]));
+            sh_low(p.sh_degree, f, dir, rx, ry, rz);
         }
-        else
+        if(p.sh_degree >= 3)
         {
-            const float* src = p.shs + row0 * p.sh_stride;
-            const int total = rows * p.sh_stride;
-            for(int e = lane; e < total; e += 64)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            stage_sh_columns<5>(p, row0, rows, wanted_rows, kShLowFloats, 48, lane, dst);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if(in_frustum)
             {
-                const int row = e / p.sh_stride;
-                const int c = e - row * p.sh_stride;
-                if(c < need)
-                    dst[row * kShPitch + c] = src[e];
+                float g[20];
+#pragma unroll
+                for(int j = 0; j < 20; ++j)
+                    g[j] = row[j];
+                sh_high(f27, g, dir, rx, ry, rz);
             }
         }
+        if(in_frustum)
+            rgb = make_float3(fmaxf(rx + 0.5f, 0.0f), fmaxf(ry + 0.5f, 0.0f), fmaxf(rz + 0.5f, 0.0f));
     }
-    __syncthreads();
 
     uint32_t count = 0;
     if(live)
     {
-        const float3 mean = make_float3(p.means3d[3 * i], p.means3d[3 * i + 1], p.means3d[3 * i + 2]);
-
         float c3[6];
         if(p.cov3d_precomp)
         {
@@ -203,30 +307,8 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
             o[2] = make_float2(c3[4], c3[5]);
         }
 
-        float3 rgb;
-        if(use_sh)
-        {
-            float f[48];
-            const float* row = sh_lds[wave] + lane * kShPitch;
-            const int need = (p.sh_degree + 1) * (p.sh_degree + 1) * 3;
-#pragma unroll
-            for(int j = 0; j < 48; ++j)
-                f[j] = j < need ? row[j] : 0.0f;
-            const float3 cam = make_float3(p.campos[0], p.campos[1], p.campos[2]);
-            rgb = sh_to_rgb(p.sh_degree, f, mean, cam);
-        }
-        else
-        {
+        if(!use_sh)
             rgb = make_float3(p.colors_precomp[3 * i], p.colors_precomp[3 * i + 1], p.colors_precomp[3 * i + 2]);
-        }
-
-        // frustum test on the centre: strict NDC box, z_ndc > 0.1 (cpp/rasterizer_kernels.cu:7-24)
-        const float* P = p.proj;
-        const float inv_w = 1.0f / (P[12] * mean.x + P[13] * mean.y + P[14] * mean.z + P[15]);
-        const float nx = inv_w * (P[0] * mean.x + P[1] * mean.y + P[2] * mean.z + P[3]);
-        const float ny = inv_w * (P[4] * mean.x + P[5] * mean.y + P[6] * mean.z + P[7]);
-        const float nz = inv_w * (P[8] * mean.x + P[9] * mean.y + P[10] * mean.z + P[11]);
-        const bool in_frustum = nx > -1.0f && nx < 1.0f && ny > -1.0f && ny < 1.0f && nz > 0.1f;
 
         // view-space position (cpp/rasterizer_kernels.cu:325-330)
         const float* V = p.view;
