@@ -148,12 +148,14 @@ static_assert(kDepthSortThreads >= kBins32 && kListSortThreads >= kBins32, "one 
 static_assert(kDepthSortTile <= 65535 && kListSortTile <= 65535, "u16 ranks");
 
 // vals_in == nullptr: the values are the input positions (iota).  keys_out == nullptr: the
-// keys are not needed after this pass.  KeyT: uint32_t, or uint16_t for tile slots that fit.
+// keys are not needed after this pass.  gather_src != nullptr: gather_dst[position] =
+// gather_src[value] for every pair.  KeyT: uint32_t, or uint16_t for tile slots that fit.
 template <typename KeyT, int kSort32Threads, int kSort32Items>
 __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     const KeyT* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, KeyT* __restrict__ keys_out,
     uint32_t* __restrict__ vals_out, int64_t count, int shift, uint32_t mask, const uint32_t* __restrict__ hist_excl,
-    uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag)
+    uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag, const uint2* __restrict__ gather_src,
+    uint2* __restrict__ gather_dst)
 {
     constexpr int kSort32Tile = kSort32Threads * kSort32Items;
     constexpr int kSort32Waves = kSort32Threads / DSX_WAVE;
@@ -261,11 +263,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     if(digit_thread)
     {
         uint32_t excl = 0;
-#ifdef EXP_NOLOOK
-        if(false)
-#else
         if(tile > 0 && (uint32_t)tid <= mask) // bins above the mask are empty in every tile
-#endif
         {
             int64_t t = tile - 1; // next predecessor to account for
             int spins = 0;
@@ -340,7 +338,14 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     {
         const int j = it * kSort32Threads + tid;
         if(j < tile_n)
-            vals_out[out[it]] = s_keys[j];
+        {
+            const uint32_t v = s_keys[j];
+            vals_out[out[it]] = v;
+            // optional: a per-value record follows its value to the sorted position (the random
+            // gather overlaps with the scatter traffic of the pass)
+            if(gather_src)
+                gather_dst[out[it]] = gather_src[v];
+        }
     }
 }
 
@@ -375,7 +380,8 @@ static int sort32_clear(int64_t count, int key_bits, int tile_keys, void* sort_w
 template <typename KeyT, int kThreads, int kItems>
 static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* vals_a, KeyT* keys_b, uint32_t* vals_b,
                          bool iota_values, bool keep_keys, void* sort_ws, const char* label, hipStream_t stream,
-                         KeyT** keys_out, uint32_t** vals_out)
+                         KeyT** keys_out, uint32_t** vals_out, const uint2* gather_src = nullptr,
+                         uint2* gather_dst = nullptr)
 {
     const Sort32Workspace w = sort32_workspace(count, key_bits, kThreads * kItems);
     const Digits32 plan = digits32(key_bits);
@@ -401,7 +407,8 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
                                (const KeyT*)kin, (const uint32_t*)((p == 0 && iota_values) ? nullptr : vin),
                                (last && !keep_keys) ? (KeyT*)nullptr : kout, vout, count, plan.shift[p], plan.mask[p],
                                (const uint32_t*)(hist + p * kBins32), status + (size_t)p * w.tiles * kBins32,
-                               counters + p, counters + w.passes);
+                               counters + p, counters + w.passes, last ? gather_src : (const uint2*)nullptr,
+                               last ? gather_dst : (uint2*)nullptr);
         }
         DSX_LAUNCH_CHECK();
         KeyT* tk = kin;
@@ -419,7 +426,7 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
 // Stable ascending sort of `count` (key, value) pairs by the low key_bits bits of the key.
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
-                  uint32_t** keys_out, uint32_t** vals_out)
+                  uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src, uint2* gather_dst)
 {
     *keys_out = keys_a;
     *vals_out = vals_a;
@@ -440,7 +447,7 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
     }
     DSX_LAUNCH_CHECK();
     return sort32_passes<uint32_t, kDepthSortThreads, kDepthSortItems>(count, key_bits, keys_a, vals_a, keys_b, vals_b, iota_values, keep_keys, sort_ws,
-                                   "onesweep32_kernel<sort>", stream, keys_out, vals_out);
+                                   "onesweep32_kernel<sort>", stream, keys_out, vals_out, gather_src, gather_dst);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -477,24 +484,17 @@ __device__ __forceinline__ uint32_t rect_count(uint2 r)
     return (r.y & 0xffffu) * ((r.y >> 16) & 0x7fffu);
 }
 
-// Tile count of each run of 256 Gaussians taken in depth order.  This is the one random
-// gather of the per-Gaussian rectangles; they are stored again in depth order so that the
-// emission reads them in sequence.
-__global__ __launch_bounds__(kProjBlock) void ordered_block_sums_kernel(const uint32_t* __restrict__ order,
-                                                                       const uint2* __restrict__ rects, int64_t n,
-                                                                       uint2* __restrict__ rects_sorted,
-                                                                       uint32_t* __restrict__ block_sums)
+// Tile count of each run of 256 Gaussians taken in depth order (the last pass of the depth sort
+// has already put the rectangles into that order).
+__global__ __launch_bounds__(kProjBlock) void ordered_block_sums_kernel(const uint2* __restrict__ rects_sorted,
+                                                                       int64_t n, uint32_t* __restrict__ block_sums)
 {
     __shared__ uint32_t wave_sums[kProjBlock / DSX_WAVE];
     const int tid = threadIdx.x;
     const int64_t p = (int64_t)blockIdx.x * kProjBlock + tid;
     uint32_t count = 0;
     if(p < n)
-    {
-        const uint2 r = rects[order[p]];
-        rects_sorted[p] = r;
-        count = rect_count(r);
-    }
+        count = rect_count(rects_sorted[p]);
     const uint32_t ws = wave_sum_u32(count);
     if((tid & 63) == 0)
         wave_sums[tid >> 6] = ws;
@@ -517,18 +517,18 @@ int launch_depth_order(int64_t n, void* order, hipStream_t stream)
     uint32_t* block_sums = reinterpret_cast<uint32_t*>(base + o.block_sums);
     uint32_t *ko, *vo;
     // 32 key bits = 4 passes: the values (iota in pass 0) go b, a, b, a and end in ids_a
-    int rc = launch_sort32(n, 32, keys_a, ids_a, keys_b, ids_b, true, false, base + o.sort, stream, &ko, &vo);
+    int rc = launch_sort32(n, 32, keys_a, ids_a, keys_b, ids_b, true, false, base + o.sort, stream, &ko, &vo,
+                           reinterpret_cast<const uint2*>(base + o.rects),
+                           reinterpret_cast<uint2*>(base + o.rects_sorted));
     if(rc)
         return rc;
     if(vo != ids_a)
         return DSX_ERR_RUNTIME;
-    const uint32_t* perm = vo;
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     {
         DSX_TIMED("ordered_block_sums_kernel", stream);
-        hipLaunchKernelGGL(ordered_block_sums_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, perm,
-                           reinterpret_cast<const uint2*>(base + o.rects), n,
-                           reinterpret_cast<uint2*>(base + o.rects_sorted), block_sums);
+        hipLaunchKernelGGL(ordered_block_sums_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
+                           reinterpret_cast<const uint2*>(base + o.rects_sorted), n, block_sums);
     }
     DSX_LAUNCH_CHECK();
     return launch_scan_u32(blocks, block_sums, block_sums + blocks, stream);
