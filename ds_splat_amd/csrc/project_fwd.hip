@@ -5,8 +5,9 @@
 // with 16-byte coalesced loads and then every lane reads its own row back with an odd LDS
 // pitch (conflict free), so the 192-byte AoS rows never produce strided HBM traffic; only
 // the columns the active degree needs are fetched, and only the rows of Gaussians whose centre
-// passes the frustum test.  The rows go through LDS in two parts (degrees 0-2, then degree 3)
-// so that a workgroup holds 30 KB instead of 50 KB and five workgroups fit a compute unit.
+// passes the frustum test.  The rows go through LDS in three parts of 16 floats (one 64-byte
+// sector of each 192-byte row at a time, so every sector is fetched exactly once) and a
+// workgroup holds 17 KB of LDS instead of 50 KB: occupancy is no longer bound by LDS.
 //
 // This translation unit is compiled with floating-point contraction OFF and uses only
 // + - * / sqrt on binary32: radii, tile counts and depth keys are integers derived from these
@@ -20,10 +21,9 @@
 namespace dsx
 {
 
-// Rows pass through LDS in two parts: floats 0..27 (degrees 0-2 need 0..26; float 27, the
-// first of degree 3, rides along because it shares a 16-byte chunk) and floats 28..47.
-constexpr int kShLowFloats = 28;
-constexpr int kShPitch = 29; // floats per row in LDS (odd pitch: conflict-free row reads)
+// Rows pass through LDS in three parts of 16 floats (64 bytes, one sector of the row).
+constexpr int kShPart = 16;
+constexpr int kShPitch = 17; // floats per row in LDS (odd pitch: conflict-free row reads)
 
 struct ProjectParams
 {
@@ -173,7 +173,7 @@ __device__ __forceinline__ void stage_sh_columns(const ProjectParams& p, int64_t
             at[it] = -1;
             if(e < chunks && ((wanted_rows >> row) & 1))
             {
-                v[it] = nt_load_f4(src + row * 12 + q0 + c4);
+                v[it] = src[row * 12 + q0 + c4]; // cached load: the other sectors of the line follow in the next parts
                 at[it] = row * kShPitch + c4 * 4;
             }
         }
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
     }
     const uint64_t wanted_rows = __ballot(in_frustum); // bit r: lane r of this wavefront needs its SH row
 
-    // ---- colours: this wavefront's SH rows through LDS, degrees 0-2 first, then degree 3 -------
+    // ---- colours: this wavefront's SH rows through LDS, one 64-byte sector of each row at a time ---
     // (each wavefront owns its part of the LDS array, so wavefront-local ordering is enough)
     const bool use_sh = p.colors_precomp == nullptr;
     float3 rgb = make_float3(0.f, 0.f, 0.f);
@@ -244,41 +244,38 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
         const int need = (p.sh_degree + 1) * (p.sh_degree + 1) * 3; // floats per row actually used
         float* dst = sh_lds[wave];
         const float* row = dst + lane * kShPitch;
-        stage_sh_columns<7>(p, row0, rows, wanted_rows, 0, min(need, kShLowFloats), lane, dst);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        float rx = 0.f, ry = 0.f, rz = 0.f, f27 = 0.f;
-        ShDir dir = {0.f, 0.f, 0.f};
+        float rx = 0.f, ry = 0.f, rz = 0.f;
+        float f[48]; // the row, collected part by part (registers of parts already used are dead)
+#pragma unroll
+        for(int part = 0; part < 3; ++part)
+        {
+            const int c0 = part * kShPart;
+            if(c0 < need) // uniform
+            {
+                if(part > 0)
+                {
+                    // the wavefront's reads of the previous part are done before it is overwritten
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                }
+                stage_sh_columns<4>(p, row0, rows, wanted_rows, c0, min(need, c0 + kShPart), lane, dst);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            }
+#pragma unroll
+            for(int j = 0; j < kShPart; ++j)
+                f[c0 + j] = (in_frustum && c0 + j < need) ? row[j] : 0.0f;
+        }
         if(in_frustum)
         {
-            float f[27];
-            const int low = min(need, 27);
-#pragma unroll
-            for(int j = 0; j < 27; ++j)
-                f[j] = j < low ? row[j] : 0.0f;
-            f27 = row[27];
+            ShDir dir = {0.f, 0.f, 0.f};
             if(p.sh_degree >= 1)
                 dir = sh_direction(mean, make_float3(p.campos[0], p.campos[1], p.campos[2]));
             sh_low(p.sh_degree, f, dir, rx, ry, rz);
-        }
-        if(p.sh_degree >= 3)
-        {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            stage_sh_columns<5>(p, row0, rows, wanted_rows, kShLowFloats, 48, lane, dst);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            if(in_frustum)
-            {
-                float g[20];
-#pragma unroll
-                for(int j = 0; j < 20; ++j)
-                    g[j] = row[j];
-                sh_high(f27, g, dir, rx, ry, rz);
-            }
+            if(p.sh_degree >= 3)
+                sh_high(f[27], f + 28, dir, rx, ry, rz);
         }
         if(in_frustum)
             rgb = make_float3(fmaxf(rx + 0.5f, 0.0f), fmaxf(ry + 0.5f, 0.0f), fmaxf(rz + 0.5f, 0.0f));
