@@ -48,14 +48,14 @@ SIGNATURES = {
     "dsx_workspace_bytes": (C.c_size_t, [_I64, _I64, _I32, _I32]),
     "dsx_sort_workspace_bytes": (C.c_size_t, [_I64, _I32]),
     "dsx_sort_u32_workspace_bytes": (C.c_size_t, [_I64, _I32]),
-    "dsx_order_bytes": (C.c_size_t, [_I64]),
+    "dsx_order_bytes": (C.c_size_t, [_I64, _I32, _I32]),
     "dsx_project_fwd": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P] * 4 + [_P, C.c_size_t, _P]),
     "dsx_scan_u32": (C.c_int, [_I64, _P, _P, _P]),
     "dsx_emit_keys": (C.c_int, [_CAM, _I64, _I64, _P, _P, _P, _P, _P]),
     "dsx_sort_pairs": (C.c_int, [_I64, _I32, _P, _P, _P, C.c_size_t, _P]),
     "dsx_tile_ranges": (C.c_int, [_I64, _P, _I32, _P, _P]),
     "dsx_sort_pairs_u32": (C.c_int, [_I64, _I32, _P, _P, _P, C.c_size_t, _P]),
-    "dsx_depth_order": (C.c_int, [_I64, _P, C.c_size_t, _P]),
+    "dsx_depth_order": (C.c_int, [_CAM, _I64, _P, C.c_size_t, _P]),
     "dsx_order_view": (C.c_int, [_I64, _P, C.POINTER(_P), C.POINTER(_P)]),
     "dsx_tile_lists": (C.c_int, [_CAM, _I64, _I64, _P, _P, _P, _P, C.c_size_t, _P]),
     "dsx_blend_fwd": (C.c_int, [_CAM] + [_P] * 6 + [_P]),

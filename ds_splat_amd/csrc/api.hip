@@ -147,9 +147,9 @@ extern "C" size_t dsx_sort_workspace_bytes(int64_t k, int32_t num_tiles)
     return sort_workspace(k < 0 ? 0 : k, num_tiles < 0 ? 0 : num_tiles).bytes;
 }
 
-extern "C" size_t dsx_order_bytes(int64_t n)
+extern "C" size_t dsx_order_bytes(int64_t n, int32_t width, int32_t height)
 {
-    return order_layout(n < 0 ? 0 : n).bytes;
+    return order_layout(n < 0 ? 0 : n, width < 0 ? 0 : width, height < 0 ? 0 : height).bytes;
 }
 
 namespace
@@ -194,7 +194,7 @@ extern "C" int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* me
     uint2* rects = nullptr;
     if(order)
     {
-        const OrderLayout o = order_layout(n);
+        const OrderLayout o = order_layout(n, cam->image_width, cam->image_height);
         if(order_bytes < o.bytes)
             return DSX_ERR_WORKSPACE;
         depth_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(order) + o.depth_keys);
@@ -300,17 +300,19 @@ extern "C" int dsx_sort_pairs_u32(int64_t count, int32_t key_bits, uint32_t* key
     return DSX_OK;
 }
 
-extern "C" int dsx_depth_order(int64_t n, void* order, size_t order_bytes, void* stream)
+extern "C" int dsx_depth_order(const dsx_camera* cam, int64_t n, void* order, size_t order_bytes, void* stream)
 {
+    if(int rc = check_camera(cam))
+        return rc;
     if(n < 0)
         return DSX_ERR_BAD_ARG;
     if(n == 0)
         return DSX_OK;
     if(!order)
         return DSX_ERR_BAD_ARG;
-    if(order_bytes < order_layout(n).bytes)
+    if(order_bytes < order_layout(n, cam->image_width, cam->image_height).bytes)
         return DSX_ERR_WORKSPACE;
-    return launch_depth_order(n, order, as_stream(stream));
+    return launch_depth_order(*cam, n, order, as_stream(stream));
 }
 
 extern "C" int dsx_order_view(int64_t n, const void* order, const uint32_t** depth_order,
@@ -419,7 +421,7 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
     bool ok = hipMemcpyAsync(num_keys, k_scratch, sizeof(uint32_t), hipMemcpyDeviceToHost, s) == hipSuccess &&
               hipEventRecord(copied, s) == hipSuccess;
     if(ok)
-        rc = launch_depth_order(n, order, s);
+        rc = launch_depth_order(*cam, n, order, s);
     ok = ok && hipEventSynchronize(copied) == hipSuccess;
     (void)hipEventDestroy(copied);
     if(!ok)
@@ -494,7 +496,7 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     o_T = align(o_ranges + (size_t)(num_tiles + 1) * 4);
     o_idx = align(o_T + (size_t)P * 4);
     o_order = align(o_idx + (size_t)P * 4);
-    const size_t order_bytes = order_layout(n).bytes;
+    const size_t order_bytes = order_layout(n, image_width, image_height).bytes;
     stage1 = align(o_order + order_bytes);
     char* buf = nullptr;
     if(hipMallocAsync(reinterpret_cast<void**>(&buf), stage1 + 256, s) != hipSuccess)

@@ -188,10 +188,14 @@ struct OrderLayout
     size_t rects;      // uint2[n]   packed tile rectangle (written by the projection)
     size_t rects_sorted; // uint2[n] the same in depth order
     size_t block_sums; // uint32[blocks + 1] tile counts of 256 consecutive Gaussians IN DEPTH ORDER, scanned
+    size_t slot_hist;  // uint32[kMaxPasses32 * 256] digit histograms of the tile slots of all pairs
+    size_t cover;      // int32[(ntx + 1) * (nty + 1) + 1] pairs per tile (corner grid, then its 2-D prefix sum)
+    size_t ranges;     // int32[tiles + 1] the tile ranges, ready before the pairs exist
     size_t sort;       // Sort32Workspace
     size_t bytes;
 };
-OrderLayout order_layout(int64_t n);
+// the grid is the last member, so every other offset depends on n alone
+OrderLayout order_layout(int64_t n, int image_width = 0, int image_height = 0);
 
 // Workspace of the tile lists for k keys.
 struct ListsWorkspace
@@ -209,8 +213,8 @@ ListsWorkspace lists_workspace(int64_t k, int num_tiles);
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
                   uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src = nullptr,
-                  uint2* gather_dst = nullptr);
-int launch_depth_order(int64_t n, void* order, hipStream_t stream);
+                  uint2* gather_dst = nullptr, size_t clear_extra_bytes = 0);
+int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream);
 int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
                       int32_t* ranges, void* workspace, hipStream_t stream);
 int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, const float* scales,

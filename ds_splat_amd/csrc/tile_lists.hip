@@ -113,14 +113,14 @@ __global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const KeyT* __re
 }
 
 // exclusive scan of each pass's 256 bins (one workgroup per pass)
-__global__ __launch_bounds__(kBins32) void hist32_scan_kernel(uint32_t* global_hist)
+__global__ __launch_bounds__(kBins32) void hist32_scan_kernel(const uint32_t* counts, uint32_t* global_hist)
 {
     __shared__ uint32_t wave_tot[kBins32 / DSX_WAVE];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     uint32_t* h = global_hist + blockIdx.x * kBins32;
-    const uint32_t v = h[tid];
+    const uint32_t v = counts[blockIdx.x * kBins32 + tid];
     const uint32_t incl = wave_incl_scan32(v, lane);
     if(lane == 63)
         wave_tot[wave] = incl;
@@ -367,21 +367,24 @@ Sort32Workspace sort32_workspace(int64_t count, int key_bits, int tile_keys)
 }
 
 // zeroes histograms, tile counters and look-back statuses of one sort
-static int sort32_clear(int64_t count, int key_bits, int tile_keys, void* sort_ws, hipStream_t stream)
+// (extra_bytes: memory right behind the workspace that the same fill clears)
+static int sort32_clear(int64_t count, int key_bits, int tile_keys, void* sort_ws, hipStream_t stream,
+                        size_t extra_bytes = 0)
 {
     const Sort32Workspace w = sort32_workspace(count, key_bits, tile_keys);
-    return launch_fill_u32(reinterpret_cast<uint32_t*>(static_cast<char*>(sort_ws) + w.hist), (int64_t)(w.bytes / 4), 0u,
-                           stream);
+    return launch_fill_u32(reinterpret_cast<uint32_t*>(static_cast<char*>(sort_ws) + w.hist),
+                           (int64_t)((w.bytes + extra_bytes) / 4), 0u, stream);
 }
 
-// The digit passes of a sort whose raw digit histograms are already in the workspace.
+// The digit passes of a sort whose raw digit histograms are in `counts` (the workspace's own
+// histogram area when counts is null).
 // Ping-pong between (keys_a, vals_a) and (keys_b, vals_b); *keys_out / *vals_out say where the
 // result is (keys only when keep_keys).
 template <typename KeyT, int kThreads, int kItems>
 static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* vals_a, KeyT* keys_b, uint32_t* vals_b,
                          bool iota_values, bool keep_keys, void* sort_ws, const char* label, hipStream_t stream,
                          KeyT** keys_out, uint32_t** vals_out, const uint2* gather_src = nullptr,
-                         uint2* gather_dst = nullptr)
+                         uint2* gather_dst = nullptr, const uint32_t* counts = nullptr)
 {
     const Sort32Workspace w = sort32_workspace(count, key_bits, kThreads * kItems);
     const Digits32 plan = digits32(key_bits);
@@ -391,7 +394,8 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
     uint32_t* status = reinterpret_cast<uint32_t*>(base + w.status);
     {
         DSX_TIMED("hist32_scan_kernel", stream);
-        hipLaunchKernelGGL(hist32_scan_kernel, dim3(w.passes), dim3(kBins32), 0, stream, hist);
+        hipLaunchKernelGGL(hist32_scan_kernel, dim3(w.passes), dim3(kBins32), 0, stream,
+                           counts ? counts : (const uint32_t*)hist, hist);
     }
     DSX_LAUNCH_CHECK();
     KeyT* kin = keys_a;
@@ -426,7 +430,8 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
 // Stable ascending sort of `count` (key, value) pairs by the low key_bits bits of the key.
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
-                  uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src, uint2* gather_dst)
+                  uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src, uint2* gather_dst,
+                  size_t clear_extra_bytes)
 {
     *keys_out = keys_a;
     *vals_out = vals_a;
@@ -434,7 +439,7 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
         return DSX_OK;
     if(count >= (1ll << 30))
         return DSX_ERR_TOO_LARGE;
-    int rc = sort32_clear(count, key_bits, kDepthSortTile, sort_ws, stream);
+    int rc = sort32_clear(count, key_bits, kDepthSortTile, sort_ws, stream, clear_extra_bytes);
     if(rc)
         return rc;
     const Sort32Workspace w = sort32_workspace(count, key_bits, kDepthSortTile);
@@ -454,7 +459,7 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
 // depth order of the Gaussians and the scanned tile counts in that order
 // ---------------------------------------------------------------------------------------
 
-OrderLayout order_layout(int64_t n)
+OrderLayout order_layout(int64_t n, int image_width, int image_height)
 {
     auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
     OrderLayout o;
@@ -473,8 +478,14 @@ OrderLayout order_layout(int64_t n)
     off = align(off + (size_t)n * 8);
     o.block_sums = off;
     off = align(off + (size_t)((n + kProjBlock - 1) / kProjBlock + 1) * 4);
+    o.slot_hist = off;
+    off = align(off + (size_t)kMaxPasses32 * kBins32 * 4);
     o.sort = off;
-    off += sort32_workspace(n, 32, kDepthSortTile).bytes;
+    off = align(off + sort32_workspace(n, 32, kDepthSortTile).bytes);
+    o.cover = off;
+    off = align(off + (size_t)((tiles_x(image_width) + 1) * (tiles_y(image_height) + 1) + 1) * 4);
+    o.ranges = off;
+    off += (size_t)(tiles_x(image_width) * tiles_y(image_height) + 1) * 4;
     o.bytes = align(off);
     return o;
 }
@@ -503,12 +514,197 @@ __global__ __launch_bounds__(kProjBlock) void ordered_block_sums_kernel(const ui
         block_sums[blockIdx.x] = wave_sums[0] + wave_sums[1] + wave_sums[2] + wave_sums[3];
 }
 
+// How many pairs each tile receives, straight from the rectangles (no pair is enumerated):
+// a rectangle [sx, ex) x [sy, ey) adds +1, -1, -1, +1 at its four corners of a
+// (nty + 1) x (ntx + 1) grid, and the two-dimensional prefix sum of that grid is the number of
+// rectangles covering each tile.  Pairs of a Gaussian with a negative depth all sit in slot 0:
+// they are counted in the cell after the grid.  From the per-tile counts come the digit
+// histograms of the tile partition (and the tile counts themselves).
+constexpr int kCoverThreads = 1024;
+constexpr int kCoverBlocks = 128;
+constexpr int kCoverLdsCells = 14 * 1024; // grids up to this many cells (56 KB) are held in LDS
+
+__global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* __restrict__ rects, int64_t n, int ntx,
+                                                                   int nty, int use_lds, int32_t* __restrict__ grid)
+{
+    extern __shared__ int32_t s_grid[];
+    const int tid = threadIdx.x;
+    const int pitch = ntx + 1;
+    const int cells = pitch * (nty + 1) + 1;
+    int32_t* acc = use_lds ? s_grid : grid;
+    if(use_lds)
+    {
+        for(int j = tid; j < cells; j += kCoverThreads)
+            s_grid[j] = 0;
+        __syncthreads();
+    }
+    for(int64_t g = (int64_t)blockIdx.x * kCoverThreads + tid; g < n; g += (int64_t)gridDim.x * kCoverThreads)
+    {
+        const uint2 r = rects[g];
+        const int w = (int)(r.y & 0xffffu), h = (int)((r.y >> 16) & 0x7fffu);
+        if(w == 0 || h == 0)
+            continue;
+        if(r.y >> 31)
+        {
+            atomicAdd(&acc[cells - 1], w * h);
+            continue;
+        }
+        const int sx = (int)(r.x & 0xffffu), sy = (int)(r.x >> 16);
+        atomicAdd(&acc[sy * pitch + sx], 1);
+        atomicAdd(&acc[sy * pitch + sx + w], -1);
+        atomicAdd(&acc[(sy + h) * pitch + sx], -1);
+        atomicAdd(&acc[(sy + h) * pitch + sx + w], 1);
+    }
+    if(use_lds)
+    {
+        __syncthreads();
+        for(int j = tid; j < cells; j += kCoverThreads)
+            if(s_grid[j])
+                atomicAdd(&grid[j], s_grid[j]);
+    }
+}
+
+// One workgroup: 2-D prefix sum of the corner grid (in LDS when the grid fits, else in place in
+// global memory, where a few ten thousand cells stay in the L2), then
+//  * the digit histograms of slot = tile + 1 (slot 0 = the negative depths),
+//  * ranges[j] = number of pairs whose tile is below j, with the two rules of the reference
+//    (cpp/rasterizer_kernels.cu:313-322, cpp/rasterizer_torch.cu:31-39): the boundary after
+//    the LAST run is never recorded, so tiles above the highest occupied tile inherit the
+//    START of that run (all zero when no tile is occupied), and ranges[num_tiles] = K.
+__global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(int32_t* grid, int ntx, int nty, int use_lds,
+                                                                    const Digits32 plan,
+                                                                    uint32_t* __restrict__ slot_hist,
+                                                                    int32_t* __restrict__ ranges)
+{
+    extern __shared__ int32_t s_cells[];
+    __shared__ uint32_t hist[kMaxPasses32 * kBins32];
+    __shared__ uint32_t wave_tot[kCoverThreads / DSX_WAVE];
+    __shared__ uint32_t s_carry;
+    __shared__ int s_last;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int pitch = ntx + 1;
+    const int cells = pitch * (nty + 1) + 1;
+    const uint32_t negatives = (uint32_t)grid[cells - 1];
+    int32_t* c = grid;
+    if(use_lds)
+    {
+        for(int j = tid; j < cells; j += kCoverThreads)
+            s_cells[j] = grid[j];
+        c = s_cells;
+    }
+    for(int j = tid; j < kMaxPasses32 * kBins32; j += kCoverThreads)
+        hist[j] = 0;
+    if(tid == 0)
+    {
+        s_carry = negatives;
+        s_last = -1;
+    }
+    __threadfence_block();
+    __syncthreads();
+    // along x: one wavefront per row, 64 columns at a time with a carry
+    for(int y = wave; y < nty; y += kCoverThreads / DSX_WAVE)
+    {
+        int32_t carry = 0;
+        for(int x0 = 0; x0 < ntx; x0 += DSX_WAVE)
+        {
+            const int x = x0 + lane;
+            const int32_t v = x < ntx ? c[y * pitch + x] : 0;
+            const int32_t incl = (int32_t)wave_incl_scan32((uint32_t)v, lane) + carry;
+            if(x < ntx)
+                c[y * pitch + x] = incl;
+            carry = __shfl(incl, 63, DSX_WAVE);
+        }
+    }
+    __threadfence_block();
+    __syncthreads();
+    // along y: one thread per column
+    for(int x = tid; x < ntx; x += kCoverThreads)
+    {
+        int32_t run = 0;
+        for(int y = 0; y < nty; ++y)
+        {
+            run += c[y * pitch + x];
+            c[y * pitch + x] = run; // pairs of tile (x, y)
+        }
+    }
+    __threadfence_block();
+    __syncthreads();
+    // histograms, exclusive scan over the tiles in row-major order, highest occupied tile
+    const int tiles = ntx * nty;
+    for(int t0 = 0; t0 < tiles; t0 += kCoverThreads)
+    {
+        const int t = t0 + tid;
+        const uint32_t cnt = t < tiles ? (uint32_t)c[(t / ntx) * pitch + (t % ntx)] : 0u;
+        // lanes hold consecutive tiles: the lowest digit differs from lane to lane (plain LDS
+        // atomics, no conflicts), a higher digit is constant over long runs (one add per run,
+        // after a wavefront sum; same-address LDS atomics would serialise)
+        {
+            const uint32_t slot = (uint32_t)t + 1u;
+            for(int p = 0; p < plan.passes; ++p)
+            {
+                const uint32_t d = (slot >> plan.shift[p]) & plan.mask[p];
+                if(plan.shift[p] == 0)
+                {
+                    if(cnt)
+                        atomicAdd(&hist[p * kBins32 + d], cnt);
+                    continue;
+                }
+                uint64_t todo = __ballot(true);
+                while(todo)
+                {
+                    const int leader = __builtin_ctzll(todo);
+                    const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)d, leader);
+                    const bool mine = d == dl;
+                    const uint32_t sum = wave_sum_u32(mine ? cnt : 0u);
+                    if(lane == leader && sum)
+                        atomicAdd(&hist[p * kBins32 + dl], sum);
+                    todo &= ~__ballot(mine);
+                }
+            }
+            const uint64_t occupied = __ballot(cnt != 0);
+            if(occupied && lane == 0)
+                atomicMax(&s_last, t0 + wave * DSX_WAVE + 63 - __builtin_clzll(occupied));
+        }
+        const uint32_t incl = wave_incl_scan32(cnt, lane);
+        if(lane == 63)
+            wave_tot[wave] = incl;
+        __syncthreads();
+        uint32_t prefix = s_carry;
+        for(int w = 0; w < wave; ++w)
+            prefix += wave_tot[w];
+        if(t < tiles)
+            ranges[t] = (int32_t)(prefix + incl - cnt);
+        __syncthreads();
+        if(tid == kCoverThreads - 1)
+            s_carry = prefix + incl;
+        __syncthreads();
+    }
+    __threadfence_block();
+    __syncthreads();
+    const int last = s_last;
+    const int32_t tail = last >= 0 ? ranges[last] : 0;
+    for(int t = tid; t < tiles; t += kCoverThreads)
+        if(t > last)
+            ranges[t] = tail;
+    if(tid == 0)
+    {
+        ranges[tiles] = (int32_t)s_carry; // K
+        for(int p = 0; p < plan.passes; ++p)
+            atomicAdd(&hist[p * kBins32], negatives);
+    }
+    __syncthreads();
+    for(int j = tid; j < kMaxPasses32 * kBins32; j += kCoverThreads)
+        slot_hist[j] = hist[j];
+}
+
 // order: the buffer of order_layout(n) whose depth_keys and rects the projection has written
-int launch_depth_order(int64_t n, void* order, hipStream_t stream)
+int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream)
 {
     if(n <= 0)
         return DSX_OK;
-    const OrderLayout o = order_layout(n);
+    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height);
     char* base = static_cast<char*>(order);
     uint32_t* keys_a = reinterpret_cast<uint32_t*>(base + o.depth_keys);
     uint32_t* keys_b = reinterpret_cast<uint32_t*>(base + o.keys_alt);
@@ -519,11 +715,35 @@ int launch_depth_order(int64_t n, void* order, hipStream_t stream)
     // 32 key bits = 4 passes: the values (iota in pass 0) go b, a, b, a and end in ids_a
     int rc = launch_sort32(n, 32, keys_a, ids_a, keys_b, ids_b, true, false, base + o.sort, stream, &ko, &vo,
                            reinterpret_cast<const uint2*>(base + o.rects),
-                           reinterpret_cast<uint2*>(base + o.rects_sorted));
+                           reinterpret_cast<uint2*>(base + o.rects_sorted), o.ranges - o.cover);
     if(rc)
         return rc;
     if(vo != ids_a)
         return DSX_ERR_RUNTIME;
+    // pairs per tile: digit histograms of the tile partition and the tile ranges that the second
+    // half of the forward needs (the grid was zeroed together with the sort's counters)
+    {
+        const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
+        const int cells = (ntx + 1) * (nty + 1) + 1;
+        int32_t* grid = reinterpret_cast<int32_t*>(base + o.cover);
+        const int use_lds = cells <= kCoverLdsCells ? 1 : 0;
+        const int64_t want = (n + kCoverThreads - 1) / kCoverThreads;
+        {
+            DSX_TIMED("tile_cover_kernel", stream);
+            hipLaunchKernelGGL(tile_cover_kernel, dim3((unsigned)min((int64_t)kCoverBlocks, want)), dim3(kCoverThreads),
+                               use_lds ? (size_t)cells * 4 : 0, stream, reinterpret_cast<const uint2*>(base + o.rects), n,
+                               ntx, nty, use_lds, grid);
+        }
+        DSX_LAUNCH_CHECK();
+        {
+            DSX_TIMED("tile_counts_kernel", stream);
+            hipLaunchKernelGGL(tile_counts_kernel, dim3(1), dim3(kCoverThreads), use_lds ? (size_t)cells * 4 : 0, stream,
+                               grid, ntx, nty, use_lds, digits32(slot_bits(ntx * nty)),
+                               reinterpret_cast<uint32_t*>(base + o.slot_hist),
+                               reinterpret_cast<int32_t*>(base + o.ranges));
+        }
+        DSX_LAUNCH_CHECK();
+    }
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     {
         DSX_TIMED("ordered_block_sums_kernel", stream);
@@ -543,9 +763,10 @@ template <typename SlotT>
 __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t* __restrict__ order,
                                                                   const uint2* __restrict__ rects_sorted,
                                                                   const uint32_t* __restrict__ block_offsets,
-                                                                  int64_t n, int64_t k, int ntx, const Digits32 plan,
+                                                                  int64_t n, int64_t k, int ntx,
                                                                   SlotT* __restrict__ slots, int32_t* __restrict__ ids,
-                                                                  uint32_t* __restrict__ global_hist)
+                                                                  const int32_t* __restrict__ ranges_in,
+                                                                  int32_t* __restrict__ ranges_out, int range_count)
 {
     __shared__ uint32_t s_off[kProjBlock + 1];
     __shared__ uint32_t s_origin[kProjBlock]; // slot of the rectangle's first tile (0 for negative depths)
@@ -553,13 +774,14 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     __shared__ float s_winv[kProjBlock];
     __shared__ uint32_t s_id[kProjBlock];
     __shared__ uint32_t wave_tot[kProjBlock / DSX_WAVE];
-    __shared__ uint32_t hist[kMaxPasses32 * kBins32]; // digit histograms of the partition that follows
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    for(int j = tid; j < plan.passes * kBins32; j += kProjBlock)
-        hist[j] = 0;
+
+    // the tile ranges were derived from the rectangles before any pair existed: hand them out
+    for(int j = blockIdx.x * kProjBlock + tid; j < range_count; j += gridDim.x * kProjBlock)
+        ranges_out[j] = ranges_in[j];
 
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     for(int64_t blk = blockIdx.x; blk < blocks; blk += gridDim.x)
@@ -593,94 +815,36 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
 
         const uint32_t total = s_off[kProjBlock];
         const int64_t base = block_offsets[blk];
-        for(uint32_t j0 = 0; j0 < total; j0 += kProjBlock) // uniform trip count: ballots below
+        for(uint32_t j = tid; j < total && base + j < k; j += kProjBlock)
         {
-            const uint32_t j = j0 + tid;
-            const bool valid = j < total && base + j < k;
+            // largest g with s_off[g] <= j
+            int lo = 0, hi = kProjBlock;
+            while(hi - lo > 1)
+            {
+                const int mid = (lo + hi) >> 1;
+                if(s_off[mid] <= j)
+                    lo = mid;
+                else
+                    hi = mid;
+            }
+            const uint32_t r = j - s_off[lo];
+            const uint32_t w = s_w[lo];
             uint32_t slot = 0;
-            uint32_t id = 0;
-            if(valid)
+            if(w)
             {
-                // largest g with s_off[g] <= j
-                int lo = 0, hi = kProjBlock;
-                while(hi - lo > 1)
-                {
-                    const int mid = (lo + hi) >> 1;
-                    if(s_off[mid] <= j)
-                        lo = mid;
-                    else
-                        hi = mid;
-                }
-                const uint32_t r = j - s_off[lo];
-                const uint32_t w = s_w[lo];
-                if(w)
-                {
-                    // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
-                    uint32_t ry = (uint32_t)((float)r * s_winv[lo]);
-                    if(ry * w > r)
-                        --ry;
-                    else if((ry + 1) * w <= r)
-                        ++ry;
-                    const uint32_t rx = r - ry * w;
-                    slot = s_origin[lo] + ry * (uint32_t)ntx + rx;
-                }
-                id = s_id[lo];
-                slots[base + j] = (SlotT)slot;
-                ids[base + j] = (int32_t)id;
+                // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
+                uint32_t ry = (uint32_t)((float)r * s_winv[lo]);
+                if(ry * w > r)
+                    --ry;
+                else if((ry + 1) * w <= r)
+                    ++ry;
+                const uint32_t rx = r - ry * w;
+                slot = s_origin[lo] + ry * (uint32_t)ntx + rx;
             }
-            // digit histograms: a run of equal digits in neighbouring lanes is added by its first lane
-            const uint64_t vmask = __ballot(valid); // valid lanes are a prefix of the wavefront
-            const int nvalid = __popcll(vmask);
-            for(int ps = 0; ps < plan.passes; ++ps)
-            {
-                const uint32_t d = (slot >> plan.shift[ps]) & plan.mask[ps];
-                const uint32_t below = lane_below32(d, ~d);
-                const bool head = valid && (lane == 0 || below != d);
-                const uint64_t heads = __ballot(head);
-                if(head)
-                {
-                    const uint64_t above = lane == 63 ? 0ull : (heads >> (lane + 1));
-                    const int run = above ? __ffsll((unsigned long long)above) : nvalid - lane;
-                    atomicAdd(&hist[ps * kBins32 + d], (uint32_t)run);
-                }
-            }
+            slots[base + j] = (SlotT)slot;
+            ids[base + j] = (int32_t)s_id[lo];
         }
     }
-    __syncthreads();
-    for(int j = tid; j < plan.passes * kBins32; j += kProjBlock)
-        if(hist[j])
-            atomicAdd(&global_hist[j], hist[j]);
-}
-
-// ranges[j] = number of pairs whose tile is below j, by binary search in the sorted slots.
-// Two rules of the reference are kept (cpp/rasterizer_kernels.cu:313-322,
-// cpp/rasterizer_torch.cu:31-39): the boundary after the LAST run is never recorded, so tiles
-// above the highest occupied tile inherit the START of that run, and ranges[num_tiles] = K.
-// Slot 0 (negative depths) is skipped by ranges[0].
-template <typename SlotT>
-__global__ __launch_bounds__(256) void ranges_slots_kernel(const SlotT* __restrict__ slots, int64_t k,
-                                                           int num_tiles, int32_t* __restrict__ ranges)
-{
-    const int j = blockIdx.x * 256 + threadIdx.x;
-    if(j > num_tiles)
-        return;
-    if(j == num_tiles || k == 0)
-    {
-        ranges[j] = j == num_tiles ? (int32_t)k : 0;
-        return;
-    }
-    const uint32_t last_slot = slots[k - 1];
-    const uint32_t target = (uint32_t)(j + 1) < last_slot ? (uint32_t)(j + 1) : last_slot;
-    int64_t lo = 0, hi = k; // first index with slots[i] >= target
-    while(lo < hi)
-    {
-        const int64_t mid = (lo + hi) >> 1;
-        if(slots[mid] < target)
-            lo = mid + 1;
-        else
-            hi = mid;
-    }
-    ranges[j] = (int32_t)lo;
 }
 
 // tile slots 0..num_tiles fit 16 bits for every image up to 65534 tiles (4K has 32400)
@@ -712,54 +876,48 @@ template <typename SlotT>
 static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_tiles, const void* order,
                            int32_t* sorted_ids, int32_t* ranges, void* workspace, hipStream_t stream)
 {
-    const SlotT* sorted_slots = nullptr;
-    if(k > 0)
+    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height);
+    const char* obase = static_cast<const char*>(order);
+    if(k <= 0)
     {
-        const OrderLayout o = order_layout(n);
-        const ListsWorkspace w = lists_workspace(k, num_tiles);
-        const int bits = slot_bits(num_tiles);
-        const char* obase = static_cast<const char*>(order);
-        char* base = static_cast<char*>(workspace);
-        SlotT* slots_a = reinterpret_cast<SlotT*>(base + w.slots_a);
-        SlotT* slots_b = reinterpret_cast<SlotT*>(base + w.slots_b);
-        uint32_t* ids_final = reinterpret_cast<uint32_t*>(sorted_ids);
-        uint32_t* ids_other = reinterpret_cast<uint32_t*>(base + w.ids_alt);
-        // ping-pong parity: start so that the last pass lands the ids in the caller's buffer
-        const bool even = (w.passes % 2) == 0;
-        uint32_t* vals_a = even ? ids_final : ids_other;
-        uint32_t* vals_b = even ? ids_other : ids_final;
-        int rc = sort32_clear(k, bits, kListSortTile, base + w.sort, stream);
-        if(rc)
-            return rc;
-        const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
-        {
-            DSX_TIMED("emit_ordered_kernel", stream);
-            hipLaunchKernelGGL(emit_ordered_kernel<SlotT>, dim3((unsigned)min(blocks, (int64_t)DSX_EMIT_BLOCKS)), dim3(kProjBlock),
-                               0, stream, reinterpret_cast<const uint32_t*>(obase + o.ids_a),
-                               reinterpret_cast<const uint2*>(obase + o.rects_sorted),
-                               reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k, tiles_x(cam.image_width),
-                               digits32(bits), slots_a, reinterpret_cast<int32_t*>(vals_a),
-                               reinterpret_cast<uint32_t*>(base + w.sort + sort32_workspace(k, bits, kListSortTile).hist));
-        }
-        DSX_LAUNCH_CHECK();
-        SlotT* ko;
-        uint32_t* vo;
-        rc = sort32_passes<SlotT, kListSortThreads, kListSortItems>(k, bits, slots_a, vals_a, slots_b, vals_b, false, true, base + w.sort,
-                                  "onesweep32_kernel<tile partition>", stream, &ko, &vo);
-        if(rc)
-            return rc;
-        if(vo != ids_final)
-            return DSX_ERR_RUNTIME;
-        sorted_slots = ko;
+        // no pairs: the ranges are all zero
+        return launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), num_tiles + 1, 0u, stream);
     }
-    const int count = num_tiles + 1;
+    const ListsWorkspace w = lists_workspace(k, num_tiles);
+    const int bits = slot_bits(num_tiles);
+    char* base = static_cast<char*>(workspace);
+    SlotT* slots_a = reinterpret_cast<SlotT*>(base + w.slots_a);
+    SlotT* slots_b = reinterpret_cast<SlotT*>(base + w.slots_b);
+    uint32_t* ids_final = reinterpret_cast<uint32_t*>(sorted_ids);
+    uint32_t* ids_other = reinterpret_cast<uint32_t*>(base + w.ids_alt);
+    // ping-pong parity: start so that the last pass lands the ids in the caller's buffer
+    const bool even = (w.passes % 2) == 0;
+    uint32_t* vals_a = even ? ids_final : ids_other;
+    uint32_t* vals_b = even ? ids_other : ids_final;
+    int rc = sort32_clear(k, bits, kListSortTile, base + w.sort, stream);
+    if(rc)
+        return rc;
+    const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     {
-        DSX_TIMED("ranges_slots_kernel", stream);
-        hipLaunchKernelGGL(ranges_slots_kernel<SlotT>, dim3((count + 255) / 256), dim3(256), 0, stream, sorted_slots, k,
-                           num_tiles, ranges);
+        DSX_TIMED("emit_ordered_kernel", stream);
+        hipLaunchKernelGGL(emit_ordered_kernel<SlotT>, dim3((unsigned)min(blocks, (int64_t)DSX_EMIT_BLOCKS)), dim3(kProjBlock),
+                           0, stream, reinterpret_cast<const uint32_t*>(obase + o.ids_a),
+                           reinterpret_cast<const uint2*>(obase + o.rects_sorted),
+                           reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k, tiles_x(cam.image_width),
+                           slots_a, reinterpret_cast<int32_t*>(vals_a),
+                           reinterpret_cast<const int32_t*>(obase + o.ranges), ranges, num_tiles + 1);
     }
     DSX_LAUNCH_CHECK();
-    return DSX_OK;
+    SlotT* ko;
+    uint32_t* vo;
+    // the sorted slots themselves are not needed: the ranges are known already
+    rc = sort32_passes<SlotT, kListSortThreads, kListSortItems>(k, bits, slots_a, vals_a, slots_b, vals_b, false, false,
+                                                                base + w.sort, "onesweep32_kernel<tile partition>",
+                                                                stream, &ko, &vo, nullptr, nullptr,
+                                                                reinterpret_cast<const uint32_t*>(obase + o.slot_hist));
+    if(rc)
+        return rc;
+    return vo == ids_final ? DSX_OK : DSX_ERR_RUNTIME;
 }
 
 // order: buffer of order_layout(n) after launch_depth_order.  Writes sorted_ids[k], ranges[T+1].

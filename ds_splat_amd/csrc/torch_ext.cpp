@@ -92,7 +92,7 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
     at::Tensor radii = at::empty({n}, i32);
     at::Tensor cov3d = at::empty({n, 6}, f32);
     at::Tensor block_sums = at::empty({dsx_num_blocks(n) + 1}, i32);
-    const size_t order_bytes = dsx_order_bytes(n);
+    const size_t order_bytes = dsx_order_bytes(n, (int32_t)width, (int32_t)height);
     at::Tensor order = at::empty({(int64_t)std::max<size_t>(order_bytes, 1)}, u8);
     at::Tensor& k_host = pinned_key_count();
     uint32_t* bs = reinterpret_cast<uint32_t*>(block_sums.data_ptr<int32_t>());

@@ -83,16 +83,17 @@ def project_fwd(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None,
     return splats, radii, cov3d, block_sums
 
 
-def new_order(n, device):
-    """The per-Gaussian buffer that carries the depth order from the projection to the tile lists."""
-    return torch.empty((max(int(N.load().dsx_order_bytes(n)), 1),), dtype=torch.uint8, device=device)
+def new_order(cam, n, device):
+    """The buffer that carries the depth order from the projection to the tile lists."""
+    nbytes = int(N.load().dsx_order_bytes(n, cam.width, cam.height))
+    return torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=device)
 
 
-def depth_order(n, order):
+def depth_order(cam, n, order):
     """Sorts the Gaussians of a projected `order` buffer by depth bits (stable).  Returns views
     (depth order int32[n], scanned tile counts of its 256-Gaussian blocks int32[blocks + 1])."""
     lib = N.load()
-    N.check(lib.dsx_depth_order(n, _ptr(order), order.numel(), _stream()))
+    N.check(lib.dsx_depth_order(cam.ref, n, _ptr(order), order.numel(), _stream()))
     p_order, p_off = C.c_void_p(), C.c_void_p()
     N.check(lib.dsx_order_view(n, _ptr(order), C.byref(p_order), C.byref(p_off)))
     base = order.data_ptr()
@@ -222,7 +223,7 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     st.cov3d = torch.empty((n, 6), dtype=torch.float32, device=dev)
     block_sums = torch.empty((int(lib.dsx_num_blocks(n)) + 1,), dtype=torch.int32, device=dev)
     k_scratch = block_sums[-1:]
-    order = new_order(n, dev)
+    order = new_order(cam, n, dev)
     k_host = _pinned_i64()
     stream = _stream()
     N.check(lib.dsx_forward_project(cam.ref, n, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(opacities), _ptr(shs),

@@ -84,7 +84,7 @@ size_t dsx_sort_workspace_bytes(int64_t k, int32_t num_tiles);
 size_t dsx_sort_u32_workspace_bytes(int64_t count, int32_t key_bits);
 /* bytes of the per-Gaussian `order` buffer that carries the depth order from the projection
  * (dsx_project_fwd / dsx_forward_project) to the tile lists (dsx_tile_lists / dsx_forward_finish) */
-size_t dsx_order_bytes(int64_t n);
+size_t dsx_order_bytes(int64_t n, int32_t width, int32_t height);
 
 /* ------------------------------------------------------------------------------------ */
 /* Per-stage entry points (each one individually parity-tested and timed)                */
@@ -95,7 +95,7 @@ size_t dsx_order_bytes(int64_t n);
  * and block_sums[dsx_num_blocks(n)] (tile count of each 256-Gaussian block; the last
  * Gaussian counts as zero, cpp/rasterizer_torch.cu:99-104).  shs may be NULL iff
  * colors_precomp is given; scales/quats may be NULL iff cov3d_precomp is given (then cov3d
- * receives a copy).  order (may be NULL): buffer of dsx_order_bytes(n) that also receives each
+ * receives a copy).  order (may be NULL): buffer of dsx_order_bytes(n, W, H) that also receives each
  * Gaussian's depth bits and packed tile rectangle, the input of dsx_depth_order. */
 int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
                     const float* quats, const float* opacities, const float* shs,
@@ -137,13 +137,15 @@ int dsx_tile_ranges(int64_t k, const int64_t* sorted_keys, int32_t num_tiles, in
  * dsx_sort_pairs_u32: stable ascending sort of (uint32 key, uint32 value) pairs by the low
  * key_bits bits of the key, in place (the building block of both (1) and (3)).
  * dsx_depth_order: step (1) on an `order` buffer the projection has filled; it also leaves the
- * scanned tile counts of the depth-ordered 256-Gaussian blocks in the buffer.
+ * scanned tile counts of the depth-ordered 256-Gaussian blocks, the number of pairs of every
+ * tile and the digit histograms of the tile slots (from the rectangles by a 2-D prefix sum of
+ * their corners: no pair is enumerated) in the buffer.
  * dsx_order_view: device pointers into the buffer (depth order uint32[n], block offsets
  * uint32[dsx_num_blocks(n)+1] whose last entry is K), for inspection.
  * dsx_tile_lists: steps (2) and (3) and the ranges. */
 int dsx_sort_pairs_u32(int64_t count, int32_t key_bits, uint32_t* keys, uint32_t* values,
                        void* workspace, size_t workspace_bytes, void* stream);
-int dsx_depth_order(int64_t n, void* order, size_t order_bytes, void* stream);
+int dsx_depth_order(const dsx_camera* cam, int64_t n, void* order, size_t order_bytes, void* stream);
 int dsx_order_view(int64_t n, const void* order, const uint32_t** depth_order,
                    const uint32_t** block_offsets);
 int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const void* order,
@@ -185,7 +187,7 @@ int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const 
  * block scan, the read-back of K (the one host wait of the forward, in place of the reference's
  * two device drains at cpp/rasterizer_torch.cu:103-104) and, overlapping that read-back, the
  * depth order.  block_sums is scanned in place.  k_scratch: device uint32[1].  order: device
- * buffer of dsx_order_bytes(n).  *num_keys (host; pinned memory lets the copy overlap)
+ * buffer of dsx_order_bytes(n, W, H).  *num_keys (host; pinned memory lets the copy overlap)
  * receives K. */
 int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
                         const float* scales, const float* quats, const float* opacities,

@@ -49,7 +49,8 @@ def test_host_helpers():
     assert lib.dsx_sort_workspace_bytes(1 << 20, 8160) > (1 << 20) * 12
     assert lib.dsx_sort_u32_workspace_bytes(1 << 20, 32) > (1 << 20) * 8
     # order buffer: 4 uint32 arrays and two uint2 arrays per Gaussian
-    assert lib.dsx_order_bytes(1 << 20) > (1 << 20) * 32
+    assert lib.dsx_order_bytes(1 << 20, 1920, 1080) > (1 << 20) * 32
+    assert lib.dsx_order_bytes(0, 3840, 2160) - lib.dsx_order_bytes(0, 16, 16) >= 241 * 136 * 4 - 512
     assert b"workspace" in lib.dsx_error_string(-5)
     assert lib.dsx_error_string(0) == b"ok"
 
@@ -64,8 +65,7 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.dsx_project_fwd(None, 10, *([None] * 12), 0, None) == -1
     assert lib.dsx_sort_pairs_u32(10, 33, 1, 1, 1, 0, None) == -1
     assert lib.dsx_sort_pairs_u32(10, 32, 1, 1, 1, 0, None) == -5
-    assert lib.dsx_depth_order(10, None, 0, None) == -1
-    assert lib.dsx_depth_order(10, 1, 16, None) == -5
+    assert lib.dsx_depth_order(None, 10, None, 0, None) == -1
 
 
 def test_python_api_surface():

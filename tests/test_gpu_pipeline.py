@@ -166,7 +166,7 @@ def test_full_size_properties_cfg2():
     n = sc["n"]
     cam = stages.camera_from_scene(sc, DEV)
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
-    order = stages.new_order(n, DEV)
+    order = stages.new_order(cam, n, DEV)
     splats, radii, cov3d, block_sums = stages.project_fwd(cam, t["means_3d"], t["scales"], t["rotations"],
                                                           t["opacities"], t["shs"], order=order)
     tiles = splats[:, 11].view(torch.int32).to(torch.int64)
@@ -193,7 +193,7 @@ def test_full_size_properties_cfg2():
     assert (ranges[1:] >= ranges[:-1]).all() and int(ranges[-1]) == k and int(ranges[0]) == 0
     # the fast route (depth order of the Gaussians, ordered emission, tile partition) gives the
     # same lists as the 64-bit sort of all keys
-    perm, offsets = stages.depth_order(n, order)
+    perm, offsets = stages.depth_order(cam, n, order)
     assert int(offsets[-1]) == k
     d_sorted = (depth_bits & 0xFFFFFFFF)[perm.to(torch.int64)]       # unsigned order of the depth bits
     assert (d_sorted[1:] >= d_sorted[:-1]).all()
