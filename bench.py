@@ -33,6 +33,12 @@ BWD_PAIR_FLOPS, BWD_REJECT_FLOPS = 72, 15
 # profiles/cfg2_hbm_traffic_per_kernel.md).  Counters cannot be read from inside this process, so
 # the figures are quoted here and only reported when workload and key count are the profiled ones.
 MEASURED_TRAFFIC = {
+    ("cfg2", 32604809): {
+        "project_fwd_kernel": 943.8e6, "hist32_kernel": 13.6e6, "onesweep32_kernel<sort>": 134.9e6,
+        "ordered_block_sums_kernel": 24.4e6, "emit_ordered_kernel": 233.2e6,
+        "onesweep32_kernel<tile partition>": 384.5e6, "gaussian_bwd_kernel": 1333.2e6,
+        "blend_fwd_kernel": 78.8e6, "blend_bwd_kernel": 194.0e6,
+    },
 }
 
 
@@ -49,11 +55,13 @@ def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, counters):
     if kernel == "onesweep32_kernel<sort>":                  # depth sort of the Gaussians: key + id, in and out
         return "hbm", 16 * n, "B"
     if kernel == "ordered_block_sums_kernel":
-        return "hbm", 12 * n, "B"
+        return "hbm", 8 * n, "B"
     if kernel == "emit_ordered_kernel":
         return "hbm", 12 * n + (slot_bytes + 4) * k, "B"
-    if kernel == "onesweep32_kernel<tile partition>":        # tile partition: slot + id, in and out
-        return "hbm", 2 * (slot_bytes + 4) * k, "B"
+    if kernel == "onesweep32_kernel<tile partition>":
+        # tile partition: slot + id in and out, except that the last pass writes no slots (average per launch)
+        passes = 1 if tiles + 1 <= 256 else (2 if tiles + 1 <= 65536 else 3)
+        return "hbm", (2 * (slot_bytes + 4) * passes - slot_bytes) * k / passes, "B"
     if kernel == "blend_fwd_kernel" and counters is not None:
         rej = counters.pairs_fwd - counters.pairs_fwd_applied
         return "valu", counters.pairs_fwd_applied * FWD_PAIR_FLOPS + rej * FWD_REJECT_FLOPS, "FLOP"

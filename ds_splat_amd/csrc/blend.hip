@@ -52,7 +52,8 @@ __device__ __forceinline__ bool entry_reaches_tile(float mx, float my, float a, 
 constexpr int kFwdBatch = 128; // sorted entries staged in LDS per round (two per lane)
 constexpr int kFwdPix = 4;
 
-__global__ __launch_bounds__(DSX_WAVE) void blend_fwd_kernel(const int32_t* __restrict__ ranges,
+// 8 wavefronts per SIMD (at most 64 VGPRs): all tiles of a 1080p image are resident at once
+__global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))) void blend_fwd_kernel(const int32_t* __restrict__ ranges,
                                                              const int32_t* __restrict__ ids,
                                                              const float4* __restrict__ splats,
                                                              float* __restrict__ image, float* __restrict__ final_T,
