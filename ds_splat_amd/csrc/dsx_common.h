@@ -213,7 +213,7 @@ ListsWorkspace lists_workspace(int64_t k, int num_tiles);
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
                   uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src = nullptr,
-                  uint2* gather_dst = nullptr, size_t clear_extra_bytes = 0);
+                  uint2* gather_dst = nullptr, bool already_cleared = false);
 int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream);
 int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
                       int32_t* ranges, void* workspace, hipStream_t stream);

@@ -12,8 +12,36 @@
 // once and moved twice, instead of 12 bytes moved five times.
 #include "dsx_common.h"
 
+#include <mutex>
+
 namespace dsx
 {
+
+// One helper stream per device (default priority, created on first use, kept until the process
+// ends): work that does not depend on the depth sort runs there, beside the sort's
+// latency-bound passes.  Returns nullptr when no stream can be made (the caller then stays on
+// its own stream).
+static hipStream_t helper_stream()
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static hipStream_t streams[kMaxDevices] = {};
+    static bool tried[kMaxDevices] = {};
+    int device = 0;
+    if(hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+        return nullptr;
+    std::lock_guard<std::mutex> lock(mutex);
+    if(!tried[device])
+    {
+        tried[device] = true;
+        hipStream_t s = nullptr;
+        if(hipStreamCreateWithFlags(&s, hipStreamNonBlocking) == hipSuccess)
+            streams[device] = s;
+        else
+            (void)hipGetLastError();
+    }
+    return streams[device];
+}
 
 __device__ __forceinline__ uint32_t wave_incl_scan32(uint32_t v, int lane)
 {
@@ -431,7 +459,7 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
                   uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src, uint2* gather_dst,
-                  size_t clear_extra_bytes)
+                  bool already_cleared)
 {
     *keys_out = keys_a;
     *vals_out = vals_a;
@@ -439,7 +467,7 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
         return DSX_OK;
     if(count >= (1ll << 30))
         return DSX_ERR_TOO_LARGE;
-    int rc = sort32_clear(count, key_bits, kDepthSortTile, sort_ws, stream, clear_extra_bytes);
+    int rc = already_cleared ? DSX_OK : sort32_clear(count, key_bits, kDepthSortTile, sort_ws, stream);
     if(rc)
         return rc;
     const Sort32Workspace w = sort32_workspace(count, key_bits, kDepthSortTile);
@@ -711,47 +739,82 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
     uint32_t* ids_a = reinterpret_cast<uint32_t*>(base + o.ids_a);
     uint32_t* ids_b = reinterpret_cast<uint32_t*>(base + o.ids_b);
     uint32_t* block_sums = reinterpret_cast<uint32_t*>(base + o.block_sums);
-    uint32_t *ko, *vo;
-    // 32 key bits = 4 passes: the values (iota in pass 0) go b, a, b, a and end in ids_a
-    int rc = launch_sort32(n, 32, keys_a, ids_a, keys_b, ids_b, true, false, base + o.sort, stream, &ko, &vo,
-                           reinterpret_cast<const uint2*>(base + o.rects),
-                           reinterpret_cast<uint2*>(base + o.rects_sorted), o.ranges - o.cover);
+    // one fill zeroes the sort's counters and, right behind them, the corner grid
+    int rc = sort32_clear(n, 32, kDepthSortTile, base + o.sort, stream, o.ranges - o.cover);
     if(rc)
         return rc;
-    if(vo != ids_a)
-        return DSX_ERR_RUNTIME;
+
     // pairs per tile: digit histograms of the tile partition and the tile ranges that the second
-    // half of the forward needs (the grid was zeroed together with the sort's counters)
+    // half of the forward needs.  They depend on the rectangles only, not on the depth order,
+    // so they run on the helper stream beside the sort (fork after the fill, join at the end).
+    hipStream_t side = helper_stream();
+    hipEvent_t fork = nullptr, join = nullptr;
+    if(side)
     {
+        const bool ok = hipEventCreateWithFlags(&fork, hipEventDisableTiming) == hipSuccess &&
+                        hipEventCreateWithFlags(&join, hipEventDisableTiming) == hipSuccess &&
+                        hipEventRecord(fork, stream) == hipSuccess && hipStreamWaitEvent(side, fork, 0) == hipSuccess;
+        if(!ok)
+        {
+            (void)hipGetLastError();
+            side = nullptr;
+        }
+    }
+    {
+        hipStream_t cs = side ? side : stream;
         const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
         const int cells = (ntx + 1) * (nty + 1) + 1;
         int32_t* grid = reinterpret_cast<int32_t*>(base + o.cover);
         const int use_lds = cells <= kCoverLdsCells ? 1 : 0;
         const int64_t want = (n + kCoverThreads - 1) / kCoverThreads;
         {
-            DSX_TIMED("tile_cover_kernel", stream);
+            DSX_TIMED("tile_cover_kernel", cs);
             hipLaunchKernelGGL(tile_cover_kernel, dim3((unsigned)min((int64_t)kCoverBlocks, want)), dim3(kCoverThreads),
-                               use_lds ? (size_t)cells * 4 : 0, stream, reinterpret_cast<const uint2*>(base + o.rects), n,
+                               use_lds ? (size_t)cells * 4 : 0, cs, reinterpret_cast<const uint2*>(base + o.rects), n,
                                ntx, nty, use_lds, grid);
         }
-        DSX_LAUNCH_CHECK();
         {
-            DSX_TIMED("tile_counts_kernel", stream);
-            hipLaunchKernelGGL(tile_counts_kernel, dim3(1), dim3(kCoverThreads), use_lds ? (size_t)cells * 4 : 0, stream,
+            DSX_TIMED("tile_counts_kernel", cs);
+            hipLaunchKernelGGL(tile_counts_kernel, dim3(1), dim3(kCoverThreads), use_lds ? (size_t)cells * 4 : 0, cs,
                                grid, ntx, nty, use_lds, digits32(slot_bits(ntx * nty)),
                                reinterpret_cast<uint32_t*>(base + o.slot_hist),
                                reinterpret_cast<int32_t*>(base + o.ranges));
         }
-        DSX_LAUNCH_CHECK();
     }
+    bool joined = true;
+    if(side)
+        joined = hipEventRecord(join, side) == hipSuccess;
+    // the caller's stream takes the helper's work back in before this function returns
+    auto finish = [&](int status) {
+        if(side && joined)
+            joined = hipStreamWaitEvent(stream, join, 0) == hipSuccess;
+        if(fork)
+            (void)hipEventDestroy(fork);
+        if(join)
+            (void)hipEventDestroy(join);
+        return status ? status : (joined ? DSX_OK : DSX_ERR_RUNTIME);
+    };
+    if(hipGetLastError() != hipSuccess)
+        return finish(DSX_ERR_LAUNCH);
+
+    uint32_t *ko, *vo;
+    // 32 key bits = 4 passes: the values (iota in pass 0) go b, a, b, a and end in ids_a
+    rc = launch_sort32(n, 32, keys_a, ids_a, keys_b, ids_b, true, false, base + o.sort, stream, &ko, &vo,
+                       reinterpret_cast<const uint2*>(base + o.rects), reinterpret_cast<uint2*>(base + o.rects_sorted),
+                       true);
+    if(rc)
+        return finish(rc);
+    if(vo != ids_a)
+        return finish(DSX_ERR_RUNTIME);
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     {
         DSX_TIMED("ordered_block_sums_kernel", stream);
         hipLaunchKernelGGL(ordered_block_sums_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
                            reinterpret_cast<const uint2*>(base + o.rects_sorted), n, block_sums);
     }
-    DSX_LAUNCH_CHECK();
-    return launch_scan_u32(blocks, block_sums, block_sums + blocks, stream);
+    if(hipGetLastError() != hipSuccess)
+        return finish(DSX_ERR_LAUNCH);
+    return finish(launch_scan_u32(blocks, block_sums, block_sums + blocks, stream));
 }
 
 // ---------------------------------------------------------------------------------------

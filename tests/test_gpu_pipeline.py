@@ -118,6 +118,23 @@ def test_api_opacity_as_vector_and_empty_scene(oracle):
         assert (v.grad == 0).all()
 
 
+def test_api_on_a_side_stream_matches_the_default_stream():
+    """Every launch and the key-count copy go to torch's current stream: the result on a side
+    stream (default priority) equals the one on the default stream bit for bit in the forward
+    and within atomic reordering in the backward."""
+    sc = make_scene("cfg1", n=20000, width=320, height=200, sh_degree=3)
+    image0, radii0, leaves0 = api_run(sc, 2.0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        image1, radii1, leaves1 = api_run(sc, 2.0)
+    side.synchronize()
+    assert torch.equal(image0, image1) and torch.equal(radii0, radii1)
+    for k in leaves0:
+        a, b = leaves0[k].grad, leaves1[k].grad
+        assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * max(1.0, float(a.abs().max())))
+
+
 def test_api_precomputed_colors_and_cov3d(oracle):
     sc = make_scene("cfg0", n=5000, width=128, height=96, sh_degree=2)
     A = arrays(sc)
