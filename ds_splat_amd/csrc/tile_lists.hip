@@ -55,6 +55,26 @@ __device__ __forceinline__ uint32_t wave_incl_scan32(uint32_t v, int lane)
     return v;
 }
 
+// inclusive max-scan over the 64 lanes with data-parallel-primitive moves only (values >= 0,
+// lanes without a source keep 0): four shifts inside each row of 16, then the row broadcasts
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ uint32_t dpp_max(uint32_t v)
+{
+    const uint32_t moved = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kCtrl, kRowMask, 0xf, false);
+    return max(v, moved);
+}
+
+__device__ __forceinline__ uint32_t wave_incl_max_scan(uint32_t v)
+{
+    v = dpp_max<0x111, 0xf>(v); // row_shr:1
+    v = dpp_max<0x112, 0xf>(v); // row_shr:2
+    v = dpp_max<0x114, 0xf>(v); // row_shr:4
+    v = dpp_max<0x118, 0xf>(v); // row_shr:8
+    v = dpp_max<0x142, 0xa>(v); // row_bcast:15 into rows 1 and 3
+    v = dpp_max<0x143, 0xc>(v); // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 // lanes of the wavefront that hold the same (up to 8-bit) digit and are valid; uniform flow only
 __device__ __forceinline__ uint64_t match_digit8(uint32_t d, bool valid, int bits)
 {
@@ -837,10 +857,14 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     __shared__ float s_winv[kProjBlock];
     __shared__ uint32_t s_id[kProjBlock];
     __shared__ uint32_t wave_tot[kProjBlock / DSX_WAVE];
+    __shared__ uint32_t s_mark[kProjBlock];
+    __shared__ uint32_t s_wave_max[kProjBlock / DSX_WAVE];
+    static_assert(kProjBlock == 4 * DSX_WAVE, "four wavefronts per workgroup");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    s_mark[tid] = 0;
 
     // the tile ranges were derived from the rectangles before any pair existed: hand them out
     for(int j = blockIdx.x * kProjBlock + tid; j < range_count; j += gridDim.x * kProjBlock)
@@ -878,34 +902,51 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
 
         const uint32_t total = s_off[kProjBlock];
         const int64_t base = block_offsets[blk];
-        for(uint32_t j = tid; j < total && base + j < k; j += kProjBlock)
+        const uint32_t my_start = s_off[tid];
+        // Which Gaussian owns output j?  Every Gaussian that emits marks the output where its run
+        // starts with (its index + 1); the owner of j is the largest mark at or before j, i.e. an
+        // inclusive max-scan over the outputs (DPP inside the wavefront, LDS across wavefronts
+        // and across rounds of 256 outputs).  Costs a dozen VALU instructions per output
+        // instead of the eight dependent LDS reads of a binary search.
+        uint32_t carry = 0; // mark of the owner of the last output of the previous round
+        for(uint32_t j0 = 0; j0 < total; j0 += kProjBlock) // uniform
         {
-            // largest g with s_off[g] <= j
-            int lo = 0, hi = kProjBlock;
-            while(hi - lo > 1)
+            if(count && my_start >= j0 && my_start < j0 + kProjBlock)
+                s_mark[my_start - j0] = (uint32_t)tid + 1u;
+            __syncthreads();
+            uint32_t m = s_mark[tid];
+            s_mark[tid] = 0; // ready for the next round (and the next block)
+            m = wave_incl_max_scan(m);
+            if(lane == 63)
+                s_wave_max[wave] = m;
+            __syncthreads();
+            uint32_t before = carry;
+            for(int w = 0; w < wave; ++w)
+                before = max(before, s_wave_max[w]);
+            const uint32_t owner = max(m, before) - 1u; // every output has an owner: never 0 - 1
+            carry = max(max(max(s_wave_max[0], s_wave_max[1]), max(s_wave_max[2], s_wave_max[3])), carry);
+            const uint32_t j = j0 + tid;
+            if(j < total && base + j < k)
             {
-                const int mid = (lo + hi) >> 1;
-                if(s_off[mid] <= j)
-                    lo = mid;
-                else
-                    hi = mid;
+                const uint32_t r = j - s_off[owner];
+                const uint32_t w = s_w[owner];
+                uint32_t slot = 0;
+                if(w)
+                {
+                    // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
+                    uint32_t ry = (uint32_t)((float)r * s_winv[owner]);
+                    if(ry * w > r)
+                        --ry;
+                    else if((ry + 1) * w <= r)
+                        ++ry;
+                    const uint32_t rx = r - ry * w;
+                    slot = s_origin[owner] + ry * (uint32_t)ntx + rx;
+                }
+                slots[base + j] = (SlotT)slot;
+                ids[base + j] = (int32_t)s_id[owner];
             }
-            const uint32_t r = j - s_off[lo];
-            const uint32_t w = s_w[lo];
-            uint32_t slot = 0;
-            if(w)
-            {
-                // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
-                uint32_t ry = (uint32_t)((float)r * s_winv[lo]);
-                if(ry * w > r)
-                    --ry;
-                else if((ry + 1) * w <= r)
-                    ++ry;
-                const uint32_t rx = r - ry * w;
-                slot = s_origin[lo] + ry * (uint32_t)ntx + rx;
-            }
-            slots[base + j] = (SlotT)slot;
-            ids[base + j] = (int32_t)s_id[lo];
+            // (the next round's marks are written after this round's reads of s_wave_max: the
+            // barrier after them orders both)
         }
     }
 }
