@@ -95,15 +95,6 @@ struct SortWorkspace
 };
 SortWorkspace sort_workspace(int64_t k, int num_tiles);
 
-struct ForwardWorkspace
-{
-    size_t keys;   // int64[k]   emitted / sorted keys
-    size_t values; // int32[k]   only used when the pass count is odd (ping-pong parity)
-    size_t sort;   // SortWorkspace
-    size_t bytes;
-};
-ForwardWorkspace forward_workspace(int64_t k, int num_tiles);
-
 // ---- 32-bit radix sort (depth order of the Gaussians, tile partition of the tile lists) ----
 constexpr int kBits32 = 8;
 constexpr int kBins32 = 1 << kBits32;

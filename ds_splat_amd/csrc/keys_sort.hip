@@ -258,21 +258,6 @@ SortWorkspace sort_workspace(int64_t k, int num_tiles)
     return w;
 }
 
-ForwardWorkspace forward_workspace(int64_t k, int num_tiles)
-{
-    auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
-    ForwardWorkspace w;
-    size_t off = 0;
-    w.keys = off;
-    off = align(off + (size_t)k * 8);
-    w.values = off;
-    off = align(off + (size_t)k * 4);
-    w.sort = off;
-    off += sort_workspace(k, num_tiles).bytes;
-    w.bytes = align(off);
-    return w;
-}
-
 struct DigitPlan
 {
     int passes;
