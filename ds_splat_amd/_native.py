@@ -57,6 +57,7 @@ SIGNATURES = {
     "dsx_sort_pairs_u32": (C.c_int, [_I64, _I32, _P, _P, _P, C.c_size_t, _P]),
     "dsx_depth_order": (C.c_int, [_CAM, _I64, _P, C.c_size_t, _P]),
     "dsx_order_view": (C.c_int, [_I64, _P, C.POINTER(_P), C.POINTER(_P)]),
+    "dsx_sort_flags": (C.c_int, [_I64, _I64, _I32, _I32, _P, _P, C.POINTER(_P), C.POINTER(_P)]),
     "dsx_tile_lists": (C.c_int, [_CAM, _I64, _I64, _P, _P, _P, _P, C.c_size_t, _P]),
     "dsx_blend_fwd": (C.c_int, [_CAM] + [_P] * 6 + [_P]),
     "dsx_blend_bwd": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P]),

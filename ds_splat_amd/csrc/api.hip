@@ -328,6 +328,38 @@ extern "C" int dsx_order_view(int64_t n, const void* order, const uint32_t** dep
     return DSX_OK;
 }
 
+extern "C" int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t height, const void* order,
+                              const void* workspace, const uint32_t** depth_sort_flag,
+                              const uint32_t** partition_flag)
+{
+    if(n < 0 || k < 0 || width <= 0 || height <= 0)
+        return DSX_ERR_BAD_ARG;
+    if(depth_sort_flag)
+    {
+        *depth_sort_flag = nullptr;
+        if(order && n > 0)
+        {
+            const OrderLayout o = order_layout(n);
+            const Sort32Workspace w = sort32_workspace(n, 32, kDepthSortTile);
+            *depth_sort_flag =
+                reinterpret_cast<const uint32_t*>(static_cast<const char*>(order) + o.sort + w.counters) + w.passes;
+        }
+    }
+    if(partition_flag)
+    {
+        *partition_flag = nullptr;
+        if(workspace && k > 0)
+        {
+            const int tiles = dsx_num_tiles(width, height);
+            const ListsWorkspace lw = lists_workspace(k, tiles);
+            const Sort32Workspace w = sort32_workspace(k, slot_bits(tiles), kListSortTile);
+            *partition_flag =
+                reinterpret_cast<const uint32_t*>(static_cast<const char*>(workspace) + lw.sort + w.counters) + w.passes;
+        }
+    }
+    return DSX_OK;
+}
+
 extern "C" int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
                               int32_t* ranges, void* workspace, size_t workspace_bytes, void* stream)
 {

@@ -103,8 +103,9 @@ def depth_order(cam, n, order):
     return as_i32[o0:o0 + n], as_i32[o1:o1 + int(lib.dsx_num_blocks(n)) + 1]
 
 
-def tile_lists(cam, n, k, order):
-    """(sorted_ids[k], ranges[T+1]) from a depth-ordered `order` buffer."""
+def tile_lists(cam, n, k, order, return_flags=False):
+    """(sorted_ids[k], ranges[T+1]) from a depth-ordered `order` buffer; with return_flags also
+    the two give-up flags of the chained scans (depth sort, tile partition) as Python ints."""
     lib = N.load()
     dev = order.device
     sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
@@ -112,7 +113,14 @@ def tile_lists(cam, n, k, order):
     nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
     N.check(lib.dsx_tile_lists(cam.ref, n, k, _ptr(order), _ptr(sorted_ids), _ptr(ranges), _ptr(ws), nbytes, _stream()))
-    return sorted_ids, ranges
+    if not return_flags:
+        return sorted_ids, ranges
+    p_a, p_b = C.c_void_p(), C.c_void_p()
+    N.check(lib.dsx_sort_flags(n, k, cam.width, cam.height, _ptr(order), _ptr(ws) if k > 0 else None,
+                               C.byref(p_a), C.byref(p_b)))
+    torch.cuda.synchronize()
+    read = lambda t, p: 0 if not p.value else int(t.view(torch.int32)[(p.value - t.data_ptr()) // 4].item())
+    return sorted_ids, ranges, (read(order, p_a), read(ws, p_b))
 
 
 def sort_pairs_u32(keys, values, key_bits=32):

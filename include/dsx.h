@@ -148,6 +148,17 @@ int dsx_sort_pairs_u32(int64_t count, int32_t key_bits, uint32_t* keys, uint32_t
 int dsx_depth_order(const dsx_camera* cam, int64_t n, void* order, size_t order_bytes, void* stream);
 int dsx_order_view(int64_t n, const void* order, const uint32_t** depth_order,
                    const uint32_t** block_offsets);
+/* The chained scan of a sort pass waits for its predecessor tile with a BOUNDED spin; a tile that
+ * gives up (it never should: tiles take their numbers in start order) sets a flag instead of
+ * hanging the GPU, and the result of that sort is then wrong.  This returns the device
+ * addresses of the two flags (uint32, non-zero = gave up) inside an `order` buffer after
+ * dsx_depth_order / dsx_forward_project and inside a `workspace` after dsx_tile_lists /
+ * dsx_forward_finish, for callers that want to check after synchronising.  Either output may
+ * be NULL; an address is NULL when its buffer is NULL or empty.  No counterpart in the
+ * reference (thrust's sort has no such wait). */
+int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t height, const void* order,
+                   const void* workspace, const uint32_t** depth_sort_flag,
+                   const uint32_t** partition_flag);
 int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const void* order,
                    int32_t* sorted_ids, int32_t* ranges, void* workspace, size_t workspace_bytes,
                    void* stream);

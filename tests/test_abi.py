@@ -66,6 +66,8 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.dsx_sort_pairs_u32(10, 33, 1, 1, 1, 0, None) == -1
     assert lib.dsx_sort_pairs_u32(10, 32, 1, 1, 1, 0, None) == -5
     assert lib.dsx_depth_order(None, 10, None, 0, None) == -1
+    assert lib.dsx_sort_flags(-1, 0, 16, 16, None, None, None, None) == -1
+    assert lib.dsx_sort_flags(10, 10, 16, 16, None, None, None, None) == 0
 
 
 def test_python_api_surface():

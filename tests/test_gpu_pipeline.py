@@ -64,7 +64,7 @@ def check_grads(leaves, B, ok):
 
 
 @pytest.mark.parametrize("name,n,W,H,deg,scale_mul,bg", [
-    ("cfg0", 16384, 256, 256, 0, 1.0, None),            # BASELINE config 0 at full size
+    ("cfg0", 16384, 256, 256, 0, 1.0, None),            # workload cfg0 at full size
     ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9)),
     ("cfg1", 40000, 480, 270, 3, 1.0, None),            # config 1 distributions, reduced size
     ("cfg4", 3000, 320, 180, 3, 0.5, None),             # heavy-overlap distributions, reduced size
@@ -214,7 +214,8 @@ def test_full_size_properties_cfg2():
     assert int(offsets[-1]) == k
     d_sorted = (depth_bits & 0xFFFFFFFF)[perm.to(torch.int64)]       # unsigned order of the depth bits
     assert (d_sorted[1:] >= d_sorted[:-1]).all()
-    ids_fast, ranges_fast = stages.tile_lists(cam, n, k, order)
+    ids_fast, ranges_fast, flags = stages.tile_lists(cam, n, k, order, return_flags=True)
+    assert flags == (0, 0)
     assert torch.equal(ids_fast, vals) and torch.equal(ranges_fast, ranges)
     del ids_fast, ranges_fast, perm, offsets, d_sorted
     tile_of = (keys >> 32).to(torch.int64)

@@ -267,8 +267,8 @@ def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip):
     sums = np.concatenate([tt_sorted, pad]).reshape(-1, 256).sum(1)
     assert (offsets.cpu().numpy().astype(np.int64) == np.concatenate([[0], np.cumsum(sums)])).all()
     assert int(offsets[-1]) == k
-    ids, ranges = st_.tile_lists(cam, n, k, order)
-    torch.cuda.synchronize()
+    ids, ranges, flags = st_.tile_lists(cam, n, k, order, return_flags=True)
+    assert flags == (0, 0)                       # no chained scan gave up waiting
     assert (ids.cpu().numpy() == S["sorted_ids"]).all()
     assert (ranges.cpu().numpy() == S["ranges"]).all()
     if flip:
