@@ -175,6 +175,35 @@ def test_forward_core_raw_pointer_entry(oracle):
     np.testing.assert_allclose(image.cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("name,n,W,H,scale_mul", [
+    ("cfg3", 200_000, 7680, 4320, 1.0),     # 129600 tiles: 32-bit slots, 3 partition passes, corner grid in global memory
+    ("cfg1", 300, 8000, 8000, 30.0),        # 250000 tiles, rectangles of thousands of tiles
+    ("cfg2", 300, 16, 16, 1.0),             # one tile
+    ("cfg4", 100_000, 1920, 1080, 1.0),     # ~850 tiles per Gaussian
+])
+def test_forward_lists_equal_the_64_bit_route(name, n, W, H, scale_mul):
+    """The whole forward's sorted ids and ranges (depth order + tile partition) against the
+    reference-shaped route (64-bit keys, radix sort, ranges from keys) at shapes the oracle is
+    too slow for."""
+    from ds_splat_amd import stages
+    sc = make_scene(name, n=n, width=W, height=H)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    cam = stages.camera_from_scene(sc, DEV)
+    img, st = stages.forward(cam, t["means_3d"], t["scales"] * scale_mul, t["rotations"], t["opacities"], t["shs"])
+    k = st.num_keys
+    tiles = st.splats[:, 11].view(torch.int32).to(torch.int64).clone()
+    tiles[-1] = 0
+    assert k == int(tiles.sum().item()) > 0
+    block_sums = torch.cat([tiles, torch.zeros((-n) % 256, dtype=torch.int64, device=DEV)]).view(-1, 256).sum(1)
+    block_sums = block_sums.to(torch.int32)
+    stages.scan_u32(block_sums)
+    keys, vals = stages.emit_keys(cam, n, k, st.splats, block_sums)
+    stages.sort_pairs(keys, vals, cam.num_tiles)
+    ranges = stages.tile_ranges(keys, cam.num_tiles)
+    assert torch.equal(vals, st.sorted_ids) and torch.equal(ranges, st.ranges)
+    assert torch.isfinite(img).all()
+
+
 # ------------------------------------------------------------------------- properties at full size
 def test_full_size_properties_cfg2():
     """3M Gaussians, 1920x1080, SH3 (the headline shape): properties that need no oracle."""
