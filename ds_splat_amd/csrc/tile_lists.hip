@@ -137,19 +137,25 @@ __global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const KeyT* __re
 #pragma unroll
         for(int it = 0; it < kHist32Items; ++it)
         {
-            const uint64_t vmask = __ballot(valid[it]); // valid lanes are a prefix of the wavefront
-            const int nvalid = __popcll(vmask);
-            for(int p = 0; p < plan.passes; ++p)
+            // lower digits: plain LDS atomics (values differ from lane to lane).  The most
+            // significant digit takes few values (the exponent byte of depths, the high bits of
+            // a tile slot): one add per distinct value of the wavefront, after a ballot, because
+            // LDS atomics on one address serialise.
+            for(int p = 0; p + 1 < plan.passes; ++p)
+                if(valid[it])
+                    atomicAdd(&hist[p * kBins32 + ((s[it] >> plan.shift[p]) & plan.mask[p])], 1u);
             {
+                const int p = plan.passes - 1;
                 const uint32_t d = (s[it] >> plan.shift[p]) & plan.mask[p];
-                const uint32_t below = lane_below32(d, ~d);
-                const bool head = valid[it] && (lane == 0 || below != d);
-                const uint64_t heads = __ballot(head);
-                if(head)
+                uint64_t todo = __ballot(valid[it]);
+                while(todo)
                 {
-                    const uint64_t above = lane == 63 ? 0ull : (heads >> (lane + 1));
-                    const int run = above ? __ffsll((unsigned long long)above) : nvalid - lane;
-                    atomicAdd(&hist[p * kBins32 + d], (uint32_t)run);
+                    const int leader = __builtin_ctzll(todo);
+                    const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)d, leader);
+                    const uint64_t same = __ballot(valid[it] && d == dl);
+                    if(lane == leader)
+                        atomicAdd(&hist[p * kBins32 + dl], (uint32_t)__popcll(same));
+                    todo &= ~same;
                 }
             }
         }
@@ -158,25 +164,6 @@ __global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const KeyT* __re
     for(int j = tid; j < plan.passes * kBins32; j += kHist32Threads)
         if(hist[j])
             atomicAdd(&global_hist[j], hist[j]);
-}
-
-// exclusive scan of each pass's 256 bins (one workgroup per pass)
-__global__ __launch_bounds__(kBins32) void hist32_scan_kernel(const uint32_t* counts, uint32_t* global_hist)
-{
-    __shared__ uint32_t wave_tot[kBins32 / DSX_WAVE];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    uint32_t* h = global_hist + blockIdx.x * kBins32;
-    const uint32_t v = counts[blockIdx.x * kBins32 + tid];
-    const uint32_t incl = wave_incl_scan32(v, lane);
-    if(lane == 63)
-        wave_tot[wave] = incl;
-    __syncthreads();
-    uint32_t prefix = 0;
-    for(int w = 0; w < wave; ++w)
-        prefix += wave_tot[w];
-    h[tid] = prefix + incl - v;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -201,7 +188,7 @@ static_assert(kDepthSortTile <= 65535 && kListSortTile <= 65535, "u16 ranks");
 template <typename KeyT, int kSort32Threads, int kSort32Items>
 __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     const KeyT* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, KeyT* __restrict__ keys_out,
-    uint32_t* __restrict__ vals_out, int64_t count, int shift, uint32_t mask, const uint32_t* __restrict__ hist_excl,
+    uint32_t* __restrict__ vals_out, int64_t count, int shift, uint32_t mask, const uint32_t* __restrict__ hist_counts,
     uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag, const uint2* __restrict__ gather_src,
     uint2* __restrict__ gather_dst)
 {
@@ -212,6 +199,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     __shared__ uint32_t s_digit_start[kBins32];
     __shared__ uint32_t s_gbase[kBins32];
     __shared__ uint32_t s_wave_tot[kBins32 / DSX_WAVE];
+    __shared__ uint32_t s_hist_tot[kBins32 / DSX_WAVE];
     __shared__ uint32_t s_tile;
 
     const int tid = threadIdx.x;
@@ -267,6 +255,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     // ---- per-digit totals of the tile (thread d <-> digit d), wave offsets, digit starts ----
     const bool digit_thread = tid < kBins32; // thread d owns digit d (bins above the mask stay empty)
     uint32_t total = 0;
+    uint32_t hist_excl = 0;
     uint32_t* my_status = status + tile * kBins32 + (digit_thread ? tid : 0);
     if(digit_thread)
     {
@@ -283,14 +272,25 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
         if(lane == 63)
             s_wave_tot[wave] = incl;
         s_gbase[tid] = incl - total; // wave-local exclusive prefix, completed after the barrier
+        // the digit's place in the whole output: exclusive scan of the pass's histogram (every
+        // tile redoes this 256-entry scan; that is cheaper than a kernel launch of its own)
+        const uint32_t hcount = hist_counts[tid];
+        const uint32_t hincl = wave_incl_scan32(hcount, lane);
+        if(lane == 63)
+            s_hist_tot[wave] = hincl;
+        hist_excl = hincl - hcount;
     }
     __syncthreads();
     if(digit_thread)
     {
-        uint32_t prefix = 0;
+        uint32_t prefix = 0, hprefix = 0;
         for(int w = 0; w < wave; ++w)
+        {
             prefix += s_wave_tot[w];
+            hprefix += s_hist_tot[w];
+        }
         s_digit_start[tid] = prefix + s_gbase[tid];
+        hist_excl += hprefix;
     }
     __syncthreads();
 
@@ -351,7 +351,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
             __hip_atomic_store(my_status, ((excl + total) & kValueMask32) | kFlagInclusive32, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
         }
-        s_gbase[tid] = hist_excl[tid] + excl - s_digit_start[tid];
+        s_gbase[tid] = hist_excl + excl - s_digit_start[tid];
     }
     __syncthreads();
 
@@ -440,12 +440,7 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
     uint32_t* hist = reinterpret_cast<uint32_t*>(base + w.hist);
     uint32_t* counters = reinterpret_cast<uint32_t*>(base + w.counters);
     uint32_t* status = reinterpret_cast<uint32_t*>(base + w.status);
-    {
-        DSX_TIMED("hist32_scan_kernel", stream);
-        hipLaunchKernelGGL(hist32_scan_kernel, dim3(w.passes), dim3(kBins32), 0, stream,
-                           counts ? counts : (const uint32_t*)hist, hist);
-    }
-    DSX_LAUNCH_CHECK();
+    const uint32_t* raw = counts ? counts : (const uint32_t*)hist; // the passes scan their histogram themselves
     KeyT* kin = keys_a;
     uint32_t* vin = vals_a;
     KeyT* kout = keys_b;
@@ -458,7 +453,7 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
             hipLaunchKernelGGL((onesweep32_kernel<KeyT, kThreads, kItems>), dim3((unsigned)w.tiles), dim3(kThreads), 0, stream,
                                (const KeyT*)kin, (const uint32_t*)((p == 0 && iota_values) ? nullptr : vin),
                                (last && !keep_keys) ? (KeyT*)nullptr : kout, vout, count, plan.shift[p], plan.mask[p],
-                               (const uint32_t*)(hist + p * kBins32), status + (size_t)p * w.tiles * kBins32,
+                               raw + p * kBins32, status + (size_t)p * w.tiles * kBins32,
                                counters + p, counters + w.passes, last ? gather_src : (const uint2*)nullptr,
                                last ? gather_dst : (uint2*)nullptr);
         }
