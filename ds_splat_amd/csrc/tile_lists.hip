@@ -148,15 +148,19 @@ __global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const KeyT* __re
                 const int p = plan.passes - 1;
                 const uint32_t d = (s[it] >> plan.shift[p]) & plan.mask[p];
                 uint64_t todo = __ballot(valid[it]);
-                while(todo)
+                for(int round = 0; round < 8 && todo; ++round)
                 {
                     const int leader = __builtin_ctzll(todo);
                     const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)d, leader);
-                    const uint64_t same = __ballot(valid[it] && d == dl);
+                    const uint64_t same = __ballot(valid[it] && d == dl) & todo;
                     if(lane == leader)
                         atomicAdd(&hist[p * kBins32 + dl], (uint32_t)__popcll(same));
                     todo &= ~same;
                 }
+                // more than eight distinct values in the wavefront: the digit is not a
+                // concentrated one after all, the rest goes the plain way
+                if((todo >> lane) & 1)
+                    atomicAdd(&hist[p * kBins32 + d], 1u);
             }
         }
     }
