@@ -84,6 +84,14 @@ class DsRasterizerFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, means_3d, means_2d, shs, colors_precomp, opacities, scales, rotations, cov_3d_precomp,
                 raster_settings):
+        image, radii, _ = DsRasterizerFunction.run_forward(ctx, means_3d, means_2d, shs, colors_precomp, opacities,
+                                                           scales, rotations, cov_3d_precomp, raster_settings)
+        return image, radii
+
+    @staticmethod
+    def run_forward(ctx, means_3d, means_2d, shs, colors_precomp, opacities, scales, rotations, cov_3d_precomp,
+                    raster_settings):
+        """The forward proper; also returns final_T (for wrappers that composite a background)."""
         s = raster_settings
         _validate(means_3d, means_2d, shs, colors_precomp, opacities, scales, rotations, cov_3d_precomp, s)
         ext = _native.load_torch_ext()
@@ -100,7 +108,7 @@ class DsRasterizerFunction(torch.autograd.Function):
         ctx.num_keys = sorted_ids.numel()
         ctx.save_for_backward(means_3d, scales, rotations, splats, cov3d, radii, ranges, sorted_ids, final_T, final_idx)
         ctx.mark_non_differentiable(radii)
-        return image, radii
+        return image, radii, final_T
 
     @staticmethod
     def backward(ctx, rendered_img_grad, _):

@@ -83,6 +83,36 @@ def test_python_api_surface():
                    "cov_3d_precomp"]
 
 
+def test_scene_dump_round_trip(tmp_path):
+    """The TorchScript scene dump carries the attribute names the reference's timing harness
+    reads (tests/rasterizer_test.cpp:147-168)."""
+    import torch
+    from ds_splat_amd import scene_io
+    from ds_splat_amd.synthetic import make_scene
+    sc = make_scene("cfg0", n=64, width=48, height=32, sh_degree=2)
+    path = str(tmp_path / "scene.pt")
+    scene_io.save_scene(path, scene_io.scene_from_synthetic(sc))
+    m = torch.jit.load(path)
+    for name in ("means_3d", "means_2d", "shs", "opacities", "scales", "rotations", "viewmatrix", "projmatrix",
+                 "campos", "image_height", "image_width", "tanfovx", "tanfovy", "scale_modifier", "sh_degree"):
+        assert hasattr(m, name), name
+    d = scene_io.load_scene(path)
+    assert d["image_height"] == 32 and d["image_width"] == 48 and d["sh_degree"] == 2
+    assert torch.equal(d["shs"], sc["shs"]) and torch.equal(d["projmatrix"], sc["projmatrix"])
+    assert abs(d["tanfovx"] - sc["tanfovx"]) < 1e-12
+
+
+def test_inria_adaptor_surface():
+    import inspect
+    from ds_splat_amd import inria_compat
+    assert inria_compat.GaussianRasterizationSettings._fields == (
+        "image_height", "image_width", "tanfovx", "tanfovy", "bg", "scale_modifier", "viewmatrix", "projmatrix",
+        "sh_degree", "campos", "prefiltered", "debug")
+    sig = list(inspect.signature(inria_compat.GaussianRasterizer.forward).parameters)
+    assert sig == ["self", "means3D", "means2D", "opacities", "shs", "colors_precomp", "scales", "rotations",
+                   "cov3D_precomp"]
+
+
 def test_input_checks_mirror_the_reference_messages():
     import torch
     from ds_splat import GaussianRasterizationSettings, GaussianRasterizer

@@ -135,6 +135,38 @@ def test_api_on_a_side_stream_matches_the_default_stream():
         assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * max(1.0, float(a.abs().max())))
 
 
+def test_inria_adaptor_composites_the_background_and_keeps_the_gradients():
+    """Channel-first image = HWC image + final_T * bg; gradients equal those of the wrapped API
+    for the same upstream gradient (the backward kernel's background term is the derivative of
+    exactly that product)."""
+    from ds_splat_amd import inria_compat, stages
+    sc = make_scene("cfg1", n=20000, width=320, height=200, sh_degree=3)
+    bg = (0.3, 0.6, 0.1)
+    image, radii, leaves = api_run(sc, 2.0, bg=bg)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    settings = inria_compat.GaussianRasterizationSettings(
+        image_height=sc["height"], image_width=sc["width"], tanfovx=sc["tanfovx"], tanfovy=sc["tanfovy"],
+        bg=torch.tensor(bg, dtype=torch.float32, device=DEV), scale_modifier=1.0, viewmatrix=t["viewmatrix"],
+        projmatrix=t["projmatrix"], sh_degree=sc["sh_degree"], campos=t["campos"])
+    p = dict(means=t["means_3d"].clone().requires_grad_(True), shs=t["shs"].clone().requires_grad_(True),
+             opac=t["opacities"].clone().requires_grad_(True), scales=(t["scales"] * 2.0).clone().requires_grad_(True),
+             rots=t["rotations"].clone().requires_grad_(True))
+    color, radii2 = inria_compat.GaussianRasterizer(settings)(
+        means3D=p["means"], means2D=torch.zeros_like(p["means"]), opacities=p["opac"], shs=p["shs"],
+        scales=p["scales"], rotations=p["rots"])
+    assert color.shape == (3, sc["height"], sc["width"]) and torch.equal(radii, radii2)
+    cam = stages.camera_from_scene(sc, DEV, bg=torch.tensor(bg))
+    _, st = stages.forward(cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
+    want = image.detach() + st.final_T.unsqueeze(-1) * torch.tensor(bg, device=DEV).view(1, 1, 3)
+    assert torch.allclose(color.detach().permute(1, 2, 0), want, rtol=0, atol=1e-6)
+    assert (st.final_T > 0.5).any() and float((color.detach().permute(1, 2, 0) - image.detach()).abs().max()) > 0.05
+    color.backward(t["v_image"].permute(2, 0, 1))
+    torch.cuda.synchronize()
+    for k in p:
+        a, b = leaves[k].grad, p[k].grad
+        assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * max(1.0, float(a.abs().max()))), k
+
+
 def test_api_precomputed_colors_and_cov3d(oracle):
     sc = make_scene("cfg0", n=5000, width=128, height=96, sh_degree=2)
     A = arrays(sc)
