@@ -93,11 +93,6 @@ __device__ __forceinline__ uint64_t match_digit8(uint32_t d, bool valid, int bit
     return ((uint64_t)hi << 32) | lo;
 }
 
-__device__ __forceinline__ uint32_t lane_below32(uint32_t v, uint32_t first)
-{
-    return (uint32_t)__builtin_amdgcn_update_dpp((int)first, (int)v, 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
-}
-
 // ---------------------------------------------------------------------------------------
 // histograms of every digit in one read (run-length merged: neighbouring keys often share a digit)
 // ---------------------------------------------------------------------------------------
