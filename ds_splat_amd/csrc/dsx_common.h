@@ -98,9 +98,10 @@ SortWorkspace sort_workspace(int64_t k, int num_tiles);
 // ---- 32-bit radix sort (depth order of the Gaussians, tile partition of the tile lists) ----
 constexpr int kBits32 = 8;
 constexpr int kBins32 = 1 << kBits32;
-// Two geometries of the same pass kernel: the depth sort of the N Gaussians (few keys: small
-// tiles so that the launch fills the chip) and the partition of the K pairs (large tiles: the
-// look-back traffic falls with the number of tiles).
+// Two geometries of the same pass kernel: the depth sort of the N Gaussians (few keys: 8192-key
+// tiles so that the launch fills the chip) and the partition of the K pairs (12288-key tiles of
+// 1024 threads, two blocks per compute unit: the look-back traffic falls with the number of
+// tiles).  A tile must stay below 65536 keys (positions inside a tile are kept as 16 bits).
 #ifndef DSX_NSORT_THREADS
 #define DSX_NSORT_THREADS 512
 #endif
@@ -108,10 +109,10 @@ constexpr int kBins32 = 1 << kBits32;
 #define DSX_NSORT_ITEMS 16
 #endif
 #ifndef DSX_KSORT_THREADS
-#define DSX_KSORT_THREADS 512
+#define DSX_KSORT_THREADS 1024
 #endif
 #ifndef DSX_KSORT_ITEMS
-#define DSX_KSORT_ITEMS 16
+#define DSX_KSORT_ITEMS 12
 #endif
 constexpr int kDepthSortThreads = DSX_NSORT_THREADS;
 constexpr int kDepthSortItems = DSX_NSORT_ITEMS;

@@ -215,21 +215,19 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     const int tile_n = (int)min((int64_t)kSort32Tile, count - tile_base);
     const int bits = 32 - __builtin_clz(mask); // mask = 2^bits - 1, bits >= 1
 
-    // ---- load (striped inside each wavefront: coalesced, order = (item, lane)) -------------
+    // ---- load the keys (striped inside each wavefront: coalesced, order = (item, lane)) -----
+    // Registers are what limits the blocks per compute unit here, so a thread keeps little per
+    // item: the key while it is ranked, the rank as 16 bits, the digit as 8 bits; the value is
+    // fetched only once the key registers are free.
     uint32_t key[kSort32Items];
-    uint32_t val[kSort32Items];
-    uint32_t pos[kSort32Items];
+    uint32_t pos2[(kSort32Items + 1) / 2]; // two 16-bit positions per register
 #pragma unroll
     for(int it = 0; it < kSort32Items; ++it)
     {
         const int local = wave * (kSort32Items * 64) + it * 64 + lane;
         key[it] = 0;
-        val[it] = 0;
         if(local < tile_n)
-        {
             key[it] = (uint32_t)__builtin_nontemporal_load(keys_in + tile_base + local);
-            val[it] = vals_in ? __builtin_nontemporal_load(vals_in + tile_base + local) : (uint32_t)(tile_base + local);
-        }
     }
 
     // ---- wave-local stable rank ------------------------------------------------------------
@@ -247,7 +245,13 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
         if(valid && below == 0)
             wh[d] = (uint16_t)(old + (uint32_t)__popcll(m));
         __builtin_amdgcn_wave_barrier();
-        pos[it] = old + below;
+        if(it & 1)
+            pos2[it >> 1] |= (old + below) << 16;
+        else
+            pos2[it >> 1] = old + below;
+        // pin the packed form here and make the key opaque: otherwise the compiler carries each
+        // item's digit, histogram address and old count into the next phase in registers of their own
+        asm volatile("" : "+v"(pos2[it >> 1]), "+v"(key[it]));
     }
     __syncthreads();
 
@@ -301,9 +305,21 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
         if(local < tile_n)
         {
             const uint32_t d = (key[it] >> shift) & mask;
-            pos[it] += s_digit_start[d] + s_whist[wave][d];
-            s_keys[pos[it]] = key[it];
+            const uint32_t p = ((pos2[it >> 1] >> (16 * (it & 1))) & 0xffffu) + s_digit_start[d] + s_whist[wave][d];
+            s_keys[p] = key[it];
+            pos2[it >> 1] = (it & 1) ? ((pos2[it >> 1] & 0xffffu) | (p << 16)) : ((pos2[it >> 1] & 0xffff0000u) | p);
         }
+    }
+
+    // ---- the values: in flight while the chained scan runs ---------------------------------
+    uint32_t val[kSort32Items];
+#pragma unroll
+    for(int it = 0; it < kSort32Items; ++it)
+    {
+        const int local = wave * (kSort32Items * 64) + it * 64 + lane;
+        val[it] = 0;
+        if(local < tile_n)
+            val[it] = vals_in ? __builtin_nontemporal_load(vals_in + tile_base + local) : (uint32_t)(tile_base + local);
     }
 
     // ---- chained scan over earlier tiles (decoupled look-back), one thread per digit -------
@@ -355,18 +371,23 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     __syncthreads();
 
     // ---- scatter keys: consecutive threads -> consecutive addresses inside a digit's run ----
-    uint32_t out[kSort32Items];
+    uint32_t dig4[(kSort32Items + 3) / 4]; // the digit of the key at tile position it * threads + tid, 8 bits each
 #pragma unroll
     for(int it = 0; it < kSort32Items; ++it)
     {
         const int j = it * kSort32Threads + tid;
-        out[it] = 0;
+        if((it & 3) == 0)
+        {
+            __builtin_amdgcn_sched_barrier(0); // four items in flight at a time: registers, not latency, are scarce
+            dig4[it >> 2] = 0;
+        }
         if(j < tile_n)
         {
             const uint32_t kk = s_keys[j];
-            out[it] = s_gbase[(kk >> shift) & mask] + (uint32_t)j;
+            const uint32_t d = (kk >> shift) & mask;
+            dig4[it >> 2] |= d << (8 * (it & 3));
             if(keys_out)
-                keys_out[out[it]] = (KeyT)kk;
+                keys_out[s_gbase[d] + (uint32_t)j] = (KeyT)kk;
         }
     }
     __syncthreads();
@@ -377,21 +398,24 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     {
         const int local = wave * (kSort32Items * 64) + it * 64 + lane;
         if(local < tile_n)
-            s_keys[pos[it]] = val[it];
+            s_keys[(pos2[it >> 1] >> (16 * (it & 1))) & 0xffffu] = val[it];
     }
     __syncthreads();
 #pragma unroll
     for(int it = 0; it < kSort32Items; ++it)
     {
         const int j = it * kSort32Threads + tid;
+        if((it & 3) == 0)
+            __builtin_amdgcn_sched_barrier(0);
         if(j < tile_n)
         {
             const uint32_t v = s_keys[j];
-            vals_out[out[it]] = v;
+            const uint32_t out = s_gbase[(dig4[it >> 2] >> (8 * (it & 3))) & 0xffu] + (uint32_t)j;
+            vals_out[out] = v;
             // optional: a per-value record follows its value to the sorted position (the random
             // gather overlaps with the scatter traffic of the pass)
             if(gather_src)
-                gather_dst[out[it]] = gather_src[v];
+                gather_dst[out] = gather_src[v];
         }
     }
 }
