@@ -8,7 +8,7 @@
 //   3. a STABLE partition of the K pairs by tile slot alone (2 passes of <= 8 bits).
 // Keys with a negative depth carry tile field -1 in the 64-bit scheme and sort first by their
 // unsigned depth bits; here they take slot 0 and real tiles move up by one, and the unsigned
-// depth order of step 1 keeps their relative order.  HBM traffic: 8 bytes per pair written
+// depth order of step 1 keeps their relative order.  HBM traffic: 6 or 8 bytes per pair written
 // once and moved twice, instead of 12 bytes moved five times.
 #include "dsx_common.h"
 
