@@ -75,17 +75,17 @@ __device__ __forceinline__ uint32_t wave_incl_max_scan(uint32_t v)
     return v;
 }
 
-// lanes of the wavefront that hold the same (up to 8-bit) digit and are valid; uniform flow only
-__device__ __forceinline__ uint64_t match_digit8(uint32_t d, bool valid, int bits)
+// lanes of the wavefront that hold the same (up to 8-bit) digit; uniform flow only
+__device__ __forceinline__ uint64_t match_digit8(uint32_t d, int bits)
 {
-    const uint64_t v = __ballot(valid);
-    uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+    uint32_t lo = 0xffffffffu, hi = 0xffffffffu;
 #pragma unroll
     for(int b = 0; b < kBits32; ++b)
     {
         if(b >= bits) // uniform: digits narrower than 8 bits need fewer rounds
             break;
-        const uint32_t x = (uint32_t)(((int32_t)(d << (31 - b))) >> 31); // all ones where bit b is set
+        uint32_t x = (uint32_t)(((int32_t)(d << (31 - b))) >> 31); // all ones where bit b is set
+        asm volatile("" : "+v"(x)); // the ballot tests x itself (one compare), not a second copy of the bit
         const uint64_t m = __ballot(x != 0);
         lo &= ~((uint32_t)m ^ x);
         hi &= ~((uint32_t)(m >> 32) ^ x);
@@ -225,7 +225,11 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     for(int it = 0; it < kSort32Items; ++it)
     {
         const int local = wave * (kSort32Items * 64) + it * 64 + lane;
-        key[it] = 0;
+        // Places past the end of the input (last tile only) hold all-ones keys: they take the
+        // highest digit and, being last in tile order, rank behind every real key, so the real
+        // keys' positions are what they would be without them and no phase needs a validity test
+        // except the stores (tile position < tile_n).
+        key[it] = 0xffffffffu;
         if(local < tile_n)
             key[it] = (uint32_t)__builtin_nontemporal_load(keys_in + tile_base + local);
     }
@@ -235,14 +239,12 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
 #pragma unroll
     for(int it = 0; it < kSort32Items; ++it)
     {
-        const int local = wave * (kSort32Items * 64) + it * 64 + lane;
-        const bool valid = local < tile_n;
         const uint32_t d = (key[it] >> shift) & mask;
-        const uint64_t m = match_digit8(d, valid, bits);
+        const uint64_t m = match_digit8(d, bits);
         const uint32_t below = (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
         const uint32_t old = wh[d];
         __builtin_amdgcn_wave_barrier();
-        if(valid && below == 0)
+        if(below == 0)
             wh[d] = (uint16_t)(old + (uint32_t)__popcll(m));
         __builtin_amdgcn_wave_barrier();
         if(it & 1)
@@ -301,14 +303,10 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
 #pragma unroll
     for(int it = 0; it < kSort32Items; ++it)
     {
-        const int local = wave * (kSort32Items * 64) + it * 64 + lane;
-        if(local < tile_n)
-        {
-            const uint32_t d = (key[it] >> shift) & mask;
-            const uint32_t p = ((pos2[it >> 1] >> (16 * (it & 1))) & 0xffffu) + s_digit_start[d] + s_whist[wave][d];
-            s_keys[p] = key[it];
-            pos2[it >> 1] = (it & 1) ? ((pos2[it >> 1] & 0xffffu) | (p << 16)) : ((pos2[it >> 1] & 0xffff0000u) | p);
-        }
+        const uint32_t d = (key[it] >> shift) & mask;
+        const uint32_t p = ((pos2[it >> 1] >> (16 * (it & 1))) & 0xffffu) + s_digit_start[d] + s_whist[wave][d];
+        s_keys[p] = key[it];
+        pos2[it >> 1] = (it & 1) ? ((pos2[it >> 1] & 0xffffu) | (p << 16)) : ((pos2[it >> 1] & 0xffff0000u) | p);
     }
 
     // ---- the values: in flight while the chained scan runs ---------------------------------
@@ -396,9 +394,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
 #pragma unroll
     for(int it = 0; it < kSort32Items; ++it)
     {
-        const int local = wave * (kSort32Items * 64) + it * 64 + lane;
-        if(local < tile_n)
-            s_keys[(pos2[it >> 1] >> (16 * (it & 1))) & 0xffffu] = val[it];
+        s_keys[(pos2[it >> 1] >> (16 * (it & 1))) & 0xffffu] = val[it];
     }
     __syncthreads();
 #pragma unroll
