@@ -75,23 +75,27 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     const int start = ranges[tile];
     const int end = ranges[tile + 1];
 
+    // A pixel that has stopped (or lies outside the image) gets the row coordinate +infinity:
+    // its exponent is then -infinity (or NaN for a degenerate conic), its alpha fails the
+    // threshold test, and the loop needs no per-pixel flag.  `alive` counts the lane's live pixels.
     float pyf[kFwdPix], T[kFwdPix], cr[kFwdPix], cg[kFwdPix], cb[kFwdPix];
     int last[kFwdPix];
-    bool done[kFwdPix];
+    int alive = 0;
 #pragma unroll
     for(int p = 0; p < kFwdPix; ++p)
     {
         const int y = y0 + 4 * p;
-        pyf[p] = (float)y + 0.5f;
+        const bool inside = x < W && y < H;
+        pyf[p] = inside ? (float)y + 0.5f : __builtin_inff();
+        alive += inside ? 1 : 0;
         T[p] = 1.0f;
         cr[p] = cg[p] = cb[p] = 0.0f;
         last[p] = 0;
-        done[p] = !(x < W && y < H);
     }
 
     for(int b = start; b < end; b += kFwdBatch)
     {
-        if(__ballot(!(done[0] && done[1] && done[2] && done[3])) == 0)
+        if(__ballot(alive != 0) == 0)
             break;
         __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
         uint64_t todo[kFwdBatch / DSX_WAVE]; // entries of this round that can touch the tile
@@ -120,7 +124,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             uint64_t mask = todo[h];
             while(mask != 0)
             {
-                if(__ballot(!(done[0] && done[1] && done[2] && done[3])) == 0)
+                if(__ballot(alive != 0) == 0)
                     break;
                 const int i = h * DSX_WAVE + __builtin_ctzll(mask);
                 mask &= mask - 1;
@@ -128,25 +132,27 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                 const float4 B = s_b[i];
                 const float C = s_c[i];
                 const float dx = pxf - A.x;
-                const float bx = A.w * dx;           // conic b * dx
+                const float bx = A.w * dx;              // conic b * dx
                 const float ax = -0.5f * A.z * dx * dx; // -1/2 conic a * dx^2
 #pragma unroll
                 for(int p = 0; p < kFwdPix; ++p)
                 {
                     const float dy = pyf[p] - A.y;
                     const float power = ax - (0.5f * B.x * dy + bx) * dy;
-                    const float alpha = fminf(0.999f, B.y * fast_exp(power));
-                    const bool pass = !done[p] && power < 0.0f && alpha >= kAlphaThreshold;
+                    const float raw = B.y * fast_exp(power);
+                    const bool pass = power < 0.0f && raw >= kAlphaThreshold; // false for NaN
+                    const float alpha = fminf(0.999f, raw);
                     const float Tn = (1.0f - alpha) * T[p];
                     const bool stop = pass && Tn < 0.0001f;
                     const bool apply = pass && !stop;
-                    done[p] = done[p] || stop;
                     const float vis = apply ? alpha * T[p] : 0.0f;
                     cr[p] += vis * B.z;
                     cg[p] += vis * B.w;
                     cb[p] += vis * C;
                     T[p] = apply ? Tn : T[p];
                     last[p] = apply ? b + i : last[p];
+                    pyf[p] = stop ? __builtin_inff() : pyf[p];
+                    alive -= stop ? 1 : 0;
                 }
             }
         }
