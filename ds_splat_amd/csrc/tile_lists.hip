@@ -584,7 +584,8 @@ __global__ __launch_bounds__(kProjBlock) void ordered_block_sums_kernel(const ui
 // histograms of the tile partition (and the tile counts themselves).
 constexpr int kCoverThreads = 1024;
 constexpr int kCoverBlocks = 128;
-constexpr int kCoverLdsCells = 14 * 1024; // grids up to this many cells (56 KB) are held in LDS
+constexpr int kCoverLdsCells = 14 * 1024;      // grids up to this many cells (56 KB) are held in LDS as they are
+constexpr int kCoverLdsCellsLarge = 38 * 1024; // up to 152 KB of the CU's 160 KB, once the kernels are allowed it
 
 __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* __restrict__ rects, int64_t n, int ntx,
                                                                    int nty, int use_lds, int32_t* __restrict__ grid)
@@ -799,7 +800,23 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
         const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
         const int cells = (ntx + 1) * (nty + 1) + 1;
         int32_t* grid = reinterpret_cast<int32_t*>(base + o.cover);
-        const int use_lds = cells <= kCoverLdsCells ? 1 : 0;
+        // The corner grid is privatised in LDS whenever it fits (a 4K image has 32 776 cells =
+        // 128 KB: one workgroup per CU); beyond 64 KB a kernel needs its limit raised first.
+        // Global atomics are the fallback: correct for any grid, but 24 M same-line atomics
+        // at 6 M Gaussians cost 0.6 ms and stall the sort passes that run beside them.
+        int use_lds = cells <= kCoverLdsCells ? 1 : 0;
+        if(!use_lds && cells <= kCoverLdsCellsLarge)
+        {
+            const int bytes = cells * 4;
+            use_lds = hipFuncSetAttribute(reinterpret_cast<const void*>(tile_cover_kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess &&
+                              hipFuncSetAttribute(reinterpret_cast<const void*>(tile_counts_kernel),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess
+                          ? 1
+                          : 0;
+            if(!use_lds)
+                (void)hipGetLastError();
+        }
         const int64_t want = (n + kCoverThreads - 1) / kCoverThreads;
         {
             DSX_TIMED("tile_cover_kernel", cs);
