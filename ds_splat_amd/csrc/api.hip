@@ -474,7 +474,12 @@ extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, c
     int rc = dsx_tile_lists(cam, n, k, order, sorted_ids, ranges, workspace, workspace_bytes, stream);
     if(rc)
         return rc;
-    return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream));
+    const uint32_t *depth_flag = nullptr, *partition_flag = nullptr;
+    rc = dsx_sort_flags(n, k, cam->image_width, cam->image_height, order, workspace, &depth_flag, &partition_flag);
+    if(rc)
+        return rc;
+    return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream), depth_flag,
+                            partition_flag);
 }
 
 extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,

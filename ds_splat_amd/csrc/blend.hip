@@ -57,7 +57,9 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                                                              const int32_t* __restrict__ ids,
                                                              const float4* __restrict__ splats,
                                                              float* __restrict__ image, float* __restrict__ final_T,
-                                                             int32_t* __restrict__ final_idx, int W, int H, int ntx)
+                                                             int32_t* __restrict__ final_idx, int W, int H, int ntx,
+                                                             const uint32_t* __restrict__ sort_flag_a,
+                                                             const uint32_t* __restrict__ sort_flag_b)
 {
     __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic a, conic b
     __shared__ float4 s_b[kFwdBatch]; // conic c, opacity, red, green
@@ -158,6 +160,14 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
         }
     }
 
+    // A sort pass that gave up waiting on its predecessor (bounded wait, never seen to happen)
+    // leaves its flag set and the tile lists wrong: make that loud instead of plausible.
+    if((sort_flag_a && *sort_flag_a) || (sort_flag_b && *sort_flag_b))
+    {
+#pragma unroll
+        for(int p = 0; p < kFwdPix; ++p)
+            cr[p] = cg[p] = cb[p] = __builtin_nanf("");
+    }
 #pragma unroll
     for(int p = 0; p < kFwdPix; ++p)
     {
@@ -175,7 +185,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
 }
 
 int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids, const float* splats,
-                     float* image, float* final_T, int32_t* final_idx, hipStream_t stream)
+                     float* image, float* final_T, int32_t* final_idx, hipStream_t stream,
+                     const uint32_t* sort_flag_a, const uint32_t* sort_flag_b)
 {
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
     if(ntx * nty == 0)
@@ -184,7 +195,7 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
         DSX_TIMED("blend_fwd_kernel", stream);
         hipLaunchKernelGGL(blend_fwd_kernel, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
                            reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                           cam.image_height, ntx);
+                           cam.image_height, ntx, sort_flag_a, sort_flag_b);
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;

@@ -225,9 +225,11 @@ int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values
                       int32_t** values_out);
 int launch_tile_ranges(int64_t k, const int64_t* sorted_keys, int num_tiles, int32_t* ranges,
                        hipStream_t stream);
+// sort_flag_*: error words of the sorts that built the lists (null: none); the image becomes NaN if one is set
 int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids,
                      const float* splats, float* image, float* final_T, int32_t* final_idx,
-                     hipStream_t stream);
+                     hipStream_t stream,
+                     const uint32_t* sort_flag_a = nullptr, const uint32_t* sort_flag_b = nullptr);
 int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges,
                      const int32_t* sorted_ids, const float* splats, const float* final_T,
                      const int32_t* final_idx, const float* v_image, float* grads,

@@ -220,8 +220,22 @@ class ForwardState:
     __slots__ = ("splats", "radii", "cov3d", "sorted_ids", "ranges", "final_T", "final_idx", "num_keys")
 
 
-def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, colors_precomp=None):
-    """Whole forward: returns (image[H,W,3], ForwardState)."""
+def sort_flag_indices(cam, n, k, order, workspace):
+    """Positions (int32 index into `order`, int32 index into `workspace`; None where absent) of
+    the give-up flags of the two chained scans."""
+    lib = N.load()
+    p_a, p_b = C.c_void_p(), C.c_void_p()
+    N.check(lib.dsx_sort_flags(n, k, cam.width, cam.height, _ptr(order), _ptr(workspace) if k > 0 else None,
+                               C.byref(p_a), C.byref(p_b)))
+    ia = (p_a.value - order.data_ptr()) // 4 if p_a.value else None
+    ib = (p_b.value - workspace.data_ptr()) // 4 if p_b.value else None
+    return ia, ib
+
+
+def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, colors_precomp=None,
+            after_project=None):
+    """Whole forward: returns (image[H,W,3], ForwardState).  after_project(order, n, k), if given,
+    runs between the two halves (diagnostics)."""
     lib = N.load()
     n = means3d.shape[0]
     dev = means3d.device
@@ -240,6 +254,8 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
                                     _ptr(k_host), stream))
     k = int(k_host.item())
     st.num_keys = k
+    if after_project is not None:
+        after_project(order, n, k)
     st.sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
     st.ranges = torch.empty((cam.num_tiles + 1,), dtype=torch.int32, device=dev)
     image = torch.empty((cam.height, cam.width, 3), dtype=torch.float32, device=dev)

@@ -208,7 +208,9 @@ int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
                         int64_t* num_keys /* host */, void* stream);
 
 /* Second half: tile lists (dsx_tile_lists) and blend.  sorted_ids[k] and ranges[T+1] are
- * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H). */
+ * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H).  If one of the two
+ * sorts gave up a bounded wait (see dsx_sort_flags) the image is written as NaN: a failure
+ * shows without a read-back of the flags. */
 int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
                        const void* order, int32_t* sorted_ids, int32_t* ranges, float* image,
                        float* final_T, int32_t* final_idx, void* workspace,

@@ -322,3 +322,28 @@ def test_full_size_forward_cfg3_4k():
     assert torch.equal(st.sorted_ids, st2.sorted_ids) and torch.equal(image, image2)
     assert (st.ranges[1:] >= st.ranges[:-1]).all() and int(st.ranges[-1]) == st.num_keys
     assert torch.isfinite(image).all()
+
+
+def test_a_sort_that_gave_up_poisons_the_image():
+    """The chained scans wait for their predecessors a bounded number of times and set a flag if
+    they give up (never observed).  Force the depth sort's flag from the host between the two
+    halves of the forward: the image must come back NaN, not plausible."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg1", n=5000, width=160, height=96, sh_degree=1)
+    cam = stages.camera_from_scene(sc, DEV)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    args = (cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
+    image, st = stages.forward(*args)
+    assert torch.isfinite(image).all() and st.num_keys > 0
+
+    def poke(order, n, k):
+        ia, _ = stages.sort_flag_indices(cam, n, 0, order, order)
+        assert ia is not None
+        torch.cuda.synchronize()
+        assert int(order.view(torch.int32)[ia].item()) == 0
+        order.view(torch.int32)[ia] = 1
+
+    image, st = stages.forward(*args, after_project=poke)
+    torch.cuda.synchronize()
+    assert torch.isnan(image).all()
+
