@@ -176,11 +176,12 @@ extern "C" size_t dsx_sort_u32_workspace_bytes(int64_t count, int32_t key_bits)
     return sort_u32_layout(count < 0 ? 0 : count, key_bits).bytes;
 }
 
-extern "C" int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
+// clear_for_depth_order: the kernel also zeroes what launch_depth_order needs zeroed in `order`
+static int project_fwd_checked(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
                                const float* quats, const float* opacities, const float* shs,
                                const float* cov3d_precomp, const float* colors_precomp, float* splats,
                                int32_t* radii, float* cov3d, uint32_t* block_sums, void* order, size_t order_bytes,
-                               void* stream)
+                               void* stream, bool clear_for_depth_order)
 {
     if(int rc = check_camera(cam))
         return rc;
@@ -204,8 +205,22 @@ extern "C" int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* me
         return DSX_ERR_BAD_ARG;
     if(!colors_precomp && !shs)
         return DSX_ERR_BAD_ARG;
+    uint32_t* clear = nullptr;
+    int64_t clear_words = 0;
+    if(order && clear_for_depth_order)
+        depth_order_clear_region(*cam, n, order, &clear, &clear_words);
     return launch_project_fwd(*cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp, splats,
-                              radii, cov3d, block_sums, depth_keys, rects, as_stream(stream));
+                              radii, cov3d, block_sums, depth_keys, rects, as_stream(stream), clear, clear_words);
+}
+
+extern "C" int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
+                               const float* quats, const float* opacities, const float* shs,
+                               const float* cov3d_precomp, const float* colors_precomp, float* splats,
+                               int32_t* radii, float* cov3d, uint32_t* block_sums, void* order, size_t order_bytes,
+                               void* stream)
+{
+    return project_fwd_checked(cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp, splats,
+                               radii, cov3d, block_sums, order, order_bytes, stream, false);
 }
 
 extern "C" int dsx_scan_u32(int64_t count, uint32_t* data, uint32_t* total, void* stream)
@@ -437,8 +452,8 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
         return DSX_ERR_BAD_ARG;
     *num_keys = 0;
     hipStream_t s = as_stream(stream);
-    int rc = dsx_project_fwd(cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp, splats,
-                             radii, cov3d, block_sums, order, order_bytes, stream);
+    int rc = project_fwd_checked(cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp,
+                                 splats, radii, cov3d, block_sums, order, order_bytes, stream, true);
     if(rc || n == 0)
         return rc;
     rc = launch_scan_u32(dsx_num_blocks(n), block_sums, k_scratch, s);
@@ -453,7 +468,7 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
     bool ok = hipMemcpyAsync(num_keys, k_scratch, sizeof(uint32_t), hipMemcpyDeviceToHost, s) == hipSuccess &&
               hipEventRecord(copied, s) == hipSuccess;
     if(ok)
-        rc = launch_depth_order(*cam, n, order, s);
+        rc = launch_depth_order(*cam, n, order, s, true);
     ok = ok && hipEventSynchronize(copied) == hipSuccess;
     (void)hipEventDestroy(copied);
     if(!ok)

@@ -206,14 +206,18 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
                   uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src = nullptr,
                   uint2* gather_dst = nullptr, bool already_cleared = false);
-int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream);
+// already_cleared: the words of depth_order_clear_region are zero already (the projection did it)
+int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream,
+                       bool already_cleared = false);
+// the part of an `order` buffer that must be zero when launch_depth_order starts
+void depth_order_clear_region(const dsx_camera& cam, int64_t n, void* order, uint32_t** words, int64_t* count);
 int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
                       int32_t* ranges, void* workspace, hipStream_t stream);
 int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, const float* scales,
                        const float* quats, const float* opacities, const float* shs,
                        const float* cov3d_precomp, const float* colors_precomp, float* splats,
                        int32_t* radii, float* cov3d, uint32_t* block_sums, uint32_t* depth_keys,
-                       uint2* rects, hipStream_t stream);
+                       uint2* rects, hipStream_t stream, uint32_t* clear = nullptr, int64_t clear_words = 0);
 int launch_scan_u32(int64_t count, uint32_t* data, uint32_t* total, hipStream_t stream);
 int launch_emit_keys(const dsx_camera& cam, int64_t n, int64_t k, const float* splats,
                      const uint32_t* block_offsets, int64_t* keys, int32_t* values,

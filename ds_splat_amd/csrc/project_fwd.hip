@@ -44,6 +44,8 @@ struct ProjectParams
     uint32_t* block_sums;
     uint32_t* depth_keys; // optional: depth bits per Gaussian, the key of the depth order
     uint2* rects;         // optional: packed tile rectangle per Gaussian (zero when it emits nothing)
+    uint32_t* clear;      // optional: words that the kernel zeroes on the side (counters of the sort that follows)
+    int64_t clear_words;
     float focal_x, focal_y, tanfovx, tanfovy, c_x, c_y, scale_modifier;
     int sh_degree, sh_stride; // active degree; floats per shs row
     int ntx, nty;
@@ -215,6 +217,11 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
     const int wave = tid >> 6;
     const int64_t i = (int64_t)blockIdx.x * kProjBlock + tid;
     const bool live = i < p.n;
+
+    // housekeeping for the sort that follows: its counters are zeroed here, a word per thread,
+    // instead of by a launch of their own
+    for(int64_t j = i; j < p.clear_words; j += (int64_t)gridDim.x * kProjBlock)
+        p.clear[j] = 0u;
 
     // frustum test on the centre: strict NDC box, z_ndc > 0.1 (cpp/rasterizer_kernels.cu:7-24).
     // It comes first because a Gaussian that fails it is culled whatever its shape is, nothing
@@ -420,11 +427,14 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
 int launch_project_fwd(const dsx_camera& cam, int64_t n, const float* means3d, const float* scales,
                        const float* quats, const float* opacities, const float* shs,
                        const float* cov3d_precomp, const float* colors_precomp, float* splats, int32_t* radii,
-                       float* cov3d, uint32_t* block_sums, uint32_t* depth_keys, uint2* rects, hipStream_t stream)
+                       float* cov3d, uint32_t* block_sums, uint32_t* depth_keys, uint2* rects, hipStream_t stream,
+                       uint32_t* clear, int64_t clear_words)
 {
     if(n == 0)
         return DSX_OK;
     ProjectParams p;
+    p.clear = clear;
+    p.clear_words = clear ? clear_words : 0;
     p.n = n;
     p.means3d = means3d;
     p.scales = scales;

@@ -763,7 +763,16 @@ __global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(int32_t* gri
 }
 
 // order: the buffer of order_layout(n) whose depth_keys and rects the projection has written
-int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream)
+void depth_order_clear_region(const dsx_camera& cam, int64_t n, void* order, uint32_t** words, int64_t* count)
+{
+    // the sort's histograms, counters and look-back statuses and, right behind them, the corner grid
+    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height);
+    const Sort32Workspace w = sort32_workspace(n, 32, kDepthSortTile);
+    *words = reinterpret_cast<uint32_t*>(static_cast<char*>(order) + o.sort + w.hist);
+    *count = (int64_t)((w.bytes + (o.ranges - o.cover)) / 4);
+}
+
+int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream, bool already_cleared)
 {
     if(n <= 0)
         return DSX_OK;
@@ -775,7 +784,14 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
     uint32_t* ids_b = reinterpret_cast<uint32_t*>(base + o.ids_b);
     uint32_t* block_sums = reinterpret_cast<uint32_t*>(base + o.block_sums);
     // one fill zeroes the sort's counters and, right behind them, the corner grid
-    int rc = sort32_clear(n, 32, kDepthSortTile, base + o.sort, stream, o.ranges - o.cover);
+    int rc = DSX_OK;
+    if(!already_cleared)
+    {
+        uint32_t* words;
+        int64_t count;
+        depth_order_clear_region(cam, n, order, &words, &count);
+        rc = launch_fill_u32(words, count, 0u, stream);
+    }
     if(rc)
         return rc;
 
@@ -880,7 +896,8 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
                                                                   int64_t n, int64_t k, int ntx,
                                                                   SlotT* __restrict__ slots, int32_t* __restrict__ ids,
                                                                   const int32_t* __restrict__ ranges_in,
-                                                                  int32_t* __restrict__ ranges_out, int range_count)
+                                                                  int32_t* __restrict__ ranges_out, int range_count,
+                                                                  uint32_t* __restrict__ clear, int64_t clear_words)
 {
     __shared__ uint32_t s_off[kProjBlock + 1];
     __shared__ uint32_t s_origin[kProjBlock]; // slot of the rectangle's first tile (0 for negative depths)
@@ -900,6 +917,9 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     // the tile ranges were derived from the rectangles before any pair existed: hand them out
     for(int j = blockIdx.x * kProjBlock + tid; j < range_count; j += gridDim.x * kProjBlock)
         ranges_out[j] = ranges_in[j];
+    // housekeeping for the partition that follows: its counters and look-back statuses start at zero
+    for(int64_t j = (int64_t)blockIdx.x * kProjBlock + tid; j < clear_words; j += (int64_t)gridDim.x * kProjBlock)
+        clear[j] = 0u;
 
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     for(int64_t blk = blockIdx.x; blk < blocks; blk += gridDim.x)
@@ -1029,9 +1049,8 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
     const bool even = (w.passes % 2) == 0;
     uint32_t* vals_a = even ? ids_final : ids_other;
     uint32_t* vals_b = even ? ids_other : ids_final;
-    int rc = sort32_clear(k, bits, kListSortTile, base + w.sort, stream);
-    if(rc)
-        return rc;
+    int rc = DSX_OK;
+    const Sort32Workspace sw = sort32_workspace(k, bits, kListSortTile);
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     {
         DSX_TIMED("emit_ordered_kernel", stream);
@@ -1040,7 +1059,8 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
                            reinterpret_cast<const uint2*>(obase + o.rects_sorted),
                            reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k, tiles_x(cam.image_width),
                            slots_a, reinterpret_cast<int32_t*>(vals_a),
-                           reinterpret_cast<const int32_t*>(obase + o.ranges), ranges, num_tiles + 1);
+                           reinterpret_cast<const int32_t*>(obase + o.ranges), ranges, num_tiles + 1,
+                           reinterpret_cast<uint32_t*>(base + w.sort + sw.hist), (int64_t)(sw.bytes / 4));
     }
     DSX_LAUNCH_CHECK();
     SlotT* ko;
