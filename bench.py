@@ -93,7 +93,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--verbose", action="store_true", help="per-kernel table on stderr")
     ap.add_argument("--copy-probe", action="store_true",
-                    help="also run one 1 GiB device copy (a kernel of known traffic that scales HBM byte counters)")
+                    help="also run one 1 GiB device copy (a kernel of known traffic that scales HBM byte counters) and "
+                         "the library's streaming probe (read / write / copy rates that plain kernels reach here)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding "
@@ -137,11 +138,33 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    stream_ceiling = None
     if args.copy_probe:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
+        # what plain streaming kernels of this library's access shape reach on this device (1 GiB each)
+        lib = _native.load()
+        stream = torch.cuda.current_stream().cuda_stream
+        nbytes = src.numel() * 4
+        for mode in (0, 1, 2):
+            for _ in range(2):
+                _native.check(lib.dsx_stream_probe(src.data_ptr(), dst.data_ptr(), nbytes, mode, stream))
+        torch.cuda.synchronize()
+        _native.trace_enable(True)
+        _native.trace_read()
+        reps = 5
+        for mode in (0, 1, 2):
+            for _ in range(reps):
+                _native.check(lib.dsx_stream_probe(src.data_ptr(), dst.data_ptr(), nbytes, mode, stream))
+        torch.cuda.synchronize()
+        times = [ms for name, ms in _native.trace_read() if name == "stream_probe_kernel"]
+        _native.trace_enable(False)
+        per_mode = [min(times[m * reps:(m + 1) * reps]) for m in range(3)]
+        stream_ceiling = {"unit": "GB/s", "bytes": nbytes,
+                          "read": round(nbytes / per_mode[0] / 1e6, 1), "write": round(nbytes / per_mode[1] / 1e6, 1),
+                          "copy": round(2 * nbytes / per_mode[2] / 1e6, 1)}
         del src, dst
 
     # timed region: K steps, nothing but the public API between the two synchronisations
@@ -261,6 +284,8 @@ def main():
         "roofline_hbm": roofline_hbm,
         "cpu_baseline": cpu_baseline,
     }
+    if stream_ceiling is not None:
+        out["stream_ceiling"] = stream_ceiling
     print(json.dumps(out))
 
 

@@ -251,6 +251,12 @@ typedef struct dsx_trace_entry
 int dsx_trace_enable(int on);
 int dsx_trace_read(dsx_trace_entry* out /* host */, int max_entries);
 
+/* Calibration of the HBM roofline: one launch that streams `bytes` (a multiple of 16) with one
+ * 16-byte element per thread, the access shape of the per-Gaussian kernels.  mode 0 reads src,
+ * 1 writes dst, 2 copies src to dst.  Traced as "stream_probe_kernel".  No counterpart in the
+ * reference. */
+int dsx_stream_probe(const void* src, void* dst, size_t bytes, int mode, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
