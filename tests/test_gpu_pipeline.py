@@ -309,6 +309,35 @@ def test_full_size_properties_cfg2():
         assert (o[key][radii <= 0] == 0).all()
 
 
+def test_full_size_cfg2_against_the_openmp_oracle():
+    """The headline shape itself (3M Gaussians, 1920x1080, SH3) against the oracle's OpenMP build
+    (same source as the serial oracle, loops over Gaussians and tiles in parallel): integers bit
+    for bit, image rtol 1e-4 / atol 1e-5 and gradients rtol 1e-3 away from threshold decisions."""
+    from oracle.binding import Oracle
+    from ds_splat_amd import stages
+    omp = Oracle(omp=True)
+    sc = make_scene("cfg2")
+    n = sc["n"]
+    image, radii, leaves = api_run(sc)
+    img_o, radii_o, S, B = oracle_run(omp, sc)
+    assert (radii.cpu().numpy() == radii_o).all()
+    ok = S["margin"] > 1e-4
+    assert ok.mean() > 0.97
+    np.testing.assert_allclose(image.detach().cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
+    gok = B["g_margin"] > 1e-5
+    assert gok.mean() > 0.9
+    check_grads(leaves, B, gok)
+    del image, leaves
+    cam = stages.camera_from_scene(sc, DEV)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    _, st = stages.forward(cam, t["means_3d"], t["scales"], t["rotations"], t["opacities"], t["shs"])
+    torch.cuda.synchronize()
+    assert st.num_keys == S["num_keys"]
+    assert (st.ranges.cpu().numpy() == S["ranges"]).all()
+    assert (st.sorted_ids.cpu().numpy() == S["sorted_ids"]).all()
+    assert (st.final_idx.cpu().numpy()[ok] == S["final_idx"][ok]).all()
+
+
 def test_full_size_forward_cfg3_4k():
     """6M Gaussians at 3840x2160 (forward only): runs, sorted, deterministic."""
     from ds_splat_amd import stages
