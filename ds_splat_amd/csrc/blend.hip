@@ -385,10 +385,11 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             if(__ballot(any) == 0)
                 continue;
             const float blue = s_c[t];
-            const float hdx2 = 0.5f * dx * dx;
-            const float adx = A.z * dx;
             float g[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; // v_x, v_y, v_conic a b c, v_opacity, v_red, v_green
             float g_blue = 0.f;
+            // dx is the same for the lane's four pixels, so the five geometric sums are built from
+            // three moments of v_sigma over dy: S0 = sum v_sigma, S1 = sum v_sigma dy, S2 = sum v_sigma dy^2
+            float S0 = 0.f, S1 = 0.f, S2 = 0.f;
 #pragma unroll
             for(int p = 0; p < kBwdPix; ++p)
             {
@@ -404,14 +405,18 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
                     const float v_alpha = rv * T[p] + bterm[p] * ra;
                     bterm[p] -= rv * fac;
                     const float v_sigma = -B.y * vis[p] * v_alpha;
-                    g[0] += v_sigma * (adx + A.w * dy[p]);
-                    g[1] += v_sigma * (bdx + B.x * dy[p]);
-                    g[2] += v_sigma * hdx2;
-                    g[3] += v_sigma * dx * dy[p];
-                    g[4] += 0.5f * v_sigma * dy[p] * dy[p];
+                    const float vsdy = v_sigma * dy[p];
+                    S0 += v_sigma;
+                    S1 += vsdy;
+                    S2 += vsdy * dy[p];
                     g[5] += vis[p] * v_alpha;
                 }
             }
+            g[0] = A.z * dx * S0 + A.w * S1; // v_sigma (a dx + b dy)
+            g[1] = bdx * S0 + B.x * S1;      // v_sigma (b dx + c dy)
+            g[2] = 0.5f * dx * dx * S0;
+            g[3] = dx * S1;
+            g[4] = 0.5f * S2;
             float s0, s1;
             wave_sum8_to_last_quad(g, lane, s0, s1);
             g_blue = wave_sum_to_lane63(g_blue);
