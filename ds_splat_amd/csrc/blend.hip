@@ -234,14 +234,14 @@ __device__ __forceinline__ float dpp_move(float v)
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
 }
 
-// Sums eight per-lane values over the wavefront in 30 VALU instructions instead of 48: the
-// first two steps are a reduce-scatter inside each quad (a lane keeps half of the values and
-// hands the other half to its partner), the rest reduces the two remaining values across
-// quads, rows and halves (every lane ends up with totals).  The lanes of the last quad are
-// the ones that use them: lane 60 + q holds out0 = total of v[4*(q&1) + 2*(q>>1)] and out1 = total of the next index.
-__device__ __forceinline__ void wave_sum8_to_last_quad(const float (&v)[8], int lane, float& out0, float& out1)
+// Sums eight per-lane values over the wavefront as a reduce-scatter: in each of the first
+// three steps a lane keeps half of its values and hands the other half to a partner (inside the
+// quad twice, then to the quad four lanes away), so one value per lane is left for the steps
+// across the row, the rows and the halves.  Lanes 56..63 end up with the eight totals: lane l
+// holds the total of v[4*(l&1) + 2*((l>>1)&1) + ((l>>2)&1)].
+__device__ __forceinline__ float wave_sum8_scatter(const float (&v)[8], int lane)
 {
-    const bool b0 = lane & 1, b1 = lane & 2;
+    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
     float r[4];
 #pragma unroll
     for(int i = 0; i < 4; ++i)
@@ -258,20 +258,20 @@ __device__ __forceinline__ void wave_sum8_to_last_quad(const float (&v)[8], int 
         const float send = b1 ? r[i] : r[2 + i];
         q[i] = keep + dpp_move<0x4E>(send); // quad_perm [2,3,0,1]
     }
-#pragma unroll
-    for(int i = 0; i < 2; ++i)
-    {
-        q[i] += dpp_move<0x124>(q[i]); // row_ror:4  -> two quads
-        q[i] += dpp_move<0x128>(q[i]); // row_ror:8  -> the whole row of 16
-        // across rows the lanes must keep their position inside the quad, so the row
-        // broadcasts of the single-value reduction cannot be used: swap rows, then halves
-        const dsx_u32x2 r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(q[i]), __float_as_uint(q[i]), false, false);
-        q[i] = __uint_as_float(r16.x) + __uint_as_float(r16.y);
-        const dsx_u32x2 r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(q[i]), __float_as_uint(q[i]), false, false);
-        q[i] = __uint_as_float(r32.x) + __uint_as_float(r32.y);
-    }
-    out0 = q[0];
-    out1 = q[1];
+    const float keep = b2 ? q[1] : q[0];
+    const float send = b2 ? q[0] : q[1];
+    // partner = lane ^ 4: banks 0 and 2 of a row read four lanes up, banks 1 and 3 four lanes down
+    int got = __builtin_amdgcn_update_dpp(0, __float_as_int(send), 0x104, 0xf, 0x5, false); // row_shl:4
+    got = __builtin_amdgcn_update_dpp(got, __float_as_int(send), 0x114, 0xf, 0xa, false);   // row_shr:4
+    float o = keep + __int_as_float(got);
+    o += dpp_move<0x128>(o); // row_ror:8 -> the whole row of 16
+    // across rows the lanes must keep their position inside the row, so the row broadcasts of
+    // the single-value reduction cannot be used: swap rows, then halves
+    const dsx_u32x2 r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(o), __float_as_uint(o), false, false);
+    o = __uint_as_float(r16.x) + __uint_as_float(r16.y);
+    const dsx_u32x2 r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(o), __float_as_uint(o), false, false);
+    o = __uint_as_float(r32.x) + __uint_as_float(r32.y);
+    return o;
 }
 
 constexpr int kBwdBatch = 128; // sorted entries staged in LDS per round (two per lane)
@@ -417,18 +417,15 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             g[2] = 0.5f * dx * dx * S0;
             g[3] = dx * S1;
             g[4] = 0.5f * S2;
-            float s0, s1;
-            wave_sum8_to_last_quad(g, lane, s0, s1);
+            const float total = wave_sum8_scatter(g, lane);
             g_blue = wave_sum_to_lane63(g_blue);
-            if(lane >= 60)
+            if(lane >= 56)
             {
-                // lane 60 + q holds the totals of g[4*(q&1) + 2*(q>>1)] and of the next index
-                const int q = lane - 60;
-                float* dst = grads + (int64_t)s_id[t] * DSX_GRAD_FLOATS + 4 * (q & 1) + 2 * (q >> 1);
-                unsafeAtomicAdd(dst, s0);
-                unsafeAtomicAdd(dst + 1, s1);
+                // lane l holds the total of g[4*(l&1) + 2*((l>>1)&1) + ((l>>2)&1)]
+                float* rec = grads + (int64_t)s_id[t] * DSX_GRAD_FLOATS;
+                unsafeAtomicAdd(rec + 4 * (lane & 1) + 2 * ((lane >> 1) & 1) + ((lane >> 2) & 1), total);
                 if(lane == 63)
-                    unsafeAtomicAdd(grads + (int64_t)s_id[t] * DSX_GRAD_FLOATS + 8, g_blue);
+                    unsafeAtomicAdd(rec + 8, g_blue);
             }
         }
     }
