@@ -89,11 +89,16 @@ __global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* data, 
 {
     __shared__ uint32_t wave_tot[kScanThreads / DSX_WAVE];
     __shared__ uint32_t carry_s;
+    __shared__ unsigned long long total64; // the true sum: the 32-bit prefixes wrap silently, the total must not
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     if(tid == 0)
+    {
         carry_s = 0;
+        total64 = 0ull;
+    }
+    unsigned long long mine64 = 0ull;
     __syncthreads();
     for(int64_t base = 0; base < count; base += kScanThreads * kScanItems)
     {
@@ -105,6 +110,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* data, 
         {
             v[j] = (i0 + j < count) ? data[i0 + j] : 0u;
             sum += v[j];
+            mine64 += v[j];
         }
         const uint32_t incl = wave_incl_scan_u32(sum, lane);
         if(lane == 63)
@@ -126,8 +132,11 @@ __global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* data, 
             carry_s = run;
         __syncthreads();
     }
+    if(mine64)
+        atomicAdd(&total64, mine64);
+    __syncthreads();
     if(tid == 0)
-        *total = carry_s;
+        *total = total64 > 0xffffffffull ? 0xffffffffu : (uint32_t)total64; // saturates: callers reject counts >= 2^30
 }
 
 int launch_scan_u32(int64_t count, uint32_t* data, uint32_t* total, hipStream_t stream)

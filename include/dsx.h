@@ -105,7 +105,9 @@ int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, cons
 
 /* Exclusive prefix of `count` uint32 values in place, total written to *total (device).
  * Replaces the in-block Hillis-Steele scan of cpp/rasterizer_kernels.cu:131-142 together
- * with thrust::exclusive_scan, cpp/rasterizer_torch.cu:95. */
+ * with thrust::exclusive_scan, cpp/rasterizer_torch.cu:95.  The prefixes are modulo 2^32; the
+ * total saturates at 0xffffffff, so a key count that does not fit is seen as too large
+ * (DSX_ERR_TOO_LARGE from dsx_forward_project) and never as a small wrapped number. */
 int dsx_scan_u32(int64_t count, uint32_t* data, uint32_t* total, void* stream);
 
 /* Stage 2a — replaces calculate_keys_and_indices_kernel, cpp/rasterizer_kernels.cu:252-306.

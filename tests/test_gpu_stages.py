@@ -124,6 +124,22 @@ def test_scan_u32(count):
     assert int(total.item()) == int(want[-1])
 
 
+def test_scan_u32_total_saturates_instead_of_wrapping():
+    """The prefixes are 32-bit and may wrap, the total may not: a key count beyond 32 bits must
+    reach the host as a number that the size check rejects, not as a small wrapped one."""
+    st_ = _stages()
+    a = np.full(5000, 2_000_000, dtype=np.int64)             # sum 1e10 > 2^32
+    d = dev(a.astype(np.uint32).view(np.int32))
+    total = st_.scan_u32(d)
+    torch.cuda.synchronize()
+    assert int(total.item()) & 0xFFFFFFFF == 0xFFFFFFFF
+    a2 = np.full(1000, 4_000_000, dtype=np.int64)            # sum 4e9 < 2^32: exact
+    d2 = dev(a2.astype(np.uint32).view(np.int32))
+    total2 = st_.scan_u32(d2)
+    torch.cuda.synchronize()
+    assert int(total2.item()) & 0xFFFFFFFF == 4_000_000_000
+
+
 # ------------------------------------------------------------------------------- stage 2a
 @pytest.mark.parametrize("n,W,H,scale_mul,flip", [(20000, 256, 256, 2.0, 0), (3000, 200, 120, 12.0, 0),
                                                   (500, 64, 48, 3.0, 120), (1, 32, 32, 1.0, 0)])
