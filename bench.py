@@ -149,25 +149,26 @@ def main():
         stream = torch.cuda.current_stream().cuda_stream
         nbytes = src.numel() * 4
         mixed_bytes = 28 * 16 * 3_000_000   # 10 + 18 arrays of 3 M 16-byte elements: the backward's volume
-        sizes = (nbytes, nbytes, nbytes, mixed_bytes)
-        for mode in (0, 1, 2, 3):
+        sizes = (nbytes, nbytes, nbytes, mixed_bytes, mixed_bytes // 2)
+        for mode in (0, 1, 2, 3, 4):
             for _ in range(2):
                 _native.check(lib.dsx_stream_probe(src.data_ptr(), dst.data_ptr(), sizes[mode], mode, stream))
         torch.cuda.synchronize()
         _native.trace_enable(True)
         _native.trace_read()
         reps = 5
-        for mode in (0, 1, 2, 3):
+        for mode in (0, 1, 2, 3, 4):
             for _ in range(reps):
                 _native.check(lib.dsx_stream_probe(src.data_ptr(), dst.data_ptr(), sizes[mode], mode, stream))
         torch.cuda.synchronize()
         times = [ms for name, ms in _native.trace_read() if name == "stream_probe_kernel"]
         _native.trace_enable(False)
-        per_mode = [min(times[m * reps:(m + 1) * reps]) for m in range(4)]
+        per_mode = [min(times[m * reps:(m + 1) * reps]) for m in range(5)]
         stream_ceiling = {"unit": "GB/s", "bytes": nbytes,
                           "read": round(nbytes / per_mode[0] / 1e6, 1), "write": round(nbytes / per_mode[1] / 1e6, 1),
                           "copy": round(2 * nbytes / per_mode[2] / 1e6, 1),
-                          "mixed_10_reads_18_writes": round(mixed_bytes / per_mode[3] / 1e6, 1)}
+                          "mixed_10_reads_18_writes": round(mixed_bytes / per_mode[3] / 1e6, 1),
+                          "mixed_5_reads_9_writes": round(mixed_bytes // 2 / per_mode[4] / 1e6, 1)}
         del src, dst
 
     # timed region: K steps, nothing but the public API between the two synchronisations

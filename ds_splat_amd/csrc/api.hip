@@ -620,7 +620,7 @@ __global__ __launch_bounds__(256) void stream_probe_mixed_kernel(const probe_f4*
 
 extern "C" int dsx_stream_probe(const void* src, void* dst, size_t bytes, int mode, void* stream)
 {
-    if(mode < 0 || mode > 3 || (bytes & 15) != 0 || (mode != 1 && !src) || (mode != 0 && !dst))
+    if(mode < 0 || mode > 4 || (bytes & 15) != 0 || (mode != 1 && !src) || (mode != 0 && !dst))
         return DSX_ERR_BAD_ARG;
     if(mode == 0 && !dst)
         dst = const_cast<void*>(src); // the sink is never written
@@ -630,15 +630,21 @@ extern "C" int dsx_stream_probe(const void* src, void* dst, size_t bytes, int mo
     if(count >= (1ll << 39))
         return DSX_ERR_TOO_LARGE;
     hipStream_t s = as_stream(stream);
-    if(mode == 3)
+    if(mode >= 3)
     {
-        // the per-Gaussian backward's mix: 10 arrays read, 18 written; `bytes` is all of it
-        count /= 28;
+        // write-heavy mixes like the per-Gaussian backward's: 10 arrays read and 18 written (its
+        // volume per element), or 5 and 9 (closer to its number of arrays); `bytes` is all of it
+        count /= mode == 3 ? 28 : 14;
         if(count == 0)
             return DSX_OK;
+        const dim3 grid((unsigned)((count + 255) / 256));
         DSX_TIMED("stream_probe_kernel", s);
-        hipLaunchKernelGGL((dsx::stream_probe_mixed_kernel<10, 18>), dim3((unsigned)((count + 255) / 256)), dim3(256), 0,
-                           s, static_cast<const dsx::probe_f4*>(src), static_cast<dsx::probe_f4*>(dst), count);
+        if(mode == 3)
+            hipLaunchKernelGGL((dsx::stream_probe_mixed_kernel<10, 18>), grid, dim3(256), 0, s,
+                               static_cast<const dsx::probe_f4*>(src), static_cast<dsx::probe_f4*>(dst), count);
+        else
+            hipLaunchKernelGGL((dsx::stream_probe_mixed_kernel<5, 9>), grid, dim3(256), 0, s,
+                               static_cast<const dsx::probe_f4*>(src), static_cast<dsx::probe_f4*>(dst), count);
         DSX_LAUNCH_CHECK();
         return DSX_OK;
     }

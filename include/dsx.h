@@ -255,10 +255,10 @@ int dsx_trace_read(dsx_trace_entry* out /* host */, int max_entries);
 
 /* Calibration of the HBM roofline: one launch that streams `bytes` (a multiple of 16) with one
  * 16-byte element per thread, the access shape of the per-Gaussian kernels.  mode 0 reads src,
- * 1 writes dst, 2 copies src to dst; mode 3 moves `bytes` in all as 10 arrays read and 18
- * arrays written per thread (src holds 10/28 of `bytes`, dst 18/28): the stream count and
- * write share of the per-Gaussian backward.  Traced as "stream_probe_kernel".  No counterpart in
- * the reference. */
+ * 1 writes dst, 2 copies src to dst; modes 3 and 4 move `bytes` in all as 10 arrays read and 18
+ * written per thread (src holds 10/28 of `bytes`, dst 18/28), respectively 5 and 9: write-heavy
+ * mixes of many streams like the per-Gaussian backward's.  Traced as "stream_probe_kernel".
+ * No counterpart in the reference. */
 int dsx_stream_probe(const void* src, void* dst, size_t bytes, int mode, void* stream);
 
 #ifdef __cplusplus
