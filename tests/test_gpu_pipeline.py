@@ -376,3 +376,48 @@ def test_a_sort_that_gave_up_poisons_the_image():
     torch.cuda.synchronize()
     assert torch.isnan(image).all()
 
+
+def test_api_rejects_bad_inputs_with_the_reference_messages():
+    """cpp/rasterizer_torch.cu:176-190 and :124-129: every check fires before anything is launched."""
+    from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
+    sc = make_scene("cfg0", n=64, width=32, height=32, sh_degree=1)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+
+    def settings(sh_degree=1, max_sh_degree=3):
+        return GaussianRasterizationSettings(32, 32, sc["tanfovx"], sc["tanfovy"], t["bg"], 1.0, t["viewmatrix"],
+                                             t["projmatrix"], sh_degree, max_sh_degree, t["campos"], False, False)
+
+    good = dict(means_3d=t["means_3d"], means_2d=torch.zeros_like(t["means_3d"]), shs=t["shs"], colors_precomp=None,
+                opacities=t["opacities"], scales=t["scales"], rotations=t["rotations"], cov_3d_precomp=None)
+
+    def run(s=None, **change):
+        a = dict(good)
+        a.update(change)
+        return GaussianRasterizer(s or settings())(a["means_3d"], a["means_2d"], a["shs"], a["colors_precomp"],
+                                                   a["opacities"], a["scales"], a["rotations"], a["cov_3d_precomp"])
+
+    image, radii = run()
+    assert image.shape == (32, 32, 3)
+    cases = [
+        (dict(means_3d=t["means_3d"].t().contiguous().t()), "means_3d must be contiguous"),
+        (dict(opacities=sc["opacities"]), "opacities must be a CUDA tensor"),
+        (dict(shs=t["shs"].transpose(1, 2)), "shs error"),
+        (dict(scales=sc["scales"]), "scales error"),
+        (dict(rotations=t["rotations"].t().contiguous().t()), "rotations error"),
+        (dict(scales=None, rotations=None), "cov3D error"),
+        (dict(shs=None), "SHS error"),
+        (dict(scales=t["scales"].double()), "scales must be float32"),
+        (dict(opacities=t["opacities"][:10].contiguous()), "opacities must have one entry per Gaussian"),
+        (dict(shs=t["shs"][:, :4].contiguous()), r"shs must have shape"),
+        (dict(rotations=t["rotations"][:, :3].contiguous()), r"scales must be \[N,3\] and rotations \[N,4\]"),
+        (dict(scales=None, rotations=None, cov_3d_precomp=torch.zeros(10, 6, device=DEV)), r"cov3D_precomp must be"),
+        (dict(shs=None, colors_precomp=torch.zeros(10, 3, device=DEV)), r"colors_precomp must be"),
+    ]
+    for change, message in cases:
+        with pytest.raises(RuntimeError, match=message):
+            run(**change)
+    with pytest.raises(RuntimeError, match="sh_degree must be in"):
+        run(s=settings(sh_degree=4))
+    with pytest.raises(RuntimeError, match="sh_degree must be in"):
+        run(s=settings(max_sh_degree=2))
+
