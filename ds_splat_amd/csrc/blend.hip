@@ -77,9 +77,9 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     const int start = ranges[tile];
     const int end = ranges[tile + 1];
 
-    // A pixel that has stopped (or lies outside the image) gets the row coordinate +infinity:
-    // its exponent is then -infinity (or NaN for a degenerate conic), its alpha fails the
-    // threshold test, and the loop needs no per-pixel flag.  `alive` counts the lane's live pixels.
+    // A pixel that has stopped (or lies outside the image) gets NaN as its row coordinate: its
+    // exponent is then NaN, the test `power < 0` fails whatever the entry holds, and the loop
+    // needs no per-pixel flag.  `alive` counts the lane's live pixels.
     float pyf[kFwdPix], T[kFwdPix], cr[kFwdPix], cg[kFwdPix], cb[kFwdPix];
     int last[kFwdPix];
     int alive = 0;
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     {
         const int y = y0 + 4 * p;
         const bool inside = x < W && y < H;
-        pyf[p] = inside ? (float)y + 0.5f : __builtin_inff();
+        pyf[p] = inside ? (float)y + 0.5f : __builtin_nanf("");
         alive += inside ? 1 : 0;
         T[p] = 1.0f;
         cr[p] = cg[p] = cb[p] = 0.0f;
@@ -141,9 +141,9 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                 {
                     const float dy = pyf[p] - A.y;
                     const float power = ax - (0.5f * B.x * dy + bx) * dy;
-                    const float raw = B.y * fast_exp(power);
-                    const bool pass = power < 0.0f && raw >= kAlphaThreshold; // false for NaN
-                    const float alpha = fminf(0.999f, raw);
+                    // (a NaN opacity gives alpha = 0.999 here as in the reference: fminf drops the NaN)
+                    const float alpha = fminf(0.999f, B.y * fast_exp(power));
+                    const bool pass = power < 0.0f && alpha >= kAlphaThreshold;
                     const float Tn = (1.0f - alpha) * T[p];
                     const bool stop = pass && Tn < 0.0001f;
                     const bool apply = pass && !stop;
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                     cb[p] += vis * C;
                     T[p] = apply ? Tn : T[p];
                     last[p] = apply ? b + i : last[p];
-                    pyf[p] = stop ? __builtin_inff() : pyf[p];
+                    pyf[p] = stop ? __builtin_nanf("") : pyf[p];
                     alive -= stop ? 1 : 0;
                 }
             }

@@ -421,3 +421,39 @@ def test_api_rejects_bad_inputs_with_the_reference_messages():
     with pytest.raises(RuntimeError, match="sh_degree must be in"):
         run(s=settings(max_sh_degree=2))
 
+
+def test_non_finite_gaussians_are_culled_and_leave_the_rest_alone():
+    """NaN / infinite means and scales fail the frustum or determinant test (radius 0): the image
+    and every other Gaussian's gradient equal those of a scene where the same Gaussians sit far
+    outside the view.  A NaN opacity is not a culling criterion (the reference blends it with
+    alpha 0.999, cpp/rasterizer_kernels.cu:341-431): that scene must simply run to completion."""
+    sc = make_scene("cfg1", n=20000, width=320, height=200, sh_degree=2)
+    bad = torch.arange(5000, 5030)
+    clean = dict(sc)
+    clean["means_3d"] = sc["means_3d"].clone()
+    clean["means_3d"][bad, 0] += 1.0e4                      # far outside the frustum
+    dirty = dict(sc)
+    dirty["means_3d"] = sc["means_3d"].clone()
+    dirty["scales"] = sc["scales"].clone()
+    dirty["means_3d"][bad[:10], 1] = float("nan")
+    dirty["scales"][bad[10:20], 2] = float("nan")
+    dirty["scales"][bad[20:30], 0] = float("inf")
+    img_c, radii_c, leaves_c = api_run(clean, 2.0)
+    img_d, radii_d, leaves_d = api_run(dirty, 2.0)
+    assert (radii_d[bad] == 0).all() and (radii_c[bad] == 0).all()
+    assert torch.equal(radii_c, radii_d)
+    assert torch.equal(img_c, img_d)
+    keep = torch.ones(20000, dtype=torch.bool, device=DEV)
+    keep[bad] = False
+    for name in ("means", "shs", "opac", "scales", "rots"):
+        gc, gd = leaves_c[name].grad, leaves_d[name].grad
+        assert torch.isfinite(gd[keep]).all()
+        scale = float(gc.abs().max())
+        assert torch.allclose(gc[keep], gd[keep], rtol=1e-3, atol=1e-4 * max(1.0, scale)), name
+    nan_opacity = dict(sc)
+    nan_opacity["opacities"] = sc["opacities"].clone()
+    nan_opacity["opacities"][bad[:5]] = float("nan")
+    img_n, radii_n, _ = api_run(nan_opacity, 2.0)
+    assert img_n.shape == img_c.shape and torch.equal(radii_n > 0, (radii_c > 0) | torch.isin(
+        torch.arange(20000, device=DEV), bad.to(DEV)) & (radii_n > 0))
+
