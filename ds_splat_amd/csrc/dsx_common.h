@@ -121,6 +121,9 @@ constexpr int kListSortThreads = DSX_KSORT_THREADS;
 constexpr int kListSortItems = DSX_KSORT_ITEMS;
 constexpr int kListSortTile = kListSortThreads * kListSortItems;
 constexpr int kMaxPasses32 = 4;
+// depth key of a Gaussian that emits no (tile, Gaussian) pair; as a float it is a NaN, which no
+// emitting Gaussian has (a NaN depth fails the frustum test)
+constexpr uint32_t kNoPairsKey = 0xffffffffu;
 
 // Digits of a key whose low `key_bits` bits are significant: fewest passes with digits of at
 // most 8 bits, bits spread evenly.

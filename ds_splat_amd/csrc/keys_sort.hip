@@ -132,7 +132,11 @@ __global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* data, 
             carry_s = run;
         __syncthreads();
     }
-    if(mine64)
+    // one LDS atomic per wavefront (1024 same-address atomics would cost more than the scan)
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1)
+        mine64 += __shfl_xor(mine64, o, DSX_WAVE);
+    if(lane == 0 && mine64)
         atomicAdd(&total64, mine64);
     __syncthreads();
     if(tid == 0)

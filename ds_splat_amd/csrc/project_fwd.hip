@@ -407,8 +407,11 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
         if(p.depth_keys)
         {
             // x = sx | sy << 16, y = width | height << 16 | (depth sign) << 31
+            // A Gaussian that emits no pair gets the all-ones key: it sorts behind every Gaussian
+            // that does (their order among themselves is immaterial) and tells the depth sort that
+            // its rectangle is empty without a look at it.
             const uint32_t depth_bits = __float_as_uint(vz);
-            p.depth_keys[i] = depth_bits;
+            p.depth_keys[i] = count ? depth_bits : kNoPairsKey;
             p.rects[i] = count ? make_uint2((uint32_t)r.sx | ((uint32_t)r.sy << 16),
                                             (uint32_t)(r.ex - r.sx) | ((uint32_t)(r.ey - r.sy) << 16) |
                                                 (depth_bits & 0x80000000u))

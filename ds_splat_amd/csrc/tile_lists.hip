@@ -99,9 +99,6 @@ __device__ __forceinline__ uint64_t match_digit8(uint32_t d, int bits)
 #ifndef DSX_HIST_BLOCKS
 #define DSX_HIST_BLOCKS 512 // few workgroups: each ends with one global atomic per bin, which serialise per address
 #endif
-#ifndef DSX_EMIT_BLOCKS
-#define DSX_EMIT_BLOCKS 2048
-#endif
 // 1024 threads share one LDS histogram: the kernel is bound by latency (3 M keys are few), so
 // it wants many wavefronts per CU, while every further workgroup adds a flush of up to 1024
 // contended global atomics (256 threads: 0.029 ms, 1024 threads: 0.020 ms at 3 M keys)
@@ -139,6 +136,9 @@ __global__ __launch_bounds__(kHist32Threads) void hist32_kernel(const KeyT* __re
             // significant digit takes few values (the exponent byte of depths, the high bits of
             // a tile slot): one add per distinct value of the wavefront, after a ballot, because
             // LDS atomics on one address serialise.
+            // (the all-ones depth keys of Gaussians that emit nothing, a third of a typical scene,
+            // share one bin in every digit; counting them apart, once per wavefront, was measured
+            // slower than letting their atomics serialise: 0.034 against 0.025 ms)
             for(int p = 0; p + 1 < plan.passes; ++p)
                 if(valid[it])
                     atomicAdd(&hist[p * kBins32 + ((s[it] >> plan.shift[p]) & plan.mask[p])], 1u);
@@ -186,7 +186,8 @@ static_assert(kDepthSortTile <= 65535 && kListSortTile <= 65535, "u16 ranks");
 
 // vals_in == nullptr: the values are the input positions (iota).  keys_out == nullptr: the
 // keys are not needed after this pass.  gather_src != nullptr: gather_dst[position] =
-// gather_src[value] for every pair.  KeyT: uint32_t, or uint16_t for tile slots that fit.
+// gather_src[value] for every pair, except that a pair whose key is kNoPairsKey gets a zero
+// record without the read.  KeyT: uint32_t, or uint16_t for tile slots that fit.
 template <typename KeyT, int kSort32Threads, int kSort32Items>
 __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     const KeyT* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, KeyT* __restrict__ keys_out,
@@ -373,6 +374,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
 
     // ---- scatter keys: consecutive threads -> consecutive addresses inside a digit's run ----
     uint32_t dig4[(kSort32Items + 3) / 4]; // the digit of the key at tile position it * threads + tid, 8 bits each
+    uint32_t no_record = 0;                // bit it: that key is kNoPairsKey (its record is known to be zero)
 #pragma unroll
     for(int it = 0; it < kSort32Items; ++it)
     {
@@ -387,6 +389,8 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
             const uint32_t kk = s_keys[j];
             const uint32_t d = (kk >> shift) & mask;
             dig4[it >> 2] |= d << (8 * (it & 3));
+            if(gather_src && kk == kNoPairsKey)
+                no_record |= 1u << it;
             if(keys_out)
                 keys_out[s_gbase[d] + (uint32_t)j] = (KeyT)kk;
         }
@@ -414,7 +418,7 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
             // optional: a per-value record follows its value to the sorted position (the random
             // gather overlaps with the scatter traffic of the pass)
             if(gather_src)
-                gather_dst[out] = gather_src[v];
+                gather_dst[out] = ((no_record >> it) & 1u) ? make_uint2(0u, 0u) : gather_src[v];
         }
     }
 }
@@ -892,6 +896,13 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
 // OUTPUT pair, so stores are contiguous however uneven the per-Gaussian tile counts are
 // ---------------------------------------------------------------------------------------
 
+#ifndef DSX_EMIT_WINDOWS
+#define DSX_EMIT_WINDOWS 4
+#endif
+constexpr int kEmitWindows = DSX_EMIT_WINDOWS; // windows of 256 outputs per round of the emission
+constexpr int kEmitChunkMax = 4096;            // outputs per workgroup: at most this many ...
+constexpr int kEmitWorkgroups = 4096;          // ... and fewer when that leaves less than this many workgroups
+
 template <typename SlotT>
 __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t* __restrict__ order,
                                                                   const uint2* __restrict__ rects_sorted,
@@ -900,7 +911,8 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
                                                                   SlotT* __restrict__ slots, int32_t* __restrict__ ids,
                                                                   const int32_t* __restrict__ ranges_in,
                                                                   int32_t* __restrict__ ranges_out, int range_count,
-                                                                  uint32_t* __restrict__ clear, int64_t clear_words)
+                                                                  uint32_t* __restrict__ clear, int64_t clear_words,
+                                                                  int chunk)
 {
     __shared__ uint32_t s_off[kProjBlock + 1];
     __shared__ uint32_t s_origin[kProjBlock]; // slot of the rectangle's first tile (0 for negative depths)
@@ -908,14 +920,16 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     __shared__ float s_winv[kProjBlock];
     __shared__ uint32_t s_id[kProjBlock];
     __shared__ uint32_t wave_tot[kProjBlock / DSX_WAVE];
-    __shared__ uint32_t s_mark[kProjBlock];
-    __shared__ uint32_t s_wave_max[kProjBlock / DSX_WAVE];
+    __shared__ uint32_t s_mark[kEmitWindows * kProjBlock];
+    __shared__ uint32_t s_wave_max[kEmitWindows][kProjBlock / DSX_WAVE];
     static_assert(kProjBlock == 4 * DSX_WAVE, "four wavefronts per workgroup");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    s_mark[tid] = 0;
+#pragma unroll
+    for(int wdw = 0; wdw < kEmitWindows; ++wdw)
+        s_mark[wdw * kProjBlock + tid] = 0;
 
     // the tile ranges were derived from the rectangles before any pair existed: hand them out
     for(int j = blockIdx.x * kProjBlock + tid; j < range_count; j += gridDim.x * kProjBlock)
@@ -924,9 +938,35 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     for(int64_t j = (int64_t)blockIdx.x * kProjBlock + tid; j < clear_words; j += (int64_t)gridDim.x * kProjBlock)
         clear[j] = 0u;
 
+    // This workgroup's share: outputs [o0, o1).  The work is cut by OUTPUTS, not by Gaussians: a
+    // block of 256 near Gaussians can own a hundred thousand pairs and a block of far ones a few
+    // hundred, and a workgroup that walked a whole heavy block alone set the kernel's time.
+    const int64_t o0 = (int64_t)blockIdx.x * chunk;
+    const int64_t o1 = min(o0 + chunk, k);
+    if(o0 >= o1) // uniform
+        return;
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
-    for(int64_t blk = blockIdx.x; blk < blocks; blk += gridDim.x)
+    // first block of 256 Gaussians (in depth order) whose outputs reach into the share: the largest
+    // b with block_offsets[b] <= o0, by a 64-way search (every wavefront does it for itself)
+    int64_t first = 0;
     {
+        int64_t lo = 0, hi = blocks; // block_offsets[lo] <= o0; the answer lies in [lo, hi)
+        while(hi - lo > 1)
+        {
+            const int64_t step = (hi - lo + 63) / 64;
+            const int64_t probe = lo + lane * step;
+            const bool ok = probe < hi && (int64_t)block_offsets[probe] <= o0; // true for a prefix of the lanes
+            const int reached = __popcll(__ballot(ok)) - 1;                   // lane 0 always holds
+            lo += reached * step;
+            hi = min(hi, lo + step);
+        }
+        first = lo;
+    }
+    for(int64_t blk = first; blk < blocks; ++blk)
+    {
+        const int64_t base = block_offsets[blk];
+        if(base >= o1) // uniform: the share is complete
+            break;
         __syncthreads(); // the previous round has finished with the LDS arrays
         const int64_t p = blk * kProjBlock + tid;
         uint32_t count = 0;
@@ -955,50 +995,79 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
         __syncthreads();
 
         const uint32_t total = s_off[kProjBlock];
-        const int64_t base = block_offsets[blk];
         const uint32_t my_start = s_off[tid];
+        // the block's outputs that fall into the share: [ja, jb) of its `total`
+        const uint32_t ja = (uint32_t)(max(o0, base) - base);
+        const uint32_t jb = (uint32_t)(min(o1, base + (int64_t)total) - base);
+        if(jb <= ja) // uniform (an empty block, or one that ends before the share)
+            continue;
         // Which Gaussian owns output j?  Every Gaussian that emits marks the output where its run
         // starts with (its index + 1); the owner of j is the largest mark at or before j, i.e. an
         // inclusive max-scan over the outputs (DPP inside the wavefront, LDS across wavefronts
         // and across rounds of 256 outputs).  Costs a dozen VALU instructions per output
         // instead of the eight dependent LDS reads of a binary search.
-        uint32_t carry = 0; // mark of the owner of the last output of the previous round
-        for(uint32_t j0 = 0; j0 < total; j0 += kProjBlock) // uniform
+        // A block of near Gaussians can own tens of thousands of outputs while the workgroup
+        // walks them serially, so a round covers kEmitWindows windows of 256 outputs with two
+        // barriers in all (the kernel's time is the longest such walk).
+        uint32_t carry = 0; // mark of the owner of the last output before the round
+        if(ja > 0)          // uniform: the share starts inside the block
         {
-            if(count && my_start >= j0 && my_start < j0 + kProjBlock)
+            // the last Gaussian whose run starts before ja (starts are monotone in the thread index)
+            const uint64_t early = __ballot(count && my_start < ja);
+            if(lane == 0)
+                s_wave_max[0][wave] = early ? (uint32_t)(wave * DSX_WAVE + 64 - __builtin_clzll(early)) : 0u;
+            __syncthreads();
+            carry = max(max(s_wave_max[0][0], s_wave_max[0][1]), max(s_wave_max[0][2], s_wave_max[0][3]));
+            __syncthreads();
+        }
+        for(uint32_t j0 = ja; j0 < jb; j0 += kEmitWindows * kProjBlock) // uniform
+        {
+            if(count && my_start >= j0 && my_start < j0 + kEmitWindows * kProjBlock)
                 s_mark[my_start - j0] = (uint32_t)tid + 1u;
             __syncthreads();
-            uint32_t m = s_mark[tid];
-            s_mark[tid] = 0; // ready for the next round (and the next block)
-            m = wave_incl_max_scan(m);
-            if(lane == 63)
-                s_wave_max[wave] = m;
-            __syncthreads();
-            uint32_t before = carry;
-            for(int w = 0; w < wave; ++w)
-                before = max(before, s_wave_max[w]);
-            const uint32_t owner = max(m, before) - 1u; // every output has an owner: never 0 - 1
-            carry = max(max(max(s_wave_max[0], s_wave_max[1]), max(s_wave_max[2], s_wave_max[3])), carry);
-            const uint32_t j = j0 + tid;
-            if(j < total && base + j < k)
+            uint32_t m[kEmitWindows];
+#pragma unroll
+            for(int wdw = 0; wdw < kEmitWindows; ++wdw)
             {
-                const uint32_t r = j - s_off[owner];
-                const uint32_t w = s_w[owner];
-                uint32_t slot = 0;
-                if(w)
-                {
-                    // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
-                    uint32_t ry = (uint32_t)((float)r * s_winv[owner]);
-                    if(ry * w > r)
-                        --ry;
-                    else if((ry + 1) * w <= r)
-                        ++ry;
-                    const uint32_t rx = r - ry * w;
-                    slot = s_origin[owner] + ry * (uint32_t)ntx + rx;
-                }
-                slots[base + j] = (SlotT)slot;
-                ids[base + j] = (int32_t)s_id[owner];
+                m[wdw] = s_mark[wdw * kProjBlock + tid];
+                s_mark[wdw * kProjBlock + tid] = 0; // ready for the next round (and the next block)
+                m[wdw] = wave_incl_max_scan(m[wdw]);
+                if(lane == 63)
+                    s_wave_max[wdw][wave] = m[wdw];
             }
+            __syncthreads();
+            uint32_t before = carry; // largest mark before this thread's output of the current window
+#pragma unroll
+            for(int wdw = 0; wdw < kEmitWindows; ++wdw)
+            {
+                uint32_t mine = before;
+                for(int w = 0; w < wave; ++w)
+                    mine = max(mine, s_wave_max[wdw][w]);
+                const uint32_t owner = max(m[wdw], mine) - 1u; // every output has an owner: never 0 - 1
+                before = max(before, max(max(s_wave_max[wdw][0], s_wave_max[wdw][1]),
+                                         max(s_wave_max[wdw][2], s_wave_max[wdw][3])));
+                const uint32_t j = j0 + wdw * kProjBlock + tid;
+                if(j < jb)
+                {
+                    const uint32_t r = j - s_off[owner];
+                    const uint32_t w = s_w[owner];
+                    uint32_t slot = 0;
+                    if(w)
+                    {
+                        // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
+                        uint32_t ry = (uint32_t)((float)r * s_winv[owner]);
+                        if(ry * w > r)
+                            --ry;
+                        else if((ry + 1) * w <= r)
+                            ++ry;
+                        const uint32_t rx = r - ry * w;
+                        slot = s_origin[owner] + ry * (uint32_t)ntx + rx;
+                    }
+                    slots[base + j] = (SlotT)slot;
+                    ids[base + j] = (int32_t)s_id[owner];
+                }
+            }
+            carry = before;
             // (the next round's marks are written after this round's reads of s_wave_max: the
             // barrier after them orders both)
         }
@@ -1054,16 +1123,18 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
     uint32_t* vals_b = even ? ids_other : ids_final;
     int rc = DSX_OK;
     const Sort32Workspace sw = sort32_workspace(k, bits, kListSortTile);
-    const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     {
         DSX_TIMED("emit_ordered_kernel", stream);
-        hipLaunchKernelGGL(emit_ordered_kernel<SlotT>, dim3((unsigned)min(blocks, (int64_t)DSX_EMIT_BLOCKS)), dim3(kProjBlock),
+        // outputs per workgroup: a multiple of 256 between 256 and kEmitChunkMax
+        const int64_t want = (k + kEmitWorkgroups - 1) / kEmitWorkgroups;
+        const int chunk = (int)min((int64_t)kEmitChunkMax, ((want + kProjBlock - 1) / kProjBlock) * kProjBlock);
+        hipLaunchKernelGGL(emit_ordered_kernel<SlotT>, dim3((unsigned)((k + chunk - 1) / chunk)), dim3(kProjBlock),
                            0, stream, reinterpret_cast<const uint32_t*>(obase + o.ids_a),
                            reinterpret_cast<const uint2*>(obase + o.rects_sorted),
                            reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k, tiles_x(cam.image_width),
                            slots_a, reinterpret_cast<int32_t*>(vals_a),
                            reinterpret_cast<const int32_t*>(obase + o.ranges), ranges, num_tiles + 1,
-                           reinterpret_cast<uint32_t*>(base + w.sort + sw.hist), (int64_t)(sw.bytes / 4));
+                           reinterpret_cast<uint32_t*>(base + w.sort + sw.hist), (int64_t)(sw.bytes / 4), chunk);
     }
     DSX_LAUNCH_CHECK();
     SlotT* ko;

@@ -273,7 +273,9 @@ def test_full_size_properties_cfg2():
     # same lists as the 64-bit sort of all keys
     perm, offsets = stages.depth_order(cam, n, order)
     assert int(offsets[-1]) == k
-    d_sorted = (depth_bits & 0xFFFFFFFF)[perm.to(torch.int64)]       # unsigned order of the depth bits
+    # unsigned order of the depth bits; Gaussians that emit nothing come last (all-ones key)
+    sort_key = torch.where(tiles_eff > 0, depth_bits & 0xFFFFFFFF, torch.full_like(depth_bits, 0xFFFFFFFF))
+    d_sorted = sort_key[perm.to(torch.int64)]
     assert (d_sorted[1:] >= d_sorted[:-1]).all()
     ids_fast, ranges_fast, flags = stages.tile_lists(cam, n, k, order, return_flags=True)
     assert flags == (0, 0)

@@ -39,12 +39,16 @@ def pack_splats(S, radii, opac):
 
 
 def oracle_scene(oracle, name="cfg0", n=20000, W=256, H=256, sh_degree=3, seed=None, scale_mul=1.0,
-                 flip_behind=0):
+                 flip_behind=0, giants=0):
     sc = make_scene(name, n=n, width=W, height=H, sh_degree=sh_degree, seed=seed)
     A = arrays(sc)
     A["scales"] = (A["scales"] * scale_mul).astype(np.float32)
     if flip_behind:
         A["means_3d"][:flip_behind, 2] *= -1.0
+    if giants:
+        # a few Gaussians that cover most of the screen among many small ones
+        pick = np.linspace(n // 7, n - n // 5, giants).astype(np.int64)
+        A["scales"][pick] *= 150.0
     s = scene_settings(sc)
     img, radii, st = oracle.forward(s, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["shs"],
                                     keep_emitted=True)
@@ -257,14 +261,14 @@ def test_sort_pairs_u32_orders_depth_bits_like_the_64_bit_keys():
                                                   (60000, 512, 384, 3.0, 500), (4000, 40, 30, 8.0, 50),
                                                   (30000, 3840, 2160, 6.0, 300), (20000, 16400, 1040, 8.0, 100),
                                                   (40, 640, 480, 1.0, 0), (60, 1920, 1080, 2.0, 30)])
-def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip):
+def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip, giants=0):
     """Depth order + ordered emission + tile partition give the oracle's sorted ids and ranges
     (the result of the stable 64-bit sort of the emitted keys) bit for bit, including keys with
     negative depths, the last Gaussian that never emits, 1-pass (<= 255 tiles) and 4K plans, and
     an image of more than 65534 tiles (32-bit instead of 16-bit tile slots)."""
     st_ = _stages()
     sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=11 + n, scale_mul=scale_mul,
-                                               flip_behind=flip)
+                                               flip_behind=flip, giants=giants)
     oracle.free(st)
     k = S["num_keys"]
     cam = st_.camera_from_scene(sc, DEV)
@@ -275,9 +279,11 @@ def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip):
     perm, offsets = st_.depth_order(cam, n, order)
     torch.cuda.synchronize()
     depth_bits = splats[:, 2].contiguous().view(torch.int32).cpu().numpy().view(np.uint32)
-    assert (perm.cpu().numpy() == np.argsort(depth_bits, kind="stable")).all()
     tt = S["tiles_touched"].astype(np.int64).copy()
     tt[-1] = 0
+    # Gaussians that emit nothing carry the all-ones key: behind all others, in index order
+    sort_keys = np.where(tt > 0, depth_bits, np.uint32(0xFFFFFFFF))
+    assert (perm.cpu().numpy() == np.argsort(sort_keys, kind="stable")).all()
     tt_sorted = tt[perm.cpu().numpy()]
     pad = np.zeros((-n) % 256, np.int64)
     sums = np.concatenate([tt_sorted, pad]).reshape(-1, 256).sum(1)
@@ -294,6 +300,13 @@ def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip):
         # one repeat the START of its run (the reference never records the boundary after it)
         r = S["ranges"]
         assert r[-1] == k and r[-2] < k and (np.diff(r[:-1]) == 0).sum() > 100
+
+
+def test_tile_lists_with_a_few_screen_filling_gaussians(oracle):
+    """Tile counts from 1 to the whole screen in one scene: the emission cuts its work by output
+    pairs, so one block of 256 Gaussians is shared by many workgroups and one workgroup spans
+    many blocks."""
+    test_tile_lists_bit_exact(oracle, 30000, 1280, 720, 0.5, 40, giants=25)
 
 
 # ------------------------------------------------------------------------------- stage 3
