@@ -915,10 +915,9 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
                                                                   int chunk)
 {
     __shared__ uint32_t s_off[kProjBlock + 1];
-    __shared__ uint32_t s_origin[kProjBlock]; // slot of the rectangle's first tile (0 for negative depths)
-    __shared__ uint32_t s_w[kProjBlock];      // width; 0 marks a negative depth (every pair goes to slot 0)
-    __shared__ float s_winv[kProjBlock];
-    __shared__ uint32_t s_id[kProjBlock];
+    // per Gaussian of the block: x = first output, y = slot of the rectangle's first tile (0 for
+    // negative depths), z = width (0 marks a negative depth: every pair goes to slot 0), w = id
+    __shared__ uint4 s_rec[kProjBlock];
     __shared__ uint32_t wave_tot[kProjBlock / DSX_WAVE];
     __shared__ uint32_t s_mark[kEmitWindows * kProjBlock];
     __shared__ uint32_t s_wave_max[kEmitWindows][kProjBlock / DSX_WAVE];
@@ -970,6 +969,7 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
         __syncthreads(); // the previous round has finished with the LDS arrays
         const int64_t p = blk * kProjBlock + tid;
         uint32_t count = 0;
+        uint4 rec = make_uint4(0u, 0u, 0u, 0u);
         if(p < n)
         {
             const uint32_t g = order[p];
@@ -977,10 +977,9 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
             count = rect_count(r);
             const uint32_t w = r.y & 0xffffu;
             const bool negative = (r.y >> 31) != 0;
-            s_origin[tid] = negative ? 0u : (r.x >> 16) * (uint32_t)ntx + (r.x & 0xffffu) + 1u;
-            s_w[tid] = negative ? 0u : w;
-            s_winv[tid] = 1.0f / (float)(w ? w : 1u);
-            s_id[tid] = g;
+            rec.y = negative ? 0u : (r.x >> 16) * (uint32_t)ntx + (r.x & 0xffffu) + 1u;
+            rec.z = negative ? 0u : w;
+            rec.w = g;
         }
         const uint32_t incl = wave_incl_scan32(count, lane);
         if(lane == 63)
@@ -989,7 +988,9 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
         uint32_t prefix = 0;
         for(int w = 0; w < wave; ++w)
             prefix += wave_tot[w];
-        s_off[tid] = prefix + incl - count;
+        rec.x = prefix + incl - count;
+        s_off[tid] = rec.x;
+        s_rec[tid] = rec;
         if(tid == kProjBlock - 1)
             s_off[kProjBlock] = prefix + incl;
         __syncthreads();
@@ -1049,22 +1050,23 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
                 const uint32_t j = j0 + wdw * kProjBlock + tid;
                 if(j < jb)
                 {
-                    const uint32_t r = j - s_off[owner];
-                    const uint32_t w = s_w[owner];
+                    const uint4 own = s_rec[owner]; // one 16-byte LDS read per output
+                    const uint32_t r = j - own.x;
+                    const uint32_t w = own.z;
                     uint32_t slot = 0;
                     if(w)
                     {
                         // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
-                        uint32_t ry = (uint32_t)((float)r * s_winv[owner]);
+                        uint32_t ry = (uint32_t)((float)r * __builtin_amdgcn_rcpf((float)w));
                         if(ry * w > r)
                             --ry;
                         else if((ry + 1) * w <= r)
                             ++ry;
                         const uint32_t rx = r - ry * w;
-                        slot = s_origin[owner] + ry * (uint32_t)ntx + rx;
+                        slot = own.y + ry * (uint32_t)ntx + rx;
                     }
                     slots[base + j] = (SlotT)slot;
-                    ids[base + j] = (int32_t)s_id[owner];
+                    ids[base + j] = (int32_t)own.w;
                 }
             }
             carry = before;
