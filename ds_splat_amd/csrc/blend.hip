@@ -388,7 +388,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             float g[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; // v_x, v_y, v_conic a b c, v_opacity, v_red, v_green
             float g_blue = 0.f;
             // dx is the same for the lane's four pixels, so the five geometric sums are built from
-            // three moments of v_sigma over dy: S0 = sum v_sigma, S1 = sum v_sigma dy, S2 = sum v_sigma dy^2
+            // three moments over dy of vis * v_alpha (v_sigma without its factor -opacity): S0, S1 (times dy), S2 (times dy^2)
             float S0 = 0.f, S1 = 0.f, S2 = 0.f;
 #pragma unroll
             for(int p = 0; p < kBwdPix; ++p)
@@ -404,19 +404,23 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
                     const float rv = B.z * vo0[p] + B.w * vo1[p] + blue * vo2[p];
                     const float v_alpha = rv * T[p] + bterm[p] * ra;
                     bterm[p] -= rv * fac;
-                    const float v_sigma = -B.y * vis[p] * v_alpha;
-                    const float vsdy = v_sigma * dy[p];
-                    S0 += v_sigma;
-                    S1 += vsdy;
-                    S2 += vsdy * dy[p];
-                    g[5] += vis[p] * v_alpha;
+                    // v_sigma = -opacity * vis * v_alpha: the moments are taken of vis * v_alpha (which is
+                    // v_opacity's own term) and the common factor -opacity is applied once per entry
+                    const float va = vis[p] * v_alpha;
+                    const float vady = va * dy[p];
+                    S0 += va;
+                    S1 += vady;
+                    S2 += vady * dy[p];
                 }
             }
+            g[5] = S0; // v_opacity
+            S0 *= -B.y;
+            S1 *= -B.y;
             g[0] = A.z * dx * S0 + A.w * S1; // v_sigma (a dx + b dy)
             g[1] = bdx * S0 + B.x * S1;      // v_sigma (b dx + c dy)
             g[2] = 0.5f * dx * dx * S0;
             g[3] = dx * S1;
-            g[4] = 0.5f * S2;
+            g[4] = -0.5f * B.y * S2;
             const float total = wave_sum8_scatter(g, lane);
             g_blue = wave_sum_to_lane63(g_blue);
             if(lane >= 56)
