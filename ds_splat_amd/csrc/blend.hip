@@ -14,6 +14,31 @@ __device__ __forceinline__ float fast_exp(float x)
     return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
 }
 
+// The exponent of a splat at a pixel, -1/2 (a dx^2 + c dy^2) - b dx dy with d = pixel - mean, in
+// ONE fixed sequence of roundings (explicit fused multiply-adds, no contraction left to the
+// compiler): the forward and the backward kernel must get the same bits, because both compare the
+// resulting alpha with 1/255 on their own.  If they disagreed on a borderline entry, the backward
+// would rebuild the transmittance of every entry in front of it from a final value that does
+// (or does not) contain its factor: an error of alpha in all their gradients at that pixel.
+struct ExponentX
+{
+    float ax, bx; // -1/2 a dx^2 and b dx
+};
+__device__ __forceinline__ ExponentX exponent_x(float a, float b, float dx)
+{
+#pragma clang fp contract(off)
+    ExponentX r;
+    r.bx = b * dx;
+    r.ax = -0.5f * a * dx * dx;
+    return r;
+}
+__device__ __forceinline__ float exponent_xy(ExponentX x, float c, float dy)
+{
+#pragma clang fp contract(off)
+    const float inner = __builtin_fmaf(0.5f * c, dy, x.bx);
+    return __builtin_fmaf(-inner, dy, x.ax);
+}
+
 // Can this entry reach alpha >= 1/255 at ANY pixel of the tile?  The exponent's quadratic form
 // q(d) = 1/2 (a dx^2 + c dy^2) + b dx dy is convex, so its minimum over the box of pixel
 // centres is 0 if the centre lies inside and otherwise sits on one of the four edges, where it
@@ -133,14 +158,11 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                 const float4 A = s_a[i];
                 const float4 B = s_b[i];
                 const float C = s_c[i];
-                const float dx = pxf - A.x;
-                const float bx = A.w * dx;              // conic b * dx
-                const float ax = -0.5f * A.z * dx * dx; // -1/2 conic a * dx^2
+                const ExponentX ex = exponent_x(A.z, A.w, pxf - A.x);
 #pragma unroll
                 for(int p = 0; p < kFwdPix; ++p)
                 {
-                    const float dy = pyf[p] - A.y;
-                    const float power = ax - (0.5f * B.x * dy + bx) * dy;
+                    const float power = exponent_xy(ex, B.x, pyf[p] - A.y);
                     // (a NaN opacity gives alpha = 0.999 here as in the reference: fminf drops the NaN)
                     const float alpha = fminf(0.999f, B.y * fast_exp(power));
                     const bool pass = power < 0.0f && alpha >= kAlphaThreshold;
@@ -366,20 +388,20 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             const int idx = top - t;
             const float4 A = s_a[t];
             const float4 B = s_b[t];
-            const float dx = A.x - pxf;
-            const float adx2 = A.z * dx * dx;
-            const float bdx = A.w * dx;
-            float alpha[kBwdPix], vis[kBwdPix], dy[kBwdPix];
+            // the exponent exactly as the forward computed it (pixel - mean); sigma = -exponent
+            const float dxf = pxf - A.x;
+            const ExponentX ex = exponent_x(A.z, A.w, dxf);
+            float alpha[kBwdPix], vis[kBwdPix], dy[kBwdPix]; // dy = pixel - mean here
             bool valid[kBwdPix];
             bool any = false;
 #pragma unroll
             for(int p = 0; p < kBwdPix; ++p)
             {
-                dy[p] = A.y - pyf[p];
-                const float sigma = 0.5f * (adx2 + B.x * dy[p] * dy[p]) + bdx * dy[p];
-                vis[p] = fast_exp(-sigma);
+                dy[p] = pyf[p] - A.y;
+                const float power = exponent_xy(ex, B.x, dy[p]);
+                vis[p] = fast_exp(power);
                 alpha[p] = fminf(0.99f, B.y * vis[p]);
-                valid[p] = idx <= bin_final[p] && !(sigma < 0.0f) && !(alpha[p] < kAlphaThreshold);
+                valid[p] = idx <= bin_final[p] && !(power > 0.0f) && !(alpha[p] < kAlphaThreshold);
                 any = any || valid[p];
             }
             if(__ballot(any) == 0)
@@ -414,10 +436,12 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
                 }
             }
             g[5] = S0; // v_opacity
+            // the gradients are written with d = mean - pixel: dx = -dxf, and S1 changes sign
+            const float dx = -dxf;
             S0 *= -B.y;
-            S1 *= -B.y;
-            g[0] = A.z * dx * S0 + A.w * S1; // v_sigma (a dx + b dy)
-            g[1] = bdx * S0 + B.x * S1;      // v_sigma (b dx + c dy)
+            S1 *= B.y;
+            g[0] = A.z * dx * S0 + A.w * S1;     // v_sigma (a dx + b dy)
+            g[1] = A.w * dx * S0 + B.x * S1;     // v_sigma (b dx + c dy)
             g[2] = 0.5f * dx * dx * S0;
             g[3] = dx * S1;
             g[4] = -0.5f * B.y * S2;

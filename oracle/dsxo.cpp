@@ -505,12 +505,15 @@ inline void blend_pixel(int x, int y, int32_t start, int32_t end, const int32_t*
         const S alpha = raw < alpha_clamp ? raw : alpha_clamp;
         if(margin)
         {
-            mg = std::min(mg, rel_margin(raw, alpha_threshold));
             /* sign of power: distance from 0 relative to the size of its terms */
             const S pa = power >= 0 ? power : -power;
             const S t1 = ca * dx * dx, t2 = cc * dy * dy, t3 = cb * dx * dy;
             const S mag = S(0.5f) * ((t1 < 0 ? -t1 : t1) + (t2 < 0 ? -t2 : t2)) + (t3 < 0 ? -t3 : t3);
             mg = std::min(mg, mag > 0 ? pa / mag : S(0));
+            /* alpha against 1/255: a rounding difference in the exponent (contraction, term
+             * order) is an absolute error of a few mag * 2^-24 there, i.e. a relative one in alpha:
+             * the distance from the threshold is counted less a guard band of mag * 1e-6 */
+            mg = std::min(mg, rel_margin(raw, alpha_threshold) - mag * S(1e-6));
         }
         if(power >= 0 || alpha < alpha_threshold)
             continue;
@@ -648,10 +651,11 @@ extern "C" void dsxo_blend_bwd(const dsxo_settings* s, int64_t n, const int32_t*
                 const float vis = expf(-sigma);
                 const float raw = opac * vis;
                 const float alpha = fminf(0.99f, raw);
-                gm = std::min(gm, rel_margin(raw, 1.f / 255.f));
                 {
                     const float mag = 0.5f * (fabsf(ca * dx * dx) + fabsf(cc * dy * dy)) + fabsf(cb * dx * dy);
                     gm = std::min(gm, mag > 0 ? fabsf(sigma) / mag : 0.f);
+                    /* as in the forward: the exponent's rounding error scales with mag */
+                    gm = std::min(gm, rel_margin(raw, 1.f / 255.f) - mag * 1e-6f);
                 }
                 if(sigma < 0.f || alpha < 1.f / 255.f)
                     continue;
