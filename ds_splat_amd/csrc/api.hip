@@ -166,7 +166,7 @@ SortU32Layout sort_u32_layout(int64_t count, int key_bits)
     l.keys_alt = 0;
     l.values_alt = align((size_t)count * 4);
     l.sort = align(l.values_alt + (size_t)count * 4);
-    l.bytes = l.sort + sort32_workspace(count, key_bits, kDepthSortTile).bytes;
+    l.bytes = l.sort + sort32_workspace(count, key_bits, sort32_tile_keys(count)).bytes;
     return l;
 }
 } // namespace
@@ -355,7 +355,7 @@ extern "C" int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t heigh
         if(order && n > 0)
         {
             const OrderLayout o = order_layout(n);
-            const Sort32Workspace w = sort32_workspace(n, 32, kDepthSortTile);
+            const Sort32Workspace w = sort32_workspace(n, 32, sort32_tile_keys(n));
             *depth_sort_flag =
                 reinterpret_cast<const uint32_t*>(static_cast<const char*>(order) + o.sort + w.counters) + w.passes;
         }

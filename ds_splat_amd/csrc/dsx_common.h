@@ -117,10 +117,19 @@ constexpr int kBins32 = 1 << kBits32;
 constexpr int kDepthSortThreads = DSX_NSORT_THREADS;
 constexpr int kDepthSortItems = DSX_NSORT_ITEMS;
 constexpr int kDepthSortTile = kDepthSortThreads * kDepthSortItems;
+// From this many keys on, the sort of (uint32 key, uint32 value) pairs uses the partition's
+// larger tiles too: its passes are bound by the chained scan over the tiles (all of them are
+// resident at once), which is shorter with fewer tiles (3 M keys: 0.028 -> 0.024 ms per pass);
+// smaller inputs keep the small tiles so that the launch still covers the chip.
+constexpr int64_t kLargeTileSortFrom = 1500000;
 constexpr int kListSortThreads = DSX_KSORT_THREADS;
 constexpr int kListSortItems = DSX_KSORT_ITEMS;
 constexpr int kListSortTile = kListSortThreads * kListSortItems;
 constexpr int kMaxPasses32 = 4;
+inline int sort32_tile_keys(int64_t count)
+{
+    return count >= kLargeTileSortFrom ? kListSortTile : kDepthSortTile;
+}
 // depth key of a Gaussian that emits no (tile, Gaussian) pair; as a float it is a NaN, which no
 // emitting Gaussian has (a NaN depth fails the frustum test)
 constexpr uint32_t kNoPairsKey = 0xffffffffu;

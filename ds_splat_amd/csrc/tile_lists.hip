@@ -508,10 +508,10 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
         return DSX_OK;
     if(count >= (1ll << 30))
         return DSX_ERR_TOO_LARGE;
-    int rc = already_cleared ? DSX_OK : sort32_clear(count, key_bits, kDepthSortTile, sort_ws, stream);
+    int rc = already_cleared ? DSX_OK : sort32_clear(count, key_bits, sort32_tile_keys(count), sort_ws, stream);
     if(rc)
         return rc;
-    const Sort32Workspace w = sort32_workspace(count, key_bits, kDepthSortTile);
+    const Sort32Workspace w = sort32_workspace(count, key_bits, sort32_tile_keys(count));
     const int64_t chunks = (count + kHist32Threads * kHist32Items - 1) / (kHist32Threads * kHist32Items);
     {
         DSX_TIMED("hist32_kernel", stream);
@@ -520,8 +520,15 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
                            reinterpret_cast<uint32_t*>(static_cast<char*>(sort_ws) + w.hist));
     }
     DSX_LAUNCH_CHECK();
-    return sort32_passes<uint32_t, kDepthSortThreads, kDepthSortItems>(count, key_bits, keys_a, vals_a, keys_b, vals_b, iota_values, keep_keys, sort_ws,
-                                   "onesweep32_kernel<sort>", stream, keys_out, vals_out, gather_src, gather_dst);
+    if(sort32_tile_keys(count) == kListSortTile)
+        return sort32_passes<uint32_t, kListSortThreads, kListSortItems>(count, key_bits, keys_a, vals_a, keys_b, vals_b,
+                                                                         iota_values, keep_keys, sort_ws,
+                                                                         "onesweep32_kernel<sort>", stream, keys_out,
+                                                                         vals_out, gather_src, gather_dst);
+    return sort32_passes<uint32_t, kDepthSortThreads, kDepthSortItems>(count, key_bits, keys_a, vals_a, keys_b, vals_b,
+                                                                       iota_values, keep_keys, sort_ws,
+                                                                       "onesweep32_kernel<sort>", stream, keys_out,
+                                                                       vals_out, gather_src, gather_dst);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -550,7 +557,7 @@ OrderLayout order_layout(int64_t n, int image_width, int image_height)
     o.slot_hist = off;
     off = align(off + (size_t)kMaxPasses32 * kBins32 * 4);
     o.sort = off;
-    off = align(off + sort32_workspace(n, 32, kDepthSortTile).bytes);
+    off = align(off + sort32_workspace(n, 32, sort32_tile_keys(n)).bytes);
     o.cover = off;
     off = align(off + (size_t)((tiles_x(image_width) + 1) * (tiles_y(image_height) + 1) + 1) * 4);
     o.ranges = off;
@@ -774,7 +781,7 @@ void depth_order_clear_region(const dsx_camera& cam, int64_t n, void* order, uin
 {
     // the sort's histograms, counters and look-back statuses and, right behind them, the corner grid
     const OrderLayout o = order_layout(n, cam.image_width, cam.image_height);
-    const Sort32Workspace w = sort32_workspace(n, 32, kDepthSortTile);
+    const Sort32Workspace w = sort32_workspace(n, 32, sort32_tile_keys(n));
     *words = reinterpret_cast<uint32_t*>(static_cast<char*>(order) + o.sort + w.hist);
     *count = (int64_t)((w.bytes + (o.ranges - o.cover)) / 4);
 }

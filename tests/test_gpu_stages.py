@@ -217,7 +217,8 @@ def test_sort_pairs_vs_oracle_on_emitted_keys(oracle):
 # ------------------------------------------------------------------------------- stages 2+3, fast route
 @pytest.mark.parametrize("count,key_bits,ties", [(2, 32, False), (1000, 32, False), (8192, 8, True), (8193, 13, False),
                                                  (70_000, 15, True), (1_000_003, 32, False), (300_001, 32, True),
-                                                 (200_000, 1, True), (123_457, 17, False)])
+                                                 (200_000, 1, True), (123_457, 17, False),
+                                                 (1_500_000, 32, False), (2_345_679, 24, True)])  # large-tile plan
 def test_sort_pairs_u32_matches_stable_sort(count, key_bits, ties):
     """Stable ascending unsigned sort of keys that use their low key_bits bits."""
     st_ = _stages()
