@@ -899,8 +899,9 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
 }
 
 // ---------------------------------------------------------------------------------------
-// emission in depth order: one workgroup per 256 Gaussians of the depth order, one thread per
-// OUTPUT pair, so stores are contiguous however uneven the per-Gaussian tile counts are
+// emission in depth order: a workgroup owns a range of OUTPUT pairs and walks the blocks of 256
+// depth-ordered Gaussians that reach into it; one thread per output pair, so the work per
+// workgroup is bounded and the stores are contiguous however uneven the tile counts are
 // ---------------------------------------------------------------------------------------
 
 #ifndef DSX_EMIT_WINDOWS
