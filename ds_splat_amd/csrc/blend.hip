@@ -3,6 +3,8 @@
 // one float array, so an entry costs two 128-bit and one 32-bit LDS broadcast read.
 #include "dsx_common.h"
 
+#include <cstdlib>
+
 namespace dsx
 {
 
@@ -53,11 +55,12 @@ __device__ __forceinline__ float edge_min(float a, float b, float c, float u, fl
     return 0.5f * (a * u * u + c * v * v) + b * u * v;
 }
 
+// (span_y: last row of pixel centres of the box, 15 for a whole tile, 3 for a band of four rows)
 __device__ __forceinline__ bool entry_reaches_tile(float mx, float my, float a, float b, float c, float opacity,
-                                                   float box_x0, float box_y0)
+                                                   float box_x0, float box_y0, float span_y = 15.0f)
 {
     const float dx0 = box_x0 - mx, dx1 = box_x0 + 15.0f - mx;
-    const float dy0 = box_y0 - my, dy1 = box_y0 + 15.0f - my;
+    const float dy0 = box_y0 - my, dy1 = box_y0 + span_y - my;
     const bool inside = dx0 <= 0.0f && dx1 >= 0.0f && dy0 <= 0.0f && dy1 >= 0.0f;
     float qmin = fminf(fminf(edge_min(a, b, c, dx0, dy0, dy1), edge_min(a, b, c, dx1, dy0, dy1)),
                        fminf(edge_min(c, b, a, dy0, dx0, dx1), edge_min(c, b, a, dy1, dx0, dx1)));
@@ -67,6 +70,26 @@ __device__ __forceinline__ bool entry_reaches_tile(float mx, float my, float a, 
     return !(well_formed && qmin > limit);
 }
 
+// Pixels per lane of the blend kernels: 4 (one wavefront per tile) when the image has enough tiles
+// to occupy the chip (8 wavefronts on each of 1024 SIMDs), else 1 (four wavefronts per tile: more
+// instructions in all, but four times as many wavefronts).  Measured crossover (500 K Gaussians,
+// 640x480 to 1920x1080): about 5000 tiles for the forward, 1600 for the backward, whose
+// one-pixel form also quadruples the atomics.  DSX_BLEND_PIXELS_PER_LANE=1|4 in the environment
+// overrides the choice (tests run both forms).
+static int blend_pixels_per_lane(int num_tiles, int four_from)
+{
+    if(const char* forced = getenv("DSX_BLEND_PIXELS_PER_LANE"))
+    {
+        if(forced[0] == '1' && forced[1] == 0)
+            return 1;
+        if(forced[0] == '4' && forced[1] == 0)
+            return 4;
+    }
+    return num_tiles >= four_from ? 4 : 1;
+}
+constexpr int kFwdFourPixelsFrom = 5000; // tiles
+constexpr int kBwdFourPixelsFrom = 1600;
+
 // -----------------------------------------------------------------------------------------
 // forward: cpp/rasterizer_kernels.cu:341-431
 // -----------------------------------------------------------------------------------------
@@ -74,10 +97,13 @@ __device__ __forceinline__ bool entry_reaches_tile(float mx, float my, float a, 
 // (l >> 4) + {0, 4, 8, 12}).  Every LDS broadcast read of an entry then feeds 256 pixel
 // updates instead of 64, which moves the kernel from the LDS pipe to the VALU, gives each
 // lane four independent dependency chains, and needs no workgroup barrier at all.
+// Images of few tiles (fewer wavefronts than the chip has slots) take kFwdPix = 1 instead: four
+// wavefronts per tile, each with one band of four rows and one pixel per lane; a tile's walk is
+// then four times shorter in time, which is what counts when the launch cannot fill the chip.
 constexpr int kFwdBatch = 128; // sorted entries staged in LDS per round (two per lane)
-constexpr int kFwdPix = 4;
 
 // 8 wavefronts per SIMD (at most 64 VGPRs): all tiles of a 1080p image are resident at once
+template <int kFwdPix>
 __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))) void blend_fwd_kernel(const int32_t* __restrict__ ranges,
                                                              const int32_t* __restrict__ ids,
                                                              const float4* __restrict__ splats,
@@ -91,13 +117,16 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     __shared__ float s_c[kFwdBatch];  // blue
 
     const int lane = threadIdx.x;
-    const int tile = blockIdx.x;
+    const int tile = kFwdPix == 4 ? blockIdx.x : blockIdx.x >> 2;
+    const int band = kFwdPix == 4 ? 0 : blockIdx.x & 3; // which four rows of the tile (one-pixel form)
     const int tx = tile % ntx;
     const int ty = tile / ntx;
     const int x = tx * kTile + (lane & 15);
-    const int y0 = ty * kTile + (lane >> 4);
+    const int y0 = ty * kTile + 4 * band + (lane >> 4);
     const float pxf = (float)x + 0.5f;
-    const float box_x0 = (float)(tx * kTile) + 0.5f, box_y0 = (float)(ty * kTile) + 0.5f; // first pixel centre
+    // first pixel centre and last row of the pixels this wavefront owns
+    const float box_x0 = (float)(tx * kTile) + 0.5f, box_y0 = (float)(ty * kTile + 4 * band) + 0.5f;
+    const float span_y = kFwdPix == 4 ? 15.0f : 3.0f;
 
     const int start = ranges[tile];
     const int end = ranges[tile + 1];
@@ -140,7 +169,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                 s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
                 s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
-                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0);
+                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
             }
             todo[h] = __ballot(useful);
         }
@@ -215,9 +244,14 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
         return DSX_OK;
     {
         DSX_TIMED("blend_fwd_kernel", stream);
-        hipLaunchKernelGGL(blend_fwd_kernel, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
-                           reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                           cam.image_height, ntx, sort_flag_a, sort_flag_b);
+        if(blend_pixels_per_lane(ntx * nty, kFwdFourPixelsFrom) == 4)
+            hipLaunchKernelGGL(blend_fwd_kernel<4>, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
+                               reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
+                               cam.image_height, ntx, sort_flag_a, sort_flag_b);
+        else
+            hipLaunchKernelGGL(blend_fwd_kernel<1>, dim3(4 * ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
+                               reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
+                               cam.image_height, ntx, sort_flag_a, sort_flag_b);
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
@@ -297,13 +331,14 @@ __device__ __forceinline__ float wave_sum8_scatter(const float (&v)[8], int lane
 }
 
 constexpr int kBwdBatch = 128; // sorted entries staged in LDS per round (two per lane)
-constexpr int kBwdPix = 4;
 
 // One wavefront per 16x16 tile, four pixels per lane (same pixel ownership as the forward).
 // The per-Gaussian gradients are first summed over a lane's four pixels, then over the
 // wavefront with DPP adds, and lane 63 issues ONE set of hardware float atomics per
 // (tile, entry).  Compared with four wavefronts of one pixel per lane this does one
 // cross-lane reduction per entry instead of four and needs no LDS accumulators or barriers.
+// (kBwdPix = 1: four wavefronts per tile with one band of four rows each, as in the forward)
+template <int kBwdPix>
 __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const int32_t* __restrict__ ranges, const int32_t* __restrict__ ids, const float4* __restrict__ splats,
     const float* __restrict__ final_T, const int32_t* __restrict__ final_idx, const float* __restrict__ v_image,
@@ -315,13 +350,16 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     __shared__ int s_id[kBwdBatch];
 
     const int lane = threadIdx.x;
-    const int tile = blockIdx.x;
+    const int tile = kBwdPix == 4 ? blockIdx.x : blockIdx.x >> 2;
+    const int band = kBwdPix == 4 ? 0 : blockIdx.x & 3;
     const int tx = tile % ntx;
     const int ty = tile / ntx;
     const int x = tx * kTile + (lane & 15);
-    const int y0 = ty * kTile + (lane >> 4);
+    const int y0 = ty * kTile + 4 * band + (lane >> 4);
     const float pxf = (float)x + 0.5f;
-    const float box_x0 = (float)(tx * kTile) + 0.5f, box_y0 = (float)(ty * kTile) + 0.5f; // first pixel centre
+    // first pixel centre and last row of the pixels this wavefront owns
+    const float box_x0 = (float)(tx * kTile) + 0.5f, box_y0 = (float)(ty * kTile + 4 * band) + 0.5f;
+    const float span_y = kBwdPix == 4 ? 15.0f : 3.0f;
     const float bg0 = bg[0], bg1 = bg[1], bg2 = bg[2];
 
     // bterm = -T_final * (bg . v_out) - sum over the entries behind of (rgb . v_out) * alpha * T:
@@ -375,7 +413,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
                 s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
                 s_id[slot] = g;
-                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0);
+                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
             }
             todo[h] = __ballot(useful);
         }
@@ -471,9 +509,14 @@ int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, co
         return DSX_OK;
     {
         DSX_TIMED("blend_bwd_kernel", stream);
-        hipLaunchKernelGGL(blend_bwd_kernel, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
-                           reinterpret_cast<const float4*>(splats), final_T, final_idx, v_image, cam.bg, grads,
-                           cam.image_width, cam.image_height, ntx);
+        if(blend_pixels_per_lane(ntx * nty, kBwdFourPixelsFrom) == 4)
+            hipLaunchKernelGGL(blend_bwd_kernel<4>, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
+                               reinterpret_cast<const float4*>(splats), final_T, final_idx, v_image, cam.bg, grads,
+                               cam.image_width, cam.image_height, ntx);
+        else
+            hipLaunchKernelGGL(blend_bwd_kernel<1>, dim3(4 * ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
+                               reinterpret_cast<const float4*>(splats), final_T, final_idx, v_image, cam.bg, grads,
+                               cam.image_width, cam.image_height, ntx);
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;

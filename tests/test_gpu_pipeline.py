@@ -70,7 +70,10 @@ def check_grads(leaves, B, ok):
     ("cfg4", 3000, 320, 180, 3, 0.5, None),             # heavy-overlap distributions, reduced size
     ("cfg2", 30000, 333, 177, 2, 1.5, None),            # ragged image (not a multiple of 16)
 ])
-def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, bg):
+@pytest.mark.parametrize("pixels_per_lane", ["1", "4"])
+def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, bg, pixels_per_lane, monkeypatch):
+    # both forms of the blend kernels, whatever the image size would pick
+    monkeypatch.setenv("DSX_BLEND_PIXELS_PER_LANE", pixels_per_lane)
     sc = make_scene(name, n=n, width=W, height=H, sh_degree=deg)
     image, radii, leaves = api_run(sc, scale_mul, bg=bg)
     img_o, radii_o, S, B = oracle_run(oracle, sc, scale_mul, bg=bg)

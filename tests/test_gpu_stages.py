@@ -337,7 +337,11 @@ def test_tile_ranges_vs_oracle(oracle, k, num_tiles, neg):
 
 # ------------------------------------------------------------------------------- stage 4
 @pytest.mark.parametrize("n,W,H,scale_mul", [(20000, 256, 256, 2.0), (4000, 200, 120, 6.0), (300, 33, 17, 4.0)])
-def test_blend_fwd_vs_oracle(oracle, n, W, H, scale_mul):
+@pytest.mark.parametrize("pixels_per_lane", ["1", "4"])
+def test_blend_fwd_vs_oracle(oracle, n, W, H, scale_mul, pixels_per_lane, monkeypatch):
+    # both forms of the kernel (four wavefronts per tile with one pixel per lane, one wavefront with
+    # four) whatever the image size would pick
+    monkeypatch.setenv("DSX_BLEND_PIXELS_PER_LANE", pixels_per_lane)
     st_ = _stages()
     sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=31 + n, scale_mul=scale_mul)
     oracle.free(st)
@@ -353,9 +357,11 @@ def test_blend_fwd_vs_oracle(oracle, n, W, H, scale_mul):
 
 
 # ------------------------------------------------------------------------------- stage 5a
+@pytest.mark.parametrize("pixels_per_lane", ["1", "4"])
 @pytest.mark.parametrize("n,W,H,scale_mul,bg", [(20000, 256, 256, 2.0, (0, 0, 0)), (4000, 200, 120, 6.0, (0.3, 0.6, 0.1)),
                                                 (300, 33, 17, 4.0, (1, 1, 1))])
-def test_blend_bwd_vs_oracle(oracle, n, W, H, scale_mul, bg):
+def test_blend_bwd_vs_oracle(oracle, n, W, H, scale_mul, bg, pixels_per_lane, monkeypatch):
+    monkeypatch.setenv("DSX_BLEND_PIXELS_PER_LANE", pixels_per_lane)
     st_ = _stages()
     sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=41 + n, scale_mul=scale_mul)
     oracle.free(st)
