@@ -21,7 +21,7 @@ std::mutex g_trace_mutex;
 std::vector<TraceSlot> g_trace;
 } // namespace
 
-dsx::KernelTimer::KernelTimer(const char* name, hipStream_t s) : slot(-1), stream(s)
+dsx::KernelTimer::KernelTimer(const char* name, hipStream_t s) : slot(-1), stream(s), stop(nullptr)
 {
     if(!g_trace_on)
         return;
@@ -37,6 +37,7 @@ dsx::KernelTimer::KernelTimer(const char* name, hipStream_t s) : slot(-1), strea
     (void)hipEventRecord(t.start, s);
     std::lock_guard<std::mutex> lock(g_trace_mutex);
     slot = (int)g_trace.size();
+    stop = t.stop;
     g_trace.push_back(t);
 }
 
@@ -45,7 +46,9 @@ dsx::KernelTimer::~KernelTimer()
     if(slot < 0)
         return;
     std::lock_guard<std::mutex> lock(g_trace_mutex);
-    (void)hipEventRecord(g_trace[slot].stop, stream);
+    // a dsx_trace_read from another thread may have emptied the list since the constructor ran
+    if((size_t)slot < g_trace.size() && g_trace[slot].stop == stop)
+        (void)hipEventRecord(stop, stream);
 }
 
 extern "C" int dsx_trace_enable(int on)

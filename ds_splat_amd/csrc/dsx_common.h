@@ -266,6 +266,7 @@ struct KernelTimer
     ~KernelTimer();
     int slot;
     hipStream_t stream;
+    hipEvent_t stop;
 };
 #define DSX_TIMED(name, stream) dsx::KernelTimer dsx_timer_##__LINE__(name, stream)
 
