@@ -34,9 +34,9 @@ BWD_PAIR_FLOPS, BWD_REJECT_FLOPS = 72, 15
 # the figures are quoted here and only reported when workload and key count are the profiled ones.
 MEASURED_TRAFFIC = {
     ("cfg2", 32604809): {
-        "project_fwd_kernel": 930.6e6, "hist32_kernel": 13.8e6, "onesweep32_kernel<sort>": 103.7e6,
+        "project_fwd_kernel": 930.9e6, "hist32_kernel": 13.3e6, "onesweep32_kernel<sort>": 103.6e6,
         "ordered_block_sums_kernel": 24.4e6, "emit_ordered_kernel": 248.5e6,
-        "onesweep32_kernel<tile partition>": 376.3e6, "gaussian_bwd_kernel": 1333.2e6,
+        "onesweep32_kernel<tile partition>": 376.7e6, "gaussian_bwd_kernel": 1225.2e6,
         "blend_fwd_kernel": 78.5e6, "blend_bwd_kernel": 156.1e6,
     },
 }
@@ -49,7 +49,9 @@ def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, counters):
         # inputs 44 + 12c bytes, outputs radii + cov3d + splat record + depth key + tile rectangle
         return "hbm", n * (44 + 12 * coeffs + 4 + 24 + 48 + 4 + 8), "B"
     if kernel == "gaussian_bwd_kernel":
-        return "hbm", n * (112 + 76 + 12 * coeffs), "B"
+        # reads 112; writes v_mean3d 12 + v_means2d 12 + v_scale 12 + v_quat 16 + v_shs 12c (v_colors and
+        # v_cov3d are not written: the step gives neither colours nor covariances, so nothing takes them)
+        return "hbm", n * (112 + 52 + 12 * coeffs), "B"
     if kernel == "hist32_kernel":
         return "hbm", 4 * n, "B"
     if kernel == "onesweep32_kernel<sort>":                  # depth sort of the Gaussians: key + id, in and out

@@ -435,9 +435,8 @@ extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_ba
         return DSX_ERR_BAD_ARG;
     if(n == 0)
         return DSX_OK;
-    if(!means3d || !splats || !cov3d || !radii || !grads || !v_mean3d || !v_means2d || !v_colors || !v_opacity ||
-       !v_scale || !v_quat || !v_cov3d)
-        return DSX_ERR_BAD_ARG;
+    if(!means3d || !splats || !cov3d || !radii || !grads)
+        return DSX_ERR_BAD_ARG; // any of the outputs may be null: that gradient is not wanted
     if((scales == nullptr) != (quats == nullptr))
         return DSX_ERR_BAD_ARG;
     return launch_gaussian_bwd(*cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,

@@ -101,13 +101,21 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
         mean = make_float3(p.means3d[3 * i], p.means3d[3 * i + 1], p.means3d[3 * i + 2]);
 
         // straight copies: screen-space mean gradient (z column zero), colour and opacity
-        p.v_means2d[3 * i] = v_x;
-        p.v_means2d[3 * i + 1] = v_y;
-        p.v_means2d[3 * i + 2] = 0.f;
-        p.v_colors[3 * i] = v_rgb[0];
-        p.v_colors[3 * i + 1] = v_rgb[1];
-        p.v_colors[3 * i + 2] = v_rgb[2];
-        p.v_opacity[i] = v_o;
+        // (every output is optional: a null pointer means that the caller has no use for it)
+        if(p.v_means2d)
+        {
+            p.v_means2d[3 * i] = v_x;
+            p.v_means2d[3 * i + 1] = v_y;
+            p.v_means2d[3 * i + 2] = 0.f;
+        }
+        if(p.v_colors)
+        {
+            p.v_colors[3 * i] = v_rgb[0];
+            p.v_colors[3 * i + 1] = v_rgb[1];
+            p.v_colors[3 * i + 2] = v_rgb[2];
+        }
+        if(p.v_opacity)
+            p.v_opacity[i] = v_o;
 
         float vm[3] = {0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f};
         float vc3[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -250,17 +258,23 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
                                2.f * z * (vR[0][0] + vR[1][1]) + w * (vR[1][0] - vR[0][1]));
             }
         }
+        if(p.v_mean3d)
 #pragma unroll
-        for(int c = 0; c < 3; ++c)
+            for(int c = 0; c < 3; ++c)
+                p.v_mean3d[3 * i + c] = vm[c];
+        if(p.v_scale)
+#pragma unroll
+            for(int c = 0; c < 3; ++c)
+                p.v_scale[3 * i + c] = vs[c];
+        if(p.v_quat)
+            reinterpret_cast<float4*>(p.v_quat)[i] = make_float4(vq[0], vq[1], vq[2], vq[3]);
+        if(p.v_cov3d)
         {
-            p.v_mean3d[3 * i + c] = vm[c];
-            p.v_scale[3 * i + c] = vs[c];
+            float2* o = reinterpret_cast<float2*>(p.v_cov3d + 6 * i);
+            o[0] = make_float2(vc3[0], vc3[1]);
+            o[1] = make_float2(vc3[2], vc3[3]);
+            o[2] = make_float2(vc3[4], vc3[5]);
         }
-        reinterpret_cast<float4*>(p.v_quat)[i] = make_float4(vq[0], vq[1], vq[2], vq[3]);
-        float2* o = reinterpret_cast<float2*>(p.v_cov3d + 6 * i);
-        o[0] = make_float2(vc3[0], vc3[1]);
-        o[1] = make_float2(vc3[2], vc3[3]);
-        o[2] = make_float2(vc3[4], vc3[5]);
     }
 
     // ---- v_shs[b][c] = Y_b(dir) * v_rgb[c], zero above the active degree -------------------

@@ -116,7 +116,8 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
 }
 
 // v_mean3d[N,3], v_means2d[N,3], v_shs[N,B,3] (undefined when num_bases == 0), v_colors[N,3],
-// v_opacity[N,1], v_scale[N,3], v_quat[N,4], v_cov3d[N,6]
+// v_opacity[N,1], v_scale[N,3], v_quat[N,4], v_cov3d[N,6].  Bit i of `wanted` asks for the i-th
+// of them; the others are neither allocated nor written and come back undefined (None).
 std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
                                  int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view,
                                  const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
@@ -124,7 +125,7 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
                                  const c10::optional<at::Tensor>& quats, const at::Tensor& splats,
                                  const at::Tensor& cov3d, const at::Tensor& radii, const at::Tensor& ranges,
                                  const at::Tensor& sorted_ids, const at::Tensor& final_T, const at::Tensor& final_idx,
-                                 const at::Tensor& v_image, int64_t stream)
+                                 const at::Tensor& v_image, int64_t wanted, int64_t stream)
 {
     const at::Device dev = means3d.device();
     c10::DeviceGuard guard(dev);
@@ -134,19 +135,23 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
     const auto f32 = at::TensorOptions().dtype(at::kFloat).device(dev);
     TORCH_CHECK(v_image.is_contiguous() && v_image.scalar_type() == at::kFloat && v_image.numel() == height * width * 3,
                 "v_image must be a contiguous float32 [H, W, 3] tensor");
-    at::Tensor v_mean3d = at::empty({n, 3}, f32), v_means2d = at::empty({n, 3}, f32);
+    auto out = [&](int bit, std::initializer_list<int64_t> shape) {
+        return (wanted >> bit) & 1 ? at::empty(shape, f32) : at::Tensor();
+    };
+    auto ptr = [](const at::Tensor& t) { return t.defined() ? t.data_ptr<float>() : nullptr; };
+    if(num_bases <= 0 || !((wanted >> 2) & 1))
+        num_bases = 0;
+    at::Tensor v_mean3d = out(0, {n, 3}), v_means2d = out(1, {n, 3});
     at::Tensor v_shs = num_bases > 0 ? at::empty({n, num_bases, 3}, f32) : at::Tensor();
-    at::Tensor v_colors = at::empty({n, 3}, f32), v_opacity = at::empty({n, 1}, f32);
-    at::Tensor v_scale = at::empty({n, 3}, f32), v_quat = at::empty({n, 4}, f32), v_cov3d = at::empty({n, 6}, f32);
+    at::Tensor v_colors = out(3, {n, 3}), v_opacity = out(4, {n, 1});
+    at::Tensor v_scale = out(5, {n, 3}), v_quat = out(6, {n, 4}), v_cov3d = out(7, {n, 6});
     at::Tensor grads = at::empty({n, DSX_GRAD_FLOATS}, f32);
     check(dsx_backward(&cam.c, n, (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
                        splats.data_ptr<float>(), cov3d.data_ptr<float>(), radii.data_ptr<int32_t>(),
                        ranges.data_ptr<int32_t>(), sorted_ids.numel() ? sorted_ids.data_ptr<int32_t>() : nullptr,
                        final_T.data_ptr<float>(), final_idx.data_ptr<int32_t>(), v_image.data_ptr<float>(),
-                       grads.data_ptr<float>(), v_mean3d.data_ptr<float>(), v_means2d.data_ptr<float>(),
-                       num_bases > 0 ? v_shs.data_ptr<float>() : nullptr, v_colors.data_ptr<float>(),
-                       v_opacity.data_ptr<float>(), v_scale.data_ptr<float>(), v_quat.data_ptr<float>(),
-                       v_cov3d.data_ptr<float>(), reinterpret_cast<void*>(stream)));
+                       grads.data_ptr<float>(), ptr(v_mean3d), ptr(v_means2d), ptr(v_shs), ptr(v_colors),
+                       ptr(v_opacity), ptr(v_scale), ptr(v_quat), ptr(v_cov3d), reinterpret_cast<void*>(stream)));
     return {v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d};
 }
 

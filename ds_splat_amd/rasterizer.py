@@ -116,15 +116,18 @@ class DsRasterizerFunction(torch.autograd.Function):
         ext = _native.load_torch_ext()
         opt = lambda t: t if t.numel() > 0 else None
         stream = torch.cuda.current_stream(means_3d.device).cuda_stream
+        # the reference computes all eight gradients and autograd drops those of inputs that take
+        # none (cpp/rasterizer_torch.cu:315, ds_splat/rasterizer.py:112); here the kernel is told
+        # which ones are wanted and writes no others (v_colors and v_cov3d in the usual training
+        # set-up with SH colours, scales and rotations: 36 of 320 bytes per Gaussian)
+        needs = ctx.needs_input_grad
+        wanted = sum(1 << i for i in range(8) if needs[i])
         v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d = ext.backward(
             *ctx.cam, ctx.num_bases, means_3d, opt(scales), opt(rotations), splats, cov3d, radii, ranges, sorted_ids,
-            final_T, final_idx, rendered_img_grad.contiguous(), stream)
-        if tuple(ctx.opacity_shape) != tuple(v_opacity.shape):
+            final_T, final_idx, rendered_img_grad.contiguous(), wanted, stream)
+        if v_opacity is not None and tuple(ctx.opacity_shape) != tuple(v_opacity.shape):
             v_opacity = v_opacity.reshape(ctx.opacity_shape)
-        needs = ctx.needs_input_grad
-        pick = lambda i, t: t if needs[i] else None
-        return (pick(0, v_mean3d), pick(1, v_means2d), pick(2, v_shs), pick(3, v_colors), pick(4, v_opacity),
-                pick(5, v_scale), pick(6, v_quat), pick(7, v_cov3d), None)
+        return (v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, None)
 
 
 @dataclass

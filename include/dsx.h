@@ -185,6 +185,9 @@ int dsx_blend_bwd(const dsx_camera* cam, int64_t n, const int32_t* ranges,
  * rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:291-313.
  * Outputs: v_mean3d[n*3], v_means2d[n*3] (xy gradient in pixels, z = 0), v_shs[n*num_bases*3]
  * (may be NULL), v_colors[n*3], v_opacity[n], v_scale[n*3], v_quat[n*4], v_cov3d[n*6].
+ * Any output may be NULL: that gradient is then not written (the reference computes all of them
+ * and lets autograd drop those of inputs that were not given, cpp/rasterizer_torch.cu:315;
+ * here an unwanted one costs no store).
  * scales/quats may be NULL when the forward used cov3d_precomp (v_scale, v_quat zeroed). */
 int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                      const float* scales, const float* quats, const float* splats,

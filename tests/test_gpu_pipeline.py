@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def api_run(sc, scale_mul=1.0, backward=True, bg=None, opac_shape=None, colors=None, cov3d=None):
+def api_run(sc, scale_mul=1.0, backward=True, bg=None, opac_shape=None, colors=None, cov3d=None, wants=None):
     from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
     settings = GaussianRasterizationSettings(
@@ -23,8 +23,8 @@ def api_run(sc, scale_mul=1.0, backward=True, bg=None, opac_shape=None, colors=N
     leaves = dict(means=t["means_3d"].clone(), means2d=torch.zeros_like(t["means_3d"]), shs=t["shs"].clone(),
                   opac=opac.clone(), scales=(t["scales"] * scale_mul).clone(), rots=t["rotations"].clone())
     if backward:
-        for v in leaves.values():
-            v.requires_grad_(True)
+        for k, v in leaves.items():
+            v.requires_grad_(wants is None or k in wants)
     r = GaussianRasterizer(settings)
     if colors is not None:
         image, radii = r(leaves["means"], leaves["means2d"], None, colors, leaves["opac"], leaves["scales"],
@@ -136,6 +136,22 @@ def test_api_on_a_side_stream_matches_the_default_stream():
     for k in leaves0:
         a, b = leaves0[k].grad, leaves1[k].grad
         assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * max(1.0, float(a.abs().max())))
+
+
+def test_only_the_gradients_asked_for_are_produced():
+    """Inputs that take no gradient get none, and the others get what they get when every input
+    takes one (the kernel skips the stores of unwanted outputs, nothing else changes)."""
+    sc = make_scene("cfg1", n=20000, width=320, height=200, sh_degree=3)
+    _, _, full = api_run(sc, 2.0)
+    for wants in (("shs", "opac"), ("means", "scales", "rots"), ("means2d",)):
+        _, _, part = api_run(sc, 2.0, wants=wants)
+        for k in full:
+            if k not in wants:
+                assert part[k].grad is None, k
+                continue
+            a, b = full[k].grad, part[k].grad
+            assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * max(1.0, float(a.abs().max()))), k
+            assert float(b.abs().max()) > 0 or k == "means2d"
 
 
 def test_inria_adaptor_composites_the_background_and_keeps_the_gradients():
