@@ -46,12 +46,13 @@ def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, counters):
     """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch."""
     slot_bytes = 2 if tiles + 1 <= 65535 else 4
     if kernel == "project_fwd_kernel":
-        # inputs 44 + 12c bytes, outputs radii + cov3d + splat record + depth key + tile rectangle
-        return "hbm", n * (44 + 12 * coeffs + 4 + 24 + 48 + 4 + 8), "B"
+        # inputs 44 + 12c bytes, outputs radii + splat record + depth key + tile rectangle (the 3-D
+        # covariance is not stored on this path: the backward rebuilds it)
+        return "hbm", n * (44 + 12 * coeffs + 4 + 48 + 4 + 8), "B"
     if kernel == "gaussian_bwd_kernel":
-        # reads 112; writes v_mean3d 12 + v_means2d 12 + v_scale 12 + v_quat 16 + v_shs 12c (v_colors and
-        # v_cov3d are not written: the step gives neither colours nor covariances, so nothing takes them)
-        return "hbm", n * (112 + 52 + 12 * coeffs), "B"
+        # reads 88 (no stored covariance); writes v_mean3d 12 + v_means2d 12 + v_scale 12 + v_quat 16 + v_shs 12c
+        # (v_colors and v_cov3d are not written: the step gives neither colours nor covariances, so nothing takes them)
+        return "hbm", n * (88 + 52 + 12 * coeffs), "B"
     if kernel == "hist32_kernel":
         return "hbm", 4 * n, "B"
     if kernel == "onesweep32_kernel<sort>":                  # depth sort of the Gaussians: key + id, in and out

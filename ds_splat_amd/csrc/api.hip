@@ -192,8 +192,8 @@ static int project_fwd_checked(const dsx_camera* cam, int64_t n, const float* me
         return DSX_ERR_BAD_ARG;
     if(n == 0)
         return DSX_OK;
-    if(!means3d || !opacities || !splats || !radii || !cov3d || !block_sums)
-        return DSX_ERR_BAD_ARG;
+    if(!means3d || !opacities || !splats || !radii || !block_sums)
+        return DSX_ERR_BAD_ARG; // cov3d may be null: not stored
     uint32_t* depth_keys = nullptr;
     uint2* rects = nullptr;
     if(order)
@@ -435,10 +435,12 @@ extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_ba
         return DSX_ERR_BAD_ARG;
     if(n == 0)
         return DSX_OK;
-    if(!means3d || !splats || !cov3d || !radii || !grads)
+    if(!means3d || !splats || !radii || !grads)
         return DSX_ERR_BAD_ARG; // any of the outputs may be null: that gradient is not wanted
     if((scales == nullptr) != (quats == nullptr))
         return DSX_ERR_BAD_ARG;
+    if(!cov3d && !scales)
+        return DSX_ERR_BAD_ARG; // without the stored covariance the kernel rebuilds it from scale and rotation
     return launch_gaussian_bwd(*cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
                                v_means2d, num_bases > 0 ? v_shs : nullptr, v_colors, v_opacity, v_scale, v_quat,
                                v_cov3d, as_stream(stream));
@@ -484,7 +486,7 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
 extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
                                   const void* order, int32_t* sorted_ids, int32_t* ranges, float* image,
                                   float* final_T, int32_t* final_idx, void* workspace, size_t workspace_bytes,
-                                  void* stream)
+                                  float* grads_to_zero, void* stream)
 {
     if(!image || !final_T || !final_idx)
         return DSX_ERR_BAD_ARG;
@@ -496,17 +498,26 @@ extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, c
     if(rc)
         return rc;
     return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream), depth_flag,
-                            partition_flag);
+                            partition_flag, grads_to_zero, n * DSX_GRAD_FLOATS);
 }
 
 extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                             const float* scales, const float* quats, const float* splats, const float* cov3d,
                             const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
                             const float* final_T, const int32_t* final_idx, const float* v_image, float* grads,
-                            float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors, float* v_opacity,
-                            float* v_scale, float* v_quat, float* v_cov3d, void* stream)
+                            int32_t grads_are_zero, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
+                            float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, void* stream)
 {
-    int rc = dsx_blend_bwd(cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads, stream);
+    if(int rc = check_camera(cam))
+        return rc;
+    if(n < 0)
+        return DSX_ERR_BAD_ARG;
+    if(n == 0)
+        return DSX_OK;
+    if(!ranges || !final_T || !final_idx || !v_image || !grads || !splats)
+        return DSX_ERR_BAD_ARG;
+    int rc = launch_blend_bwd(*cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
+                              as_stream(stream), grads_are_zero != 0);
     if(rc)
         return rc;
     return dsx_gaussian_bwd(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
@@ -572,7 +583,7 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
                                     reinterpret_cast<int32_t*>(buf2 + o_ids),
                                     reinterpret_cast<int32_t*>(buf + o_ranges), image,
                                     reinterpret_cast<float*>(buf + o_T), reinterpret_cast<int32_t*>(buf + o_idx),
-                                    buf2, ws, stream);
+                                    buf2, ws, nullptr, stream);
     }
     if(buf2)
         (void)hipFreeAsync(buf2, s);

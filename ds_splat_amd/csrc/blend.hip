@@ -110,7 +110,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                                                              float* __restrict__ image, float* __restrict__ final_T,
                                                              int32_t* __restrict__ final_idx, int W, int H, int ntx,
                                                              const uint32_t* __restrict__ sort_flag_a,
-                                                             const uint32_t* __restrict__ sort_flag_b)
+                                                             const uint32_t* __restrict__ sort_flag_b,
+                                                             float4* __restrict__ zero, int64_t zero_vecs)
 {
     __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic a, conic b
     __shared__ float4 s_b[kFwdBatch]; // conic c, opacity, red, green
@@ -233,25 +234,48 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             final_idx[pix] = last[p];
         }
     }
+    // A side job for the memory system, which this kernel leaves idle: every wavefront zeroes its
+    // share of a buffer that the caller needs cleared (the backward's gradient accumulator).  At
+    // the end, where nothing waits for the stores and the wavefronts arrive spread over time (at
+    // the start they would all come at once and hold up the first loads: 0.147 against 0.140 ms).
+    if(zero_vecs > 0)
+    {
+        const int64_t share = (zero_vecs + gridDim.x - 1) / gridDim.x;
+        const int64_t z0 = (int64_t)blockIdx.x * share;
+        const int64_t z1 = min(z0 + share, zero_vecs);
+        for(int64_t j = z0 + lane; j < z1; j += DSX_WAVE)
+            zero[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
 }
 
 int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids, const float* splats,
                      float* image, float* final_T, int32_t* final_idx, hipStream_t stream,
-                     const uint32_t* sort_flag_a, const uint32_t* sort_flag_b)
+                     const uint32_t* sort_flag_a, const uint32_t* sort_flag_b, float* zero, int64_t zero_floats)
 {
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
+    if(zero == nullptr)
+        zero_floats = 0;
+    // the kernel zeroes in 16-byte units; anything else (or no kernel at all) takes the plain fill
+    if(zero_floats > 0 && (ntx * nty == 0 || (zero_floats & 3) != 0 || ((uintptr_t)zero & 15) != 0))
+    {
+        if(int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(zero), zero_floats, 0u, stream))
+            return rc;
+        zero_floats = 0;
+    }
     if(ntx * nty == 0)
         return DSX_OK;
+    float4* zero4 = reinterpret_cast<float4*>(zero);
+    const int64_t zero_vecs = zero_floats / 4;
     {
         DSX_TIMED("blend_fwd_kernel", stream);
         if(blend_pixels_per_lane(ntx * nty, kFwdFourPixelsFrom) == 4)
             hipLaunchKernelGGL(blend_fwd_kernel<4>, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
                                reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                               cam.image_height, ntx, sort_flag_a, sort_flag_b);
+                               cam.image_height, ntx, sort_flag_a, sort_flag_b, zero4, zero_vecs);
         else
             hipLaunchKernelGGL(blend_fwd_kernel<1>, dim3(4 * ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
                                reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                               cam.image_height, ntx, sort_flag_a, sort_flag_b);
+                               cam.image_height, ntx, sort_flag_a, sort_flag_b, zero4, zero_vecs);
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
@@ -499,11 +523,11 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
 
 int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, const int32_t* sorted_ids,
                      const float* splats, const float* final_T, const int32_t* final_idx, const float* v_image,
-                     float* grads, hipStream_t stream)
+                     float* grads, hipStream_t stream, bool grads_are_zero)
 {
-    int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(grads), n * DSX_GRAD_FLOATS, 0u, stream);
-    if(rc)
-        return rc;
+    if(!grads_are_zero)
+        if(int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(grads), n * DSX_GRAD_FLOATS, 0u, stream))
+            return rc;
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
     if(ntx * nty == 0 || n == 0)
         return DSX_OK;

@@ -245,11 +245,12 @@ int launch_tile_ranges(int64_t k, const int64_t* sorted_keys, int num_tiles, int
 int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids,
                      const float* splats, float* image, float* final_T, int32_t* final_idx,
                      hipStream_t stream,
-                     const uint32_t* sort_flag_a = nullptr, const uint32_t* sort_flag_b = nullptr);
+                     const uint32_t* sort_flag_a = nullptr, const uint32_t* sort_flag_b = nullptr,
+                     float* zero = nullptr, int64_t zero_floats = 0);
 int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges,
                      const int32_t* sorted_ids, const float* splats, const float* final_T,
                      const int32_t* final_idx, const float* v_image, float* grads,
-                     hipStream_t stream);
+                     hipStream_t stream, bool grads_are_zero = false);
 int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d,
                         const float* scales, const float* quats, const float* splats,
                         const float* cov3d, const int32_t* radii, const float* grads,
@@ -275,6 +276,37 @@ struct KernelTimer
 __device__ __forceinline__ int lane_id()
 {
     return __lane_id();
+}
+
+// cov3D = (R S)(R S)^T from scale and (w,x,y,z) quaternion; cpp/rasterizer_kernels.cu:615-659
+__device__ __forceinline__ void cov3d_from_scale_rot(const float* sc, float4 q, float mod, float* out)
+{
+#pragma clang fp contract(off) // same bits in every translation unit (radii and tile counts derive from them)
+    float r = q.x, x = q.y, y = q.z, z = q.w;
+    const float inv_norm = 1.0f / sqrtf(r * r + x * x + y * y + z * z);
+    r = r * inv_norm;
+    x = x * inv_norm;
+    y = y * inv_norm;
+    z = z * inv_norm;
+    const float s0 = sc[0] * mod, s1 = sc[1] * mod, s2 = sc[2] * mod;
+    const float r00 = 1.0f - 2.0f * (y * y + z * z);
+    const float r01 = 2.0f * (x * y - r * z);
+    const float r02 = 2.0f * (x * z + r * y);
+    const float r10 = 2.0f * (x * y + r * z);
+    const float r11 = 1.0f - 2.0f * (x * x + z * z);
+    const float r12 = 2.0f * (y * z - r * x);
+    const float r20 = 2.0f * (x * z - r * y);
+    const float r21 = 2.0f * (y * z + r * x);
+    const float r22 = 1.0f - 2.0f * (x * x + y * y);
+    const float m00 = s0 * r00, m01 = s1 * r01, m02 = s2 * r02;
+    const float m10 = s0 * r10, m11 = s1 * r11, m12 = s2 * r12;
+    const float m20 = s0 * r20, m21 = s1 * r21, m22 = s2 * r22;
+    out[0] = m00 * m00 + m01 * m01 + m02 * m02;
+    out[1] = m00 * m10 + m01 * m11 + m02 * m12;
+    out[2] = m00 * m20 + m01 * m21 + m02 * m22;
+    out[3] = m10 * m10 + m11 * m11 + m12 * m12;
+    out[4] = m10 * m20 + m11 * m21 + m12 * m22;
+    out[5] = m20 * m20 + m21 * m21 + m22 * m22;
 }
 
 // float -> int32 with the hardware conversion's semantics made explicit (saturate, NaN -> 0).

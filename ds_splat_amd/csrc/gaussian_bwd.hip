@@ -167,7 +167,21 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
 #pragma unroll
                     for(int c = 0; c < 3; ++c)
                         T[r][c] = J[r][0] * R[0][c] + J[r][1] * R[1][c] + J[r][2] * R[2][c];
-                const float* c3 = p.cov3d + 6 * i;
+                // the covariance the forward projected: stored by it, or rebuilt here from scale and
+                // rotation with the forward's own routine (same bits; 24 bytes per Gaussian less to
+                // write there and to read here)
+                float c3[6];
+                if(p.cov3d)
+                {
+                    const float2* cs = reinterpret_cast<const float2*>(p.cov3d + 6 * i);
+                    const float2 c01 = cs[0], c23 = cs[1], c45 = cs[2];
+                    c3[0] = c01.x, c3[1] = c01.y, c3[2] = c23.x, c3[3] = c23.y, c3[4] = c45.x, c3[5] = c45.y;
+                }
+                else
+                {
+                    const float sc[3] = {p.scales[3 * i], p.scales[3 * i + 1], p.scales[3 * i + 2]};
+                    cov3d_from_scale_rot(sc, reinterpret_cast<const float4*>(p.quats)[i], p.glob, c3);
+                }
                 const float S[3][3] = {{c3[0], c3[1], c3[2]}, {c3[1], c3[3], c3[4]}, {c3[2], c3[4], c3[5]}};
                 const float Gc[2][2] = {{v_cov2d[0], 0.5f * v_cov2d[1]}, {0.5f * v_cov2d[1], v_cov2d[2]}};
                 // GT = Gc T (2x3)

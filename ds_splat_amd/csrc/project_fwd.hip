@@ -51,36 +51,6 @@ struct ProjectParams
     int ntx, nty;
 };
 
-// cov3D = (R S)(R S)^T from scale and (w,x,y,z) quaternion; cpp/rasterizer_kernels.cu:615-659
-__device__ __forceinline__ void cov3d_from_scale_rot(const float* sc, float4 q, float mod, float* out)
-{
-    float r = q.x, x = q.y, y = q.z, z = q.w;
-    const float inv_norm = 1.0f / sqrtf(r * r + x * x + y * y + z * z);
-    r = r * inv_norm;
-    x = x * inv_norm;
-    y = y * inv_norm;
-    z = z * inv_norm;
-    const float s0 = sc[0] * mod, s1 = sc[1] * mod, s2 = sc[2] * mod;
-    const float r00 = 1.0f - 2.0f * (y * y + z * z);
-    const float r01 = 2.0f * (x * y - r * z);
-    const float r02 = 2.0f * (x * z + r * y);
-    const float r10 = 2.0f * (x * y + r * z);
-    const float r11 = 1.0f - 2.0f * (x * x + z * z);
-    const float r12 = 2.0f * (y * z - r * x);
-    const float r20 = 2.0f * (x * z - r * y);
-    const float r21 = 2.0f * (y * z + r * x);
-    const float r22 = 1.0f - 2.0f * (x * x + y * y);
-    const float m00 = s0 * r00, m01 = s1 * r01, m02 = s2 * r02;
-    const float m10 = s0 * r10, m11 = s1 * r11, m12 = s2 * r12;
-    const float m20 = s0 * r20, m21 = s1 * r21, m22 = s2 * r22;
-    out[0] = m00 * m00 + m01 * m01 + m02 * m02;
-    out[1] = m00 * m10 + m01 * m11 + m02 * m12;
-    out[2] = m00 * m20 + m01 * m21 + m02 * m22;
-    out[3] = m10 * m10 + m11 * m11 + m12 * m12;
-    out[4] = m10 * m20 + m11 * m21 + m12 * m22;
-    out[5] = m20 * m20 + m21 * m21 + m22 * m22;
-}
-
 // SH degree 0..3 -> RGB (+0.5, clamped at 0), term order as cpp/rasterizer_kernels.cu:433-554,
 // in two steps that add to the same accumulators in the reference's order: degrees 0-2 from
 // floats 0..26 of the row, then degree 3 from float 27 (f27) and floats 28..47 (g[0..19]).
@@ -304,6 +274,7 @@ __global__ __launch_bounds__(kProjBlock) void project_fwd_kernel(const ProjectPa
             const float4 q = reinterpret_cast<const float4*>(p.quats)[i];
             cov3d_from_scale_rot(sc, q, p.scale_modifier, c3);
         }
+        if(p.cov3d) // optional: the backward can rebuild it from scale and rotation
         {
             float2* o = reinterpret_cast<float2*>(p.cov3d + 6 * i);
             o[0] = make_float2(c3[0], c3[1]);

@@ -69,14 +69,18 @@ at::Tensor& pinned_key_count()
 
 } // namespace
 
-// image[H,W,3], radii[N], splats[N,12], cov3d[N,6], sorted_ids[K], ranges[T+1], final_T[H,W], final_idx[H,W]
+// image[H,W,3], radii[N], splats[N,12], sorted_ids[K], ranges[T+1], final_T[H,W], final_idx[H,W]
+// (the 3-D covariances are not kept: the backward rebuilds them from scales and rotations, or
+// reads cov3d_precomp) and, when prepare_backward is set, the backward's gradient accumulator
+// [N,12], which the blend kernel zeroes on the side (undefined otherwise)
 std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
                                 int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view,
                                 const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
                                 const at::Tensor& means3d, const c10::optional<at::Tensor>& scales,
                                 const c10::optional<at::Tensor>& quats, const at::Tensor& opacities,
                                 const c10::optional<at::Tensor>& shs, const c10::optional<at::Tensor>& cov3d_precomp,
-                                const c10::optional<at::Tensor>& colors_precomp, int64_t stream)
+                                const c10::optional<at::Tensor>& colors_precomp, bool prepare_backward,
+                                int64_t stream)
 {
     const at::Device dev = means3d.device();
     c10::DeviceGuard guard(dev);
@@ -90,7 +94,6 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
 
     at::Tensor splats = at::empty({n, DSX_SPLAT_FLOATS}, f32);
     at::Tensor radii = at::empty({n}, i32);
-    at::Tensor cov3d = at::empty({n, 6}, f32);
     at::Tensor block_sums = at::empty({dsx_num_blocks(n) + 1}, i32);
     const size_t order_bytes = dsx_order_bytes(n, (int32_t)width, (int32_t)height);
     at::Tensor order = at::empty({(int64_t)std::max<size_t>(order_bytes, 1)}, u8);
@@ -98,7 +101,7 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
     uint32_t* bs = reinterpret_cast<uint32_t*>(block_sums.data_ptr<int32_t>());
     check(dsx_forward_project(&cam.c, n, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
                               opacities.data_ptr<float>(), fptr(shs), fptr(cov3d_precomp), fptr(colors_precomp),
-                              splats.data_ptr<float>(), radii.data_ptr<int32_t>(), cov3d.data_ptr<float>(), bs,
+                              splats.data_ptr<float>(), radii.data_ptr<int32_t>(), nullptr, bs,
                               bs + dsx_num_blocks(n), order.data_ptr(), order_bytes, k_host.data_ptr<int64_t>(), s));
     const int64_t k = *k_host.data_ptr<int64_t>();
     const int64_t tiles = dsx_num_tiles((int32_t)width, (int32_t)height);
@@ -109,10 +112,12 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
     at::Tensor final_idx = at::empty({height, width}, i32);
     const size_t ws_bytes = dsx_workspace_bytes(n, k, (int32_t)width, (int32_t)height);
     at::Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 1)}, u8);
+    at::Tensor grads = prepare_backward && n > 0 ? at::empty({n, DSX_GRAD_FLOATS}, f32) : at::Tensor();
     check(dsx_forward_finish(&cam.c, n, k, splats.data_ptr<float>(), order.data_ptr(), sorted_ids.data_ptr<int32_t>(),
                              ranges.data_ptr<int32_t>(), image.data_ptr<float>(), final_T.data_ptr<float>(),
-                             final_idx.data_ptr<int32_t>(), ws.data_ptr(), ws_bytes, s));
-    return {image, radii, splats, cov3d, sorted_ids, ranges, final_T, final_idx};
+                             final_idx.data_ptr<int32_t>(), ws.data_ptr(), ws_bytes,
+                             grads.defined() ? grads.data_ptr<float>() : nullptr, s));
+    return {image, radii, splats, sorted_ids, ranges, final_T, final_idx, grads};
 }
 
 // v_mean3d[N,3], v_means2d[N,3], v_shs[N,B,3] (undefined when num_bases == 0), v_colors[N,3],
@@ -123,9 +128,11 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
                                  const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
                                  int64_t num_bases, const at::Tensor& means3d, const c10::optional<at::Tensor>& scales,
                                  const c10::optional<at::Tensor>& quats, const at::Tensor& splats,
-                                 const at::Tensor& cov3d, const at::Tensor& radii, const at::Tensor& ranges,
+                                 const c10::optional<at::Tensor>& cov3d_precomp, const at::Tensor& radii,
+                                 const at::Tensor& ranges,
                                  const at::Tensor& sorted_ids, const at::Tensor& final_T, const at::Tensor& final_idx,
-                                 const at::Tensor& v_image, int64_t wanted, int64_t stream)
+                                 const at::Tensor& v_image, const c10::optional<at::Tensor>& zeroed_grads,
+                                 int64_t wanted, int64_t stream)
 {
     const at::Device dev = means3d.device();
     c10::DeviceGuard guard(dev);
@@ -145,12 +152,18 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
     at::Tensor v_shs = num_bases > 0 ? at::empty({n, num_bases, 3}, f32) : at::Tensor();
     at::Tensor v_colors = out(3, {n, 3}), v_opacity = out(4, {n, 1});
     at::Tensor v_scale = out(5, {n, 3}), v_quat = out(6, {n, 4}), v_cov3d = out(7, {n, 6});
-    at::Tensor grads = at::empty({n, DSX_GRAD_FLOATS}, f32);
+    // the accumulator that the forward zeroed (good for one backward), or a new one that the call fills
+    const bool zeroed = zeroed_grads.has_value() && zeroed_grads->defined();
+    if(zeroed)
+        TORCH_CHECK(zeroed_grads->is_contiguous() && zeroed_grads->scalar_type() == at::kFloat &&
+                        zeroed_grads->numel() == n * DSX_GRAD_FLOATS && zeroed_grads->device() == dev,
+                    "zeroed_grads must be the float32 [N, 12] accumulator of this forward");
+    at::Tensor grads = zeroed ? *zeroed_grads : at::empty({n, DSX_GRAD_FLOATS}, f32);
     check(dsx_backward(&cam.c, n, (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
-                       splats.data_ptr<float>(), cov3d.data_ptr<float>(), radii.data_ptr<int32_t>(),
+                       splats.data_ptr<float>(), fptr(cov3d_precomp), radii.data_ptr<int32_t>(),
                        ranges.data_ptr<int32_t>(), sorted_ids.numel() ? sorted_ids.data_ptr<int32_t>() : nullptr,
                        final_T.data_ptr<float>(), final_idx.data_ptr<int32_t>(), v_image.data_ptr<float>(),
-                       grads.data_ptr<float>(), ptr(v_mean3d), ptr(v_means2d), ptr(v_shs), ptr(v_colors),
+                       grads.data_ptr<float>(), zeroed ? 1 : 0, ptr(v_mean3d), ptr(v_means2d), ptr(v_shs), ptr(v_colors),
                        ptr(v_opacity), ptr(v_scale), ptr(v_quat), ptr(v_cov3d), reinterpret_cast<void*>(stream)));
     return {v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d};
 }

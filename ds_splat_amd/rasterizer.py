@@ -99,20 +99,27 @@ class DsRasterizerFunction(torch.autograd.Function):
         stream = torch.cuda.current_stream(means_3d.device).cuda_stream
         cam = (int(s.image_height), int(s.image_width), float(s.tanfovx), float(s.tanfovy), float(s.scale_modifier),
                int(s.sh_degree), int(s.max_sh_degree), s.view_matrix, s.proj_matrix, s.campos, s.bg)
-        image, radii, splats, cov3d, sorted_ids, ranges, final_T, final_idx = ext.forward(
+        # a backward will follow: the forward's blend kernel, which leaves the memory system idle,
+        # zeroes the gradient accumulator on the side, and the first backward needs no fill
+        prepare_backward = any(ctx.needs_input_grad[:8])
+        image, radii, splats, sorted_ids, ranges, final_T, final_idx, ctx.zeroed_grads = ext.forward(
             *cam, means_3d, opt(scales), opt(rotations), opacities, opt(shs), opt(cov_3d_precomp), opt(colors_precomp),
-            stream)
+            prepare_backward, stream)
         ctx.cam = cam
         ctx.num_bases = _num_bases(shs) if shs.numel() > 0 else 0
         ctx.opacity_shape = opacities.shape
         ctx.num_keys = sorted_ids.numel()
-        ctx.save_for_backward(means_3d, scales, rotations, splats, cov3d, radii, ranges, sorted_ids, final_T, final_idx)
+        # the reference also keeps the 3-D covariances (cpp/rasterizer_torch.cu:207); the backward here
+        # rebuilds them from scales and rotations, or reads the ones that were passed in
+        ctx.save_for_backward(means_3d, scales, rotations, splats, cov_3d_precomp, radii, ranges, sorted_ids, final_T,
+                              final_idx)
         ctx.mark_non_differentiable(radii)
         return image, radii, final_T
 
     @staticmethod
     def backward(ctx, rendered_img_grad, _):
-        means_3d, scales, rotations, splats, cov3d, radii, ranges, sorted_ids, final_T, final_idx = ctx.saved_tensors
+        means_3d, scales, rotations, splats, cov3d_precomp, radii, ranges, sorted_ids, final_T, final_idx = \
+            ctx.saved_tensors
         ext = _native.load_torch_ext()
         opt = lambda t: t if t.numel() > 0 else None
         stream = torch.cuda.current_stream(means_3d.device).cuda_stream
@@ -122,9 +129,10 @@ class DsRasterizerFunction(torch.autograd.Function):
         # set-up with SH colours, scales and rotations: 36 of 320 bytes per Gaussian)
         needs = ctx.needs_input_grad
         wanted = sum(1 << i for i in range(8) if needs[i])
+        zeroed_grads, ctx.zeroed_grads = ctx.zeroed_grads, None   # good for one backward: it leaves sums behind
         v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d = ext.backward(
-            *ctx.cam, ctx.num_bases, means_3d, opt(scales), opt(rotations), splats, cov3d, radii, ranges, sorted_ids,
-            final_T, final_idx, rendered_img_grad.contiguous(), wanted, stream)
+            *ctx.cam, ctx.num_bases, means_3d, opt(scales), opt(rotations), splats, opt(cov3d_precomp), radii, ranges,
+            sorted_ids, final_T, final_idx, rendered_img_grad.contiguous(), zeroed_grads, wanted, stream)
         if v_opacity is not None and tuple(ctx.opacity_shape) != tuple(v_opacity.shape):
             v_opacity = v_opacity.reshape(ctx.opacity_shape)
         return (v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, None)

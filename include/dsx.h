@@ -95,7 +95,8 @@ size_t dsx_order_bytes(int64_t n, int32_t width, int32_t height);
  * and block_sums[dsx_num_blocks(n)] (tile count of each 256-Gaussian block; the last
  * Gaussian counts as zero, cpp/rasterizer_torch.cu:99-104).  shs may be NULL iff
  * colors_precomp is given; scales/quats may be NULL iff cov3d_precomp is given (then cov3d
- * receives a copy).  order (may be NULL): buffer of dsx_order_bytes(n, W, H) that also receives each
+ * receives a copy).  cov3d may be NULL: it is then not stored (the reference keeps it for its
+ * backward, cpp/rasterizer_torch.cu:207; dsx_gaussian_bwd can do without).  order (may be NULL): buffer of dsx_order_bytes(n, W, H) that also receives each
  * Gaussian's depth bits and packed tile rectangle, the input of dsx_depth_order. */
 int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
                     const float* quats, const float* opacities, const float* shs,
@@ -188,7 +189,9 @@ int dsx_blend_bwd(const dsx_camera* cam, int64_t n, const int32_t* ranges,
  * Any output may be NULL: that gradient is then not written (the reference computes all of them
  * and lets autograd drop those of inputs that were not given, cpp/rasterizer_torch.cu:315;
  * here an unwanted one costs no store).
- * scales/quats may be NULL when the forward used cov3d_precomp (v_scale, v_quat zeroed). */
+ * scales/quats may be NULL when the forward used cov3d_precomp (v_scale, v_quat zeroed).
+ * cov3d is what the forward stored, or cov3d_precomp itself, or NULL when scales/quats are
+ * given: the kernel then rebuilds it with the forward's own routine (bit-identical). */
 int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                      const float* scales, const float* quats, const float* splats,
                      const float* cov3d, const int32_t* radii, const float* grads, float* v_mean3d,
@@ -215,19 +218,25 @@ int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
 /* Second half: tile lists (dsx_tile_lists) and blend.  sorted_ids[k] and ranges[T+1] are
  * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H).  If one of the two
  * sorts gave up a bounded wait (see dsx_sort_flags) the image is written as NaN: a failure
- * shows without a read-back of the flags. */
+ * shows without a read-back of the flags.
+ * grads_to_zero (may be NULL): the [n*12] accumulator that a dsx_backward of this forward will
+ * use.  The blend kernel, which leaves the memory system idle, zeroes it on the side, and that
+ * dsx_backward is then called with grads_are_zero = 1 and needs no fill of its own. */
 int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
                        const void* order, int32_t* sorted_ids, int32_t* ranges, float* image,
                        float* final_T, int32_t* final_idx, void* workspace,
-                       size_t workspace_bytes, void* stream);
+                       size_t workspace_bytes, float* grads_to_zero, void* stream);
 
-/* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316. grads is scratch [n*12]. */
+/* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316. grads is scratch [n*12];
+ * grads_are_zero != 0 says that it holds zeros already (see dsx_forward_finish; true once: the
+ * call leaves sums in it). */
 int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                  const float* scales, const float* quats, const float* splats, const float* cov3d,
                  const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
                  const float* final_T, const int32_t* final_idx, const float* v_image,
-                 float* grads, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
-                 float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, void* stream);
+                 float* grads, int32_t grads_are_zero, float* v_mean3d, float* v_means2d,
+                 float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
+                 float* v_cov3d, void* stream);
 
 /* Raw-pointer forward-only render, the role of rasterizer_forward_core_deepsense
  * (cpp/ds_cuda_rasterizer/rasterizer_cuda.hpp:4-9, cpp/rasterizer_cuda.cu:128-158) without

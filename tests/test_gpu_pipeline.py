@@ -154,6 +154,60 @@ def test_only_the_gradients_asked_for_are_produced():
             assert float(b.abs().max()) > 0 or k == "means2d"
 
 
+@pytest.mark.parametrize("pixels_per_lane", ["1", "4"])
+@pytest.mark.parametrize("n", [20000, 20001])
+def test_forward_zeroes_the_accumulator_for_one_backward(monkeypatch, pixels_per_lane, n):
+    """With zero_grads the blend forward clears the backward's accumulator on the side (both kernel
+    forms, a Gaussian count that does and does not divide by the wavefronts' shares); a backward on
+    it equals one that fills for itself, and a second backward on the same state fills again."""
+    from ds_splat_amd import stages
+    monkeypatch.setenv("DSX_BLEND_PIXELS_PER_LANE", pixels_per_lane)
+    sc = make_scene("cfg1", n=n, width=320, height=200, sh_degree=3)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    cam = stages.camera_from_scene(sc, DEV)
+    args = (t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
+    image0, st0 = stages.forward(cam, *args)
+    poison = torch.full((n, 12), float("nan"), device=DEV)      # the allocator hands this block out again
+    del poison
+    image1, st1 = stages.forward(cam, *args, zero_grads=True)
+    torch.cuda.synchronize()
+    assert st0.grads is None and st1.grads.shape == (n, 12) and bool((st1.grads == 0).all())
+    assert torch.equal(image0, image1)
+    bwd = lambda st: stages.backward(cam, st, 16, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["v_image"])
+    o0, o1 = bwd(st0), bwd(st1)
+    assert st1.grads is None
+    o2 = bwd(st1)
+    torch.cuda.synchronize()
+    for k in o0:
+        scale = max(1.0, float(o0[k].abs().max()))
+        for other in (o1, o2):
+            assert torch.allclose(o0[k], other[k], rtol=1e-3, atol=1e-4 * scale), k
+
+
+def test_backward_twice_through_the_api_gives_the_same_gradients():
+    """retain_graph: the second backward finds the accumulator used and clears it for itself."""
+    from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
+    sc = make_scene("cfg1", n=20000, width=320, height=200, sh_degree=3)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    settings = GaussianRasterizationSettings(
+        image_height=sc["height"], image_width=sc["width"], tanfovx=sc["tanfovx"], tanfovy=sc["tanfovy"], bg=t["bg"],
+        scale_modifier=1.0, viewmatrix=t["viewmatrix"], projmatrix=t["projmatrix"], sh_degree=sc["sh_degree"],
+        max_sh_degree=3, campos=t["campos"], prefiltered=False, debug=False)
+    means = t["means_3d"].clone().requires_grad_(True)
+    shs = t["shs"].clone().requires_grad_(True)
+    image, _ = GaussianRasterizer(settings)(means, torch.zeros_like(means), shs, None, t["opacities"],
+                                            t["scales"] * 2.0, t["rotations"], None)
+    image.backward(t["v_image"], retain_graph=True)
+    first = (means.grad.clone(), shs.grad.clone())
+    means.grad = None
+    shs.grad = None
+    image.backward(t["v_image"])
+    torch.cuda.synchronize()
+    for a, b in zip(first, (means.grad, shs.grad)):
+        assert float(a.abs().max()) > 0
+        assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * max(1.0, float(a.abs().max())))
+
+
 def test_inria_adaptor_composites_the_background_and_keeps_the_gradients():
     """Channel-first image = HWC image + final_T * bg; gradients equal those of the wrapped API
     for the same upstream gradient (the backward kernel's background term is the derivative of

@@ -418,3 +418,10 @@ def test_gaussian_bwd_vs_oracle(oracle, sh_degree, num_bases, n):
     assert (m2[:, 2] == 0).all()
     culled = radii <= 0
     assert culled.any() and (o["v_mean3d"].cpu().numpy()[culled] == 0).all()
+    # without the stored covariances the kernel rebuilds them from scales and rotations with the
+    # forward's routine: the oracle's cov3d equals the forward's bit for bit, so nothing may change
+    o2 = st_.gaussian_bwd(cam, num_bases, dev(A["means_3d"]), dev(A["scales"]), dev(A["rotations"]),
+                          dev(pack_splats(S, radii, A["opacities"])), None, dev(radii), dev(grads))
+    torch.cuda.synchronize()
+    for key in o:
+        assert torch.equal(o[key], o2[key]), key
