@@ -509,13 +509,15 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             g[4] = -0.5f * B.y * S2;
             const float total = wave_sum8_scatter(g, lane);
             g_blue = wave_sum_to_lane63(g_blue);
-            if(lane >= 56)
+            // lane 63's blue total goes to lane 55 (row_shl:8: a lane reads the one eight up in its
+            // row), so that ONE atomic instruction carries all nine sums, each lane its own address
+            const float blue55 = dpp_move<0x108>(g_blue);
+            if(lane >= 55)
             {
-                // lane l holds the total of g[4*(l&1) + 2*((l>>1)&1) + ((l>>2)&1)]
+                // lane l >= 56 holds the total of g[4*(l&1) + 2*((l>>1)&1) + ((l>>2)&1)]
                 float* rec = grads + (int64_t)s_id[t] * DSX_GRAD_FLOATS;
-                unsafeAtomicAdd(rec + 4 * (lane & 1) + 2 * ((lane >> 1) & 1) + ((lane >> 2) & 1), total);
-                if(lane == 63)
-                    unsafeAtomicAdd(rec + 8, g_blue);
+                const int slot = lane == 55 ? 8 : 4 * (lane & 1) + 2 * ((lane >> 1) & 1) + ((lane >> 2) & 1);
+                unsafeAtomicAdd(rec + slot, lane == 55 ? blue55 : total);
             }
         }
     }
