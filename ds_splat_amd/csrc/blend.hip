@@ -134,7 +134,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
 
     // A pixel that has stopped (or lies outside the image) gets NaN as its row coordinate: its
     // exponent is then NaN, the test `power < 0` fails whatever the entry holds, and the loop
-    // needs no per-pixel flag.  `alive` counts the lane's live pixels.
+    // needs no per-pixel flag.  `alive` counts the wavefront's live pixels (a scalar: it is kept
+    // from ballots, on the scalar unit, and costs the vector unit nothing).
     float pyf[kFwdPix], T[kFwdPix], cr[kFwdPix], cg[kFwdPix], cb[kFwdPix];
     int last[kFwdPix];
     int alive = 0;
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
         const int y = y0 + 4 * p;
         const bool inside = x < W && y < H;
         pyf[p] = inside ? (float)y + 0.5f : __builtin_nanf("");
-        alive += inside ? 1 : 0;
+        alive += __popcll(__builtin_amdgcn_ballot_w64(inside));
         T[p] = 1.0f;
         cr[p] = cg[p] = cb[p] = 0.0f;
         last[p] = 0;
@@ -152,7 +153,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
 
     for(int b = start; b < end; b += kFwdBatch)
     {
-        if(__ballot(alive != 0) == 0)
+        if(alive == 0)
             break;
         __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
         uint64_t todo[kFwdBatch / DSX_WAVE]; // entries of this round that can touch the tile
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             uint64_t mask = todo[h];
             while(mask != 0)
             {
-                if(__ballot(alive != 0) == 0)
+                if(alive == 0)
                     break;
                 const int i = h * DSX_WAVE + __builtin_ctzll(mask);
                 mask &= mask - 1;
@@ -195,10 +196,15 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                     const float power = exponent_xy(ex, B.x, pyf[p] - A.y);
                     // (a NaN opacity gives alpha = 0.999 here as in the reference: fminf drops the NaN)
                     const float alpha = fminf(0.999f, B.y * fast_exp(power));
-                    const bool pass = power < 0.0f && alpha >= kAlphaThreshold;
+                    // the three decisions as wavefront masks (each is its compare's own result register),
+                    // combined on the scalar unit and handed back to the lanes as conditions
                     const float Tn = (1.0f - alpha) * T[p];
-                    const bool stop = pass && Tn < 0.0001f;
-                    const bool apply = pass && !stop;
+                    const uint64_t m_pass = __builtin_amdgcn_ballot_w64(power < 0.0f) &
+                                            __builtin_amdgcn_ballot_w64(alpha >= kAlphaThreshold);
+                    const uint64_t m_low = __builtin_amdgcn_ballot_w64(Tn < 0.0001f);
+                    const uint64_t m_stop = m_pass & m_low;
+                    const bool stop = __builtin_amdgcn_inverse_ballot_w64(m_stop);
+                    const bool apply = __builtin_amdgcn_inverse_ballot_w64(m_pass & ~m_low);
                     const float vis = apply ? alpha * T[p] : 0.0f;
                     cr[p] += vis * B.z;
                     cg[p] += vis * B.w;
@@ -206,7 +212,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                     T[p] = apply ? Tn : T[p];
                     last[p] = apply ? b + i : last[p];
                     pyf[p] = stop ? __builtin_nanf("") : pyf[p];
-                    alive -= stop ? 1 : 0;
+                    alive -= __popcll(m_stop);
                 }
             }
         }
@@ -454,8 +460,10 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             const float dxf = pxf - A.x;
             const ExponentX ex = exponent_x(A.z, A.w, dxf);
             float alpha[kBwdPix], vis[kBwdPix], dy[kBwdPix]; // dy = pixel - mean here
-            bool valid[kBwdPix];
-            bool any = false;
+            // which lanes' pixel p takes part: wavefront masks (each compare's own result register),
+            // combined on the scalar unit
+            uint64_t m_valid[kBwdPix];
+            uint64_t m_any = 0;
 #pragma unroll
             for(int p = 0; p < kBwdPix; ++p)
             {
@@ -463,10 +471,12 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
                 const float power = exponent_xy(ex, B.x, dy[p]);
                 vis[p] = fast_exp(power);
                 alpha[p] = fminf(0.99f, B.y * vis[p]);
-                valid[p] = idx <= bin_final[p] && !(power > 0.0f) && !(alpha[p] < kAlphaThreshold);
-                any = any || valid[p];
+                m_valid[p] = __builtin_amdgcn_ballot_w64(idx <= bin_final[p]) &
+                             __builtin_amdgcn_ballot_w64(!(power > 0.0f)) &
+                             __builtin_amdgcn_ballot_w64(!(alpha[p] < kAlphaThreshold));
+                m_any |= m_valid[p];
             }
-            if(__ballot(any) == 0)
+            if(m_any == 0)
                 continue;
             const float blue = s_c[t];
             float g[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; // v_x, v_y, v_conic a b c, v_opacity, v_red, v_green
@@ -477,7 +487,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
 #pragma unroll
             for(int p = 0; p < kBwdPix; ++p)
             {
-                if(valid[p])
+                if(__builtin_amdgcn_inverse_ballot_w64(m_valid[p]))
                 {
                     const float ra = __builtin_amdgcn_rcpf(1.0f - alpha[p]);
                     T[p] *= ra;
