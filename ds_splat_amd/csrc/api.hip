@@ -449,10 +449,10 @@ extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_ba
 extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
                                    const float* quats, const float* opacities, const float* shs,
                                    const float* cov3d_precomp, const float* colors_precomp, float* splats,
-                                   int32_t* radii, float* cov3d, uint32_t* block_sums, uint32_t* k_scratch,
-                                   void* order, size_t order_bytes, int64_t* num_keys, void* stream)
+                                   int32_t* radii, float* cov3d, uint32_t* block_sums, void* order, size_t order_bytes,
+                                   int64_t* num_keys, void* stream)
 {
-    if(!num_keys || !k_scratch || (n > 0 && !order))
+    if(!num_keys || (n > 0 && !order))
         return DSX_ERR_BAD_ARG;
     *num_keys = 0;
     hipStream_t s = as_stream(stream);
@@ -460,27 +460,22 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
                                  splats, radii, cov3d, block_sums, order, order_bytes, stream, true);
     if(rc || n == 0)
         return rc;
-    rc = launch_scan_u32(dsx_num_blocks(n), block_sums, k_scratch, s);
-    if(rc)
-        return rc;
-    // K travels to the host while the depth order is computed: the wait below is for the copy
-    // only (it overlaps when *num_keys is pinned host memory; with pageable memory the copy is
-    // synchronous and nothing is lost)
+    // K is the sum of the rectangles' tile counts: the corner-grid kernel, first thing beside the
+    // depth sort, adds them up, and K travels to the host while the depth order is computed.  The
+    // wait below is for that copy only (it overlaps when *num_keys is pinned host memory; with
+    // pageable memory the copy is synchronous and nothing is lost).
     hipEvent_t copied;
     if(hipEventCreateWithFlags(&copied, hipEventDisableTiming) != hipSuccess)
         return DSX_ERR_RUNTIME;
-    bool ok = hipMemcpyAsync(num_keys, k_scratch, sizeof(uint32_t), hipMemcpyDeviceToHost, s) == hipSuccess &&
-              hipEventRecord(copied, s) == hipSuccess;
-    if(ok)
-        rc = launch_depth_order(*cam, n, order, s, true);
-    ok = ok && hipEventSynchronize(copied) == hipSuccess;
+    rc = launch_depth_order(*cam, n, order, s, true, num_keys, copied);
+    // (an event that was never recorded counts as complete: no wait after a failed launch)
+    const bool ok = hipEventSynchronize(copied) == hipSuccess;
     (void)hipEventDestroy(copied);
-    if(!ok)
-        return DSX_ERR_RUNTIME;
     if(rc)
         return rc;
-    *num_keys &= 0xffffffffll; // four bytes were copied into the low half (little endian)
-    return *num_keys >= (1ll << 30) ? DSX_ERR_TOO_LARGE : DSX_OK;
+    if(!ok)
+        return DSX_ERR_RUNTIME;
+    return *num_keys >= (1ll << 30) || *num_keys < 0 ? DSX_ERR_TOO_LARGE : DSX_OK;
 }
 
 extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
@@ -552,12 +547,11 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     const int64_t nb = dsx_num_blocks(n);
 
     auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
-    size_t o_splats = 0, o_radii, o_cov3d, o_bs, o_k, o_ranges, o_T, o_idx, o_order, stage1;
+    size_t o_splats = 0, o_radii, o_cov3d, o_bs, o_ranges, o_T, o_idx, o_order, stage1;
     o_radii = align(o_splats + (size_t)n * 48);
     o_cov3d = align(o_radii + (size_t)n * 4);
     o_bs = align(o_cov3d + (size_t)n * 24);
-    o_k = align(o_bs + (size_t)nb * 4);
-    o_ranges = align(o_k + 4);
+    o_ranges = align(o_bs + (size_t)nb * 4);
     o_T = align(o_ranges + (size_t)(num_tiles + 1) * 4);
     o_idx = align(o_T + (size_t)P * 4);
     o_order = align(o_idx + (size_t)P * 4);
@@ -570,7 +564,7 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     int rc = dsx_forward_project(&cam, n, means3d, scales, quats, opacities, shs, nullptr, nullptr,
                                  reinterpret_cast<float*>(buf + o_splats), reinterpret_cast<int32_t*>(buf + o_radii),
                                  reinterpret_cast<float*>(buf + o_cov3d), reinterpret_cast<uint32_t*>(buf + o_bs),
-                                 reinterpret_cast<uint32_t*>(buf + o_k), buf + o_order, order_bytes, &k, stream);
+                                 buf + o_order, order_bytes, &k, stream);
     char* buf2 = nullptr;
     if(rc == DSX_OK)
     {

@@ -194,6 +194,7 @@ struct OrderLayout
     size_t block_sums; // uint32[blocks + 1] tile counts of 256 consecutive Gaussians IN DEPTH ORDER, scanned
     size_t slot_hist;  // uint32[kMaxPasses32 * 256] digit histograms of the tile slots of all pairs
     size_t cover;      // int32[(ntx + 1) * (nty + 1) + 1] pairs per tile (corner grid, then its 2-D prefix sum)
+    size_t key_count;  // uint64     number of pairs of the scene (summed by the corner-grid kernel)
     size_t ranges;     // int32[tiles + 1] the tile ranges, ready before the pairs exist
     size_t sort;       // Sort32Workspace
     size_t bytes;
@@ -220,7 +221,7 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
                   uint2* gather_dst = nullptr, bool already_cleared = false);
 // already_cleared: the words of depth_order_clear_region are zero already (the projection did it)
 int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream,
-                       bool already_cleared = false);
+                       bool already_cleared = false, void* k_host = nullptr, hipEvent_t k_copied = nullptr);
 // the part of an `order` buffer that must be zero when launch_depth_order starts
 void depth_order_clear_region(const dsx_camera& cam, int64_t n, void* order, uint32_t** words, int64_t* count);
 int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,

@@ -572,7 +572,10 @@ OrderLayout order_layout(int64_t n, int image_width, int image_height)
     o.sort = off;
     off = align(off + sort32_workspace(n, 32, sort32_tile_keys(n)).bytes);
     o.cover = off;
-    off = align(off + (size_t)((tiles_x(image_width) + 1) * (tiles_y(image_height) + 1) + 1) * 4);
+    off += (size_t)((tiles_x(image_width) + 1) * (tiles_y(image_height) + 1) + 1) * 4;
+    off = (off + 7) & ~(size_t)7;
+    o.key_count = off; // inside the region that is zeroed with the corner grid
+    off = align(off + 8);
     o.ranges = off;
     off += (size_t)(tiles_x(image_width) * tiles_y(image_height) + 1) * 4;
     o.bytes = align(off);
@@ -615,10 +618,12 @@ constexpr int kCoverLdsCells = 14 * 1024;      // grids up to this many cells (5
 constexpr int kCoverLdsCellsLarge = 38 * 1024; // up to 152 KB of the CU's 160 KB, once the kernels are allowed it
 
 __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* __restrict__ rects, int64_t n, int ntx,
-                                                                   int nty, int use_lds, int32_t* __restrict__ grid)
+                                                                   int nty, int use_lds, int32_t* __restrict__ grid,
+                                                                   unsigned long long* __restrict__ key_count)
 {
     extern __shared__ int32_t s_grid[];
     const int tid = threadIdx.x;
+    unsigned long long pairs = 0; // tiles of this thread's rectangles: summed over the launch this is K
     const int pitch = ntx + 1;
     const int cells = pitch * (nty + 1) + 1;
     int32_t* acc = use_lds ? s_grid : grid;
@@ -634,6 +639,7 @@ __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* 
         const int w = (int)(r.y & 0xffffu), h = (int)((r.y >> 16) & 0x7fffu);
         if(w == 0 || h == 0)
             continue;
+        pairs += (unsigned long long)(w * h);
         if(r.y >> 31)
         {
             atomicAdd(&acc[cells - 1], w * h);
@@ -651,6 +657,23 @@ __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* 
         for(int j = tid; j < cells; j += kCoverThreads)
             if(s_grid[j])
                 atomicAdd(&grid[j], s_grid[j]);
+    }
+    // the number of pairs of the whole scene (64 bits: it is compared with the 2^30 limit, not wrapped)
+    // (one atomic per workgroup: atomics on one address serialise in the L2)
+    __shared__ unsigned long long s_pairs[kCoverThreads / DSX_WAVE];
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1)
+        pairs += __shfl_xor(pairs, o, DSX_WAVE);
+    if((tid & 63) == 0)
+        s_pairs[tid >> 6] = pairs;
+    __syncthreads();
+    if(tid == 0)
+    {
+        unsigned long long total = 0;
+        for(int w = 0; w < kCoverThreads / DSX_WAVE; ++w)
+            total += s_pairs[w];
+        if(total)
+            atomicAdd(key_count, total);
     }
 }
 
@@ -799,7 +822,10 @@ void depth_order_clear_region(const dsx_camera& cam, int64_t n, void* order, uin
     *count = (int64_t)((w.bytes + (o.ranges - o.cover)) / 4);
 }
 
-int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream, bool already_cleared)
+// k_host (optional, with k_copied): receives the number of pairs as 8 bytes as soon as the
+// rectangles have been counted; k_copied is recorded behind that copy.
+int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream, bool already_cleared,
+                       void* k_host, hipEvent_t k_copied)
 {
     if(n <= 0)
         return DSX_OK;
@@ -838,6 +864,7 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
             side = nullptr;
         }
     }
+    bool k_copy_ok = true;
     {
         hipStream_t cs = side ? side : stream;
         const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
@@ -865,8 +892,11 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
             DSX_TIMED("tile_cover_kernel", cs);
             hipLaunchKernelGGL(tile_cover_kernel, dim3((unsigned)min((int64_t)kCoverBlocks, want)), dim3(kCoverThreads),
                                use_lds ? (size_t)cells * 4 : 0, cs, reinterpret_cast<const uint2*>(base + o.rects), n,
-                               ntx, nty, use_lds, grid);
+                               ntx, nty, use_lds, grid, reinterpret_cast<unsigned long long*>(base + o.key_count));
         }
+        if(k_host)
+            k_copy_ok = hipMemcpyAsync(k_host, base + o.key_count, 8, hipMemcpyDeviceToHost, cs) == hipSuccess &&
+                        hipEventRecord(k_copied, cs) == hipSuccess;
         {
             DSX_TIMED("tile_counts_kernel", cs);
             hipLaunchKernelGGL(tile_counts_kernel, dim3(1), dim3(kCoverThreads), use_lds ? (size_t)cells * 4 : 0, cs,
@@ -890,6 +920,8 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
     };
     if(hipGetLastError() != hipSuccess)
         return finish(DSX_ERR_LAUNCH);
+    if(!k_copy_ok)
+        return finish(DSX_ERR_RUNTIME);
 
     uint32_t *ko, *vo;
     // 32 key bits = 4 passes: the values (iota in pass 0) go b, a, b, a and end in ids_a

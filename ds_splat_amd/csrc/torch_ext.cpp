@@ -94,15 +94,15 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
 
     at::Tensor splats = at::empty({n, DSX_SPLAT_FLOATS}, f32);
     at::Tensor radii = at::empty({n}, i32);
-    at::Tensor block_sums = at::empty({dsx_num_blocks(n) + 1}, i32);
+    at::Tensor block_sums = at::empty({std::max<int64_t>(dsx_num_blocks(n), 1)}, i32);
     const size_t order_bytes = dsx_order_bytes(n, (int32_t)width, (int32_t)height);
     at::Tensor order = at::empty({(int64_t)std::max<size_t>(order_bytes, 1)}, u8);
     at::Tensor& k_host = pinned_key_count();
     uint32_t* bs = reinterpret_cast<uint32_t*>(block_sums.data_ptr<int32_t>());
     check(dsx_forward_project(&cam.c, n, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
                               opacities.data_ptr<float>(), fptr(shs), fptr(cov3d_precomp), fptr(colors_precomp),
-                              splats.data_ptr<float>(), radii.data_ptr<int32_t>(), nullptr, bs,
-                              bs + dsx_num_blocks(n), order.data_ptr(), order_bytes, k_host.data_ptr<int64_t>(), s));
+                              splats.data_ptr<float>(), radii.data_ptr<int32_t>(), nullptr, bs, order.data_ptr(),
+                              order_bytes, k_host.data_ptr<int64_t>(), s));
     const int64_t k = *k_host.data_ptr<int64_t>();
     const int64_t tiles = dsx_num_tiles((int32_t)width, (int32_t)height);
     at::Tensor sorted_ids = at::empty({k}, i32);

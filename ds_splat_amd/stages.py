@@ -244,14 +244,13 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     st.splats = torch.empty((n, N.SPLAT_FLOATS), dtype=torch.float32, device=dev)
     st.radii = torch.empty((n,), dtype=torch.int32, device=dev)
     st.cov3d = torch.empty((n, 6), dtype=torch.float32, device=dev)
-    block_sums = torch.empty((int(lib.dsx_num_blocks(n)) + 1,), dtype=torch.int32, device=dev)
-    k_scratch = block_sums[-1:]
+    block_sums = torch.empty((int(lib.dsx_num_blocks(n)),), dtype=torch.int32, device=dev)
     order = new_order(cam, n, dev)
     k_host = _pinned_i64()
     stream = _stream()
     N.check(lib.dsx_forward_project(cam.ref, n, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(opacities), _ptr(shs),
                                     _ptr(cov3d_precomp), _ptr(colors_precomp), _ptr(st.splats), _ptr(st.radii),
-                                    _ptr(st.cov3d), _ptr(block_sums), _ptr(k_scratch), _ptr(order), order.numel(),
+                                    _ptr(st.cov3d), _ptr(block_sums), _ptr(order), order.numel(),
                                     _ptr(k_host), stream))
     k = int(k_host.item())
     st.num_keys = k

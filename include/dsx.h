@@ -203,17 +203,18 @@ int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const 
 /* ------------------------------------------------------------------------------------ */
 
 /* First half of rasterizer_forward_deepsense (cpp/rasterizer_torch.cu:170-208): projection,
- * block scan, the read-back of K (the one host wait of the forward, in place of the reference's
- * two device drains at cpp/rasterizer_torch.cu:103-104) and, overlapping that read-back, the
- * depth order.  block_sums is scanned in place.  k_scratch: device uint32[1].  order: device
- * buffer of dsx_order_bytes(n, W, H).  *num_keys (host; pinned memory lets the copy overlap)
- * receives K. */
+ * the read-back of K (the one host wait of the forward, in place of the reference's block scan
+ * and two device drains at cpp/rasterizer_torch.cu:95-104; K is summed from the tile rectangles
+ * by the first kernel that runs beside the depth sort) and, overlapping that read-back, the depth
+ * order.  block_sums[dsx_num_blocks(n)] receives the tile count of each 256-Gaussian block
+ * (not scanned).  order: device buffer of dsx_order_bytes(n, W, H).  *num_keys (host; pinned
+ * memory lets the copy overlap) receives K. */
 int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
                         const float* scales, const float* quats, const float* opacities,
                         const float* shs, const float* cov3d_precomp, const float* colors_precomp,
                         float* splats, int32_t* radii, float* cov3d, uint32_t* block_sums,
-                        uint32_t* k_scratch, void* order, size_t order_bytes,
-                        int64_t* num_keys /* host */, void* stream);
+                        void* order, size_t order_bytes, int64_t* num_keys /* host */,
+                        void* stream);
 
 /* Second half: tile lists (dsx_tile_lists) and blend.  sorted_ids[k] and ranges[T+1] are
  * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H).  If one of the two
