@@ -423,11 +423,12 @@ extern "C" int dsx_blend_bwd(const dsx_camera* cam, int64_t n, const int32_t* ra
                             as_stream(stream));
 }
 
-extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+// conic_in_grads: places 9..11 of every accumulator record hold the conic (dsx_forward_finish put it there)
+static int gaussian_bwd_checked(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                                 const float* scales, const float* quats, const float* splats, const float* cov3d,
                                 const int32_t* radii, const float* grads, float* v_mean3d, float* v_means2d,
                                 float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
-                                float* v_cov3d, void* stream)
+                                float* v_cov3d, void* stream, bool conic_in_grads)
 {
     if(int rc = check_camera(cam))
         return rc;
@@ -443,7 +444,17 @@ extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_ba
         return DSX_ERR_BAD_ARG; // without the stored covariance the kernel rebuilds it from scale and rotation
     return launch_gaussian_bwd(*cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
                                v_means2d, num_bases > 0 ? v_shs : nullptr, v_colors, v_opacity, v_scale, v_quat,
-                               v_cov3d, as_stream(stream));
+                               v_cov3d, as_stream(stream), conic_in_grads);
+}
+
+extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+                                const float* scales, const float* quats, const float* splats, const float* cov3d,
+                                const int32_t* radii, const float* grads, float* v_mean3d, float* v_means2d,
+                                float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
+                                float* v_cov3d, void* stream)
+{
+    return gaussian_bwd_checked(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
+                                v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, stream, false);
 }
 
 extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
@@ -481,7 +492,7 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
 extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
                                   const void* order, int32_t* sorted_ids, int32_t* ranges, float* image,
                                   float* final_T, int32_t* final_idx, void* workspace, size_t workspace_bytes,
-                                  float* grads_to_zero, void* stream)
+                                  float* grads_to_prepare, void* stream)
 {
     if(!image || !final_T || !final_idx)
         return DSX_ERR_BAD_ARG;
@@ -493,14 +504,14 @@ extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, c
     if(rc)
         return rc;
     return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream), depth_flag,
-                            partition_flag, grads_to_zero, n * DSX_GRAD_FLOATS);
+                            partition_flag, n > 0 ? grads_to_prepare : nullptr, n);
 }
 
 extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                             const float* scales, const float* quats, const float* splats, const float* cov3d,
                             const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
                             const float* final_T, const int32_t* final_idx, const float* v_image, float* grads,
-                            int32_t grads_are_zero, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
+                            int32_t grads_prepared, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
                             float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, void* stream)
 {
     if(int rc = check_camera(cam))
@@ -512,11 +523,12 @@ extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases,
     if(!ranges || !final_T || !final_idx || !v_image || !grads || !splats)
         return DSX_ERR_BAD_ARG;
     int rc = launch_blend_bwd(*cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
-                              as_stream(stream), grads_are_zero != 0);
+                              as_stream(stream), grads_prepared != 0);
     if(rc)
         return rc;
-    return dsx_gaussian_bwd(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
-                            v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, stream);
+    return gaussian_bwd_checked(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
+                                v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, stream,
+                                grads_prepared != 0);
 }
 
 extern "C" int dsx_forward_core(const float* means3d, const float* shs, const float* opacities, const float* scales,

@@ -111,7 +111,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                                                              int32_t* __restrict__ final_idx, int W, int H, int ntx,
                                                              const uint32_t* __restrict__ sort_flag_a,
                                                              const uint32_t* __restrict__ sort_flag_b,
-                                                             float4* __restrict__ zero, int64_t zero_vecs)
+                                                             float4* __restrict__ prep, int64_t prep_count)
 {
     __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic a, conic b
     __shared__ float4 s_b[kFwdBatch]; // conic c, opacity, red, green
@@ -240,48 +240,51 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             final_idx[pix] = last[p];
         }
     }
-    // A side job for the memory system, which this kernel leaves idle: every wavefront zeroes its
-    // share of a buffer that the caller needs cleared (the backward's gradient accumulator).  At
-    // the end, where nothing waits for the stores and the wavefronts arrive spread over time (at
+    // A side job for the memory system, which this kernel leaves idle: every wavefront prepares
+    // its share of the backward's gradient accumulator, twelve floats per Gaussian: the nine sums
+    // zeroed and, in the three spare places, the conic, which the per-Gaussian backward then has
+    // at hand with the sums instead of fetching the splat records for it.  At the end of the
+    // kernel, where nothing waits for the stores and the wavefronts arrive spread over time (at
     // the start they would all come at once and hold up the first loads: 0.147 against 0.140 ms).
-    if(zero_vecs > 0)
+    if(prep_count > 0)
     {
-        const int64_t share = (zero_vecs + gridDim.x - 1) / gridDim.x;
-        const int64_t z0 = (int64_t)blockIdx.x * share;
-        const int64_t z1 = min(z0 + share, zero_vecs);
-        for(int64_t j = z0 + lane; j < z1; j += DSX_WAVE)
-            zero[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        static_assert(DSX_GRAD_FLOATS == 12, "three float4 per Gaussian");
+        const int64_t share = (prep_count + gridDim.x - 1) / gridDim.x;
+        const int64_t g0 = (int64_t)blockIdx.x * share;
+        const int64_t g1 = min(g0 + share, prep_count);
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+        for(int64_t g = g0 + lane; g < g1; g += DSX_WAVE)
+        {
+            const float4 q1 = splats[3 * g + 1]; // conic a, b, c, opacity
+            prep[3 * g] = zero;
+            prep[3 * g + 1] = zero;
+            prep[3 * g + 2] = make_float4(0.f, q1.x, q1.y, q1.z);
+        }
     }
 }
 
 int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids, const float* splats,
                      float* image, float* final_T, int32_t* final_idx, hipStream_t stream,
-                     const uint32_t* sort_flag_a, const uint32_t* sort_flag_b, float* zero, int64_t zero_floats)
+                     const uint32_t* sort_flag_a, const uint32_t* sort_flag_b, float* prepare_grads,
+                     int64_t num_gaussians)
 {
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
-    if(zero == nullptr)
-        zero_floats = 0;
-    // the kernel zeroes in 16-byte units; anything else (or no kernel at all) takes the plain fill
-    if(zero_floats > 0 && (ntx * nty == 0 || (zero_floats & 3) != 0 || ((uintptr_t)zero & 15) != 0))
-    {
-        if(int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(zero), zero_floats, 0u, stream))
-            return rc;
-        zero_floats = 0;
-    }
     if(ntx * nty == 0)
-        return DSX_OK;
-    float4* zero4 = reinterpret_cast<float4*>(zero);
-    const int64_t zero_vecs = zero_floats / 4;
+        return prepare_grads ? DSX_ERR_BAD_ARG : DSX_OK; // (no image, no kernel, nothing prepared)
+    if(prepare_grads && (((uintptr_t)prepare_grads & 15) != 0 || splats == nullptr))
+        return DSX_ERR_BAD_ARG;
+    float4* prep = reinterpret_cast<float4*>(prepare_grads);
+    const int64_t prep_count = prepare_grads ? num_gaussians : 0;
     {
         DSX_TIMED("blend_fwd_kernel", stream);
         if(blend_pixels_per_lane(ntx * nty, kFwdFourPixelsFrom) == 4)
             hipLaunchKernelGGL(blend_fwd_kernel<4>, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
                                reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                               cam.image_height, ntx, sort_flag_a, sort_flag_b, zero4, zero_vecs);
+                               cam.image_height, ntx, sort_flag_a, sort_flag_b, prep, prep_count);
         else
             hipLaunchKernelGGL(blend_fwd_kernel<1>, dim3(4 * ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
                                reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                               cam.image_height, ntx, sort_flag_a, sort_flag_b, zero4, zero_vecs);
+                               cam.image_height, ntx, sort_flag_a, sort_flag_b, prep, prep_count);
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
@@ -535,9 +538,9 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
 
 int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, const int32_t* sorted_ids,
                      const float* splats, const float* final_T, const int32_t* final_idx, const float* v_image,
-                     float* grads, hipStream_t stream, bool grads_are_zero)
+                     float* grads, hipStream_t stream, bool grads_prepared)
 {
-    if(!grads_are_zero)
+    if(!grads_prepared)
         if(int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(grads), n * DSX_GRAD_FLOATS, 0u, stream))
             return rc;
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);

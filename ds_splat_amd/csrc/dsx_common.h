@@ -247,17 +247,17 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
                      const float* splats, float* image, float* final_T, int32_t* final_idx,
                      hipStream_t stream,
                      const uint32_t* sort_flag_a = nullptr, const uint32_t* sort_flag_b = nullptr,
-                     float* zero = nullptr, int64_t zero_floats = 0);
+                     float* prepare_grads = nullptr, int64_t num_gaussians = 0);
 int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges,
                      const int32_t* sorted_ids, const float* splats, const float* final_T,
                      const int32_t* final_idx, const float* v_image, float* grads,
-                     hipStream_t stream, bool grads_are_zero = false);
+                     hipStream_t stream, bool grads_prepared = false);
 int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d,
                         const float* scales, const float* quats, const float* splats,
                         const float* cov3d, const int32_t* radii, const float* grads,
                         float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
                         float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d,
-                        hipStream_t stream);
+                        hipStream_t stream, bool conic_in_grads = false);
 int launch_fill_u32(uint32_t* p, int64_t count, uint32_t value, hipStream_t stream);
 
 // Optional per-kernel timing (diagnostics for benchmarks): when switched on through

@@ -34,6 +34,7 @@ struct GaussianBwdParams
     float* v_cov3d;
     float fx, fy, glob;
     int sh_degree, num_bases;
+    int conic_in_grads; // the accumulator's places 9..11 hold the conic (the forward put it there)
 };
 
 __device__ __forceinline__ void mat3_mul(const float (&A)[3][3], const float (&B)[3][3], float (&C)[3][3])
@@ -138,7 +139,12 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
             // conic -> cov2d:  v_Sigma = -X G X, X = conic, G = symmetrised v_conic
             float v_cov2d[3];
             {
-                const float4 q1 = p.splats[3 * i + 1];
+                // the conic: behind the sums when the forward prepared the accumulator, else from the splat record
+                float4 q1;
+                if(p.conic_in_grads)
+                    q1 = make_float4(g2.y, g2.z, g2.w, 0.f);
+                else
+                    q1 = p.splats[3 * i + 1];
                 const float X[2][2] = {{q1.x, q1.y}, {q1.y, q1.z}};
                 const float G[2][2] = {{vc[0], 0.5f * vc[1]}, {0.5f * vc[1], vc[2]}};
                 float M[2][2], N[2][2];
@@ -350,7 +356,8 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
 int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d, const float* scales,
                         const float* quats, const float* splats, const float* cov3d, const int32_t* radii,
                         const float* grads, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
-                        float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, hipStream_t stream)
+                        float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, hipStream_t stream,
+                        bool conic_in_grads)
 {
     if(n == 0)
         return DSX_OK;
@@ -382,6 +389,7 @@ int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const f
     p.glob = cam.scale_modifier;
     p.sh_degree = cam.sh_degree;
     p.num_bases = num_bases;
+    p.conic_in_grads = conic_in_grads ? 1 : 0;
     const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
     {
         DSX_TIMED("gaussian_bwd_kernel", stream);

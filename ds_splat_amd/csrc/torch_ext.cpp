@@ -72,7 +72,8 @@ at::Tensor& pinned_key_count()
 // image[H,W,3], radii[N], splats[N,12], sorted_ids[K], ranges[T+1], final_T[H,W], final_idx[H,W]
 // (the 3-D covariances are not kept: the backward rebuilds them from scales and rotations, or
 // reads cov3d_precomp) and, when prepare_backward is set, the backward's gradient accumulator
-// [N,12], which the blend kernel zeroes on the side (undefined otherwise)
+// [N,12], which the blend kernel prepares on the side: sums zeroed, conics in the spare places
+// (undefined otherwise)
 std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
                                 int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view,
                                 const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
@@ -131,7 +132,7 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
                                  const c10::optional<at::Tensor>& cov3d_precomp, const at::Tensor& radii,
                                  const at::Tensor& ranges,
                                  const at::Tensor& sorted_ids, const at::Tensor& final_T, const at::Tensor& final_idx,
-                                 const at::Tensor& v_image, const c10::optional<at::Tensor>& zeroed_grads,
+                                 const at::Tensor& v_image, const c10::optional<at::Tensor>& prepared_grads,
                                  int64_t wanted, int64_t stream)
 {
     const at::Device dev = means3d.device();
@@ -152,18 +153,19 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
     at::Tensor v_shs = num_bases > 0 ? at::empty({n, num_bases, 3}, f32) : at::Tensor();
     at::Tensor v_colors = out(3, {n, 3}), v_opacity = out(4, {n, 1});
     at::Tensor v_scale = out(5, {n, 3}), v_quat = out(6, {n, 4}), v_cov3d = out(7, {n, 6});
-    // the accumulator that the forward zeroed (good for one backward), or a new one that the call fills
-    const bool zeroed = zeroed_grads.has_value() && zeroed_grads->defined();
-    if(zeroed)
-        TORCH_CHECK(zeroed_grads->is_contiguous() && zeroed_grads->scalar_type() == at::kFloat &&
-                        zeroed_grads->numel() == n * DSX_GRAD_FLOATS && zeroed_grads->device() == dev,
-                    "zeroed_grads must be the float32 [N, 12] accumulator of this forward");
-    at::Tensor grads = zeroed ? *zeroed_grads : at::empty({n, DSX_GRAD_FLOATS}, f32);
+    // the accumulator that the forward prepared (sums zeroed, conics in place; good for one
+    // backward), or a new one that the call fills
+    const bool prepared = prepared_grads.has_value() && prepared_grads->defined();
+    if(prepared)
+        TORCH_CHECK(prepared_grads->is_contiguous() && prepared_grads->scalar_type() == at::kFloat &&
+                        prepared_grads->numel() == n * DSX_GRAD_FLOATS && prepared_grads->device() == dev,
+                    "prepared_grads must be the float32 [N, 12] accumulator of this forward");
+    at::Tensor grads = prepared ? *prepared_grads : at::empty({n, DSX_GRAD_FLOATS}, f32);
     check(dsx_backward(&cam.c, n, (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
                        splats.data_ptr<float>(), fptr(cov3d_precomp), radii.data_ptr<int32_t>(),
                        ranges.data_ptr<int32_t>(), sorted_ids.numel() ? sorted_ids.data_ptr<int32_t>() : nullptr,
                        final_T.data_ptr<float>(), final_idx.data_ptr<int32_t>(), v_image.data_ptr<float>(),
-                       grads.data_ptr<float>(), zeroed ? 1 : 0, ptr(v_mean3d), ptr(v_means2d), ptr(v_shs), ptr(v_colors),
+                       grads.data_ptr<float>(), prepared ? 1 : 0, ptr(v_mean3d), ptr(v_means2d), ptr(v_shs), ptr(v_colors),
                        ptr(v_opacity), ptr(v_scale), ptr(v_quat), ptr(v_cov3d), reinterpret_cast<void*>(stream)));
     return {v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d};
 }

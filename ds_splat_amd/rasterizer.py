@@ -100,9 +100,10 @@ class DsRasterizerFunction(torch.autograd.Function):
         cam = (int(s.image_height), int(s.image_width), float(s.tanfovx), float(s.tanfovy), float(s.scale_modifier),
                int(s.sh_degree), int(s.max_sh_degree), s.view_matrix, s.proj_matrix, s.campos, s.bg)
         # a backward will follow: the forward's blend kernel, which leaves the memory system idle,
-        # zeroes the gradient accumulator on the side, and the first backward needs no fill
+        # prepares the gradient accumulator on the side (sums zeroed, conics beside them), and the
+        # first backward needs no fill and no second look at the splat records
         prepare_backward = any(ctx.needs_input_grad[:8])
-        image, radii, splats, sorted_ids, ranges, final_T, final_idx, ctx.zeroed_grads = ext.forward(
+        image, radii, splats, sorted_ids, ranges, final_T, final_idx, ctx.prepared_grads = ext.forward(
             *cam, means_3d, opt(scales), opt(rotations), opacities, opt(shs), opt(cov_3d_precomp), opt(colors_precomp),
             prepare_backward, stream)
         ctx.cam = cam
@@ -129,10 +130,10 @@ class DsRasterizerFunction(torch.autograd.Function):
         # set-up with SH colours, scales and rotations: 36 of 320 bytes per Gaussian)
         needs = ctx.needs_input_grad
         wanted = sum(1 << i for i in range(8) if needs[i])
-        zeroed_grads, ctx.zeroed_grads = ctx.zeroed_grads, None   # good for one backward: it leaves sums behind
+        prepared_grads, ctx.prepared_grads = ctx.prepared_grads, None   # good for one backward: it leaves sums behind
         v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d = ext.backward(
             *ctx.cam, ctx.num_bases, means_3d, opt(scales), opt(rotations), splats, opt(cov3d_precomp), radii, ranges,
-            sorted_ids, final_T, final_idx, rendered_img_grad.contiguous(), zeroed_grads, wanted, stream)
+            sorted_ids, final_T, final_idx, rendered_img_grad.contiguous(), prepared_grads, wanted, stream)
         if v_opacity is not None and tuple(ctx.opacity_shape) != tuple(v_opacity.shape):
             v_opacity = v_opacity.reshape(ctx.opacity_shape)
         return (v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, None)

@@ -233,10 +233,11 @@ def sort_flag_indices(cam, n, k, order, workspace):
 
 
 def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, colors_precomp=None,
-            after_project=None, zero_grads=False):
+            after_project=None, prepare_grads=False):
     """Whole forward: returns (image[H,W,3], ForwardState).  after_project(order, n, k), if given,
-    runs between the two halves (diagnostics).  zero_grads: also allocate the backward's gradient
-    accumulator and let the blend kernel zero it on the side (one backward may then skip its fill)."""
+    runs between the two halves (diagnostics).  prepare_grads: also allocate the backward's gradient
+    accumulator and let the blend kernel prepare it on the side: sums zeroed, conics in the spare
+    places (one backward may then skip its fill and its reads of the splat records)."""
     lib = N.load()
     n = means3d.shape[0]
     dev = means3d.device
@@ -263,7 +264,7 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     st.final_idx = torch.empty((cam.height, cam.width), dtype=torch.int32, device=dev)
     nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
-    st.grads = torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=dev) if zero_grads else None
+    st.grads = torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=dev) if prepare_grads else None
     N.check(lib.dsx_forward_finish(cam.ref, n, k, _ptr(st.splats), _ptr(order), _ptr(st.sorted_ids),
                                    _ptr(st.ranges), _ptr(image), _ptr(st.final_T), _ptr(st.final_idx), _ptr(ws),
                                    nbytes, _ptr(st.grads), stream))
@@ -275,13 +276,13 @@ def backward(cam, st, num_bases, means3d, scales, quats, v_image):
     n = means3d.shape[0]
     dev = means3d.device
     o = _bwd_outputs(n, num_bases, dev)
-    # an accumulator that the forward zeroed serves one backward; after that it holds sums
-    zeroed = getattr(st, "grads", None) is not None
-    grads = st.grads if zeroed else torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=dev)
+    # an accumulator that the forward prepared serves one backward; after that it holds sums
+    prepared = getattr(st, "grads", None) is not None
+    grads = st.grads if prepared else torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=dev)
     st.grads = None
     N.check(lib.dsx_backward(cam.ref, n, num_bases, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(st.splats),
                              _ptr(st.cov3d), _ptr(st.radii), _ptr(st.ranges), _ptr(st.sorted_ids), _ptr(st.final_T),
-                             _ptr(st.final_idx), _ptr(v_image), _ptr(grads), int(zeroed), _ptr(o["v_mean3d"]),
+                             _ptr(st.final_idx), _ptr(v_image), _ptr(grads), int(prepared), _ptr(o["v_mean3d"]),
                              _ptr(o["v_means2d"]), _ptr(o["v_shs"]), _ptr(o["v_colors"]), _ptr(o["v_opacity"]),
                              _ptr(o["v_scale"]), _ptr(o["v_quat"]), _ptr(o["v_cov3d"]), _stream()))
     o["grads"] = grads

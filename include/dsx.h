@@ -220,22 +220,24 @@ int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
  * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H).  If one of the two
  * sorts gave up a bounded wait (see dsx_sort_flags) the image is written as NaN: a failure
  * shows without a read-back of the flags.
- * grads_to_zero (may be NULL): the [n*12] accumulator that a dsx_backward of this forward will
- * use.  The blend kernel, which leaves the memory system idle, zeroes it on the side, and that
- * dsx_backward is then called with grads_are_zero = 1 and needs no fill of its own. */
+ * grads_to_prepare (may be NULL; 16-byte aligned): the [n*12] accumulator that a dsx_backward of
+ * this forward will use.  The blend kernel, which leaves the memory system idle, prepares it on
+ * the side (the nine sums zeroed, each Gaussian's conic in the three spare places), and that
+ * dsx_backward is then called with grads_prepared = 1: it needs no fill of its own and its
+ * per-Gaussian kernel does not fetch the splat records for the conic. */
 int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
                        const void* order, int32_t* sorted_ids, int32_t* ranges, float* image,
                        float* final_T, int32_t* final_idx, void* workspace,
-                       size_t workspace_bytes, float* grads_to_zero, void* stream);
+                       size_t workspace_bytes, float* grads_to_prepare, void* stream);
 
 /* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316. grads is scratch [n*12];
- * grads_are_zero != 0 says that it holds zeros already (see dsx_forward_finish; true once: the
- * call leaves sums in it). */
+ * grads_prepared != 0 says that dsx_forward_finish has prepared it (true for one call: this
+ * one leaves sums in it). */
 int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                  const float* scales, const float* quats, const float* splats, const float* cov3d,
                  const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
                  const float* final_T, const int32_t* final_idx, const float* v_image,
-                 float* grads, int32_t grads_are_zero, float* v_mean3d, float* v_means2d,
+                 float* grads, int32_t grads_prepared, float* v_mean3d, float* v_means2d,
                  float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
                  float* v_cov3d, void* stream);
 
