@@ -115,10 +115,15 @@ class DsRasterizerFunction(torch.autograd.Function):
         ctx.save_for_backward(means_3d, scales, rotations, splats, cov_3d_precomp, radii, ranges, sorted_ids, final_T,
                               final_idx)
         ctx.mark_non_differentiable(radii)
+        # no zero tensors for outputs that take no gradient (autograd would fill an int32[N] of zeros
+        # for radii before every backward: a kernel launch in the middle of the step)
+        ctx.set_materialize_grads(False)
         return image, radii, final_T
 
     @staticmethod
     def backward(ctx, rendered_img_grad, _):
+        if rendered_img_grad is None:   # nothing flows into the image (gradients are not materialised)
+            return (None,) * 9
         means_3d, scales, rotations, splats, cov3d_precomp, radii, ranges, sorted_ids, final_T, final_idx = \
             ctx.saved_tensors
         ext = _native.load_torch_ext()
