@@ -973,7 +973,7 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     __shared__ uint4 s_rec[kProjBlock];
     __shared__ uint32_t wave_tot[kProjBlock / DSX_WAVE];
     __shared__ uint32_t s_mark[kEmitWindows * kProjBlock];
-    __shared__ uint32_t s_wave_max[kEmitWindows][kProjBlock / DSX_WAVE];
+    __shared__ __attribute__((aligned(16))) uint32_t s_wave_max[kEmitWindows][kProjBlock / DSX_WAVE];
     static_assert(kProjBlock == 4 * DSX_WAVE, "four wavefronts per workgroup");
 
     const int tid = threadIdx.x;
@@ -1094,12 +1094,12 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
 #pragma unroll
             for(int wdw = 0; wdw < kEmitWindows; ++wdw)
             {
-                uint32_t mine = before;
-                for(int w = 0; w < wave; ++w)
-                    mine = max(mine, s_wave_max[wdw][w]);
+                // the four wavefronts' maxima in one 16-byte read; the earlier wavefronts' count for this one
+                static_assert(kProjBlock / DSX_WAVE == 4, "four wavefronts per emission workgroup");
+                const uint4 wm = *reinterpret_cast<const uint4*>(s_wave_max[wdw]);
+                const uint32_t mine = max(max(before, wave > 0 ? wm.x : 0u), max(wave > 1 ? wm.y : 0u, wave > 2 ? wm.z : 0u));
                 const uint32_t owner = max(m[wdw], mine) - 1u; // every output has an owner: never 0 - 1
-                before = max(before, max(max(s_wave_max[wdw][0], s_wave_max[wdw][1]),
-                                         max(s_wave_max[wdw][2], s_wave_max[wdw][3])));
+                before = max(before, max(max(wm.x, wm.y), max(wm.z, wm.w)));
                 const uint32_t j = j0 + wdw * kProjBlock + tid;
                 if(j < jb)
                 {
