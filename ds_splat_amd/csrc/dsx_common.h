@@ -279,6 +279,24 @@ __device__ __forceinline__ int lane_id()
     return __lane_id();
 }
 
+// Sum of the first `wave` entries of a 16-byte aligned LDS array of kWaves per-wavefront totals
+// (kWaves a multiple of four): 16-byte reads and selects on the wavefront's index.  A loop
+// `for(w = 0; w < wave; ++w)` compiles to dependent 4-byte reads under an exec mask.
+template <int kWaves>
+__device__ __forceinline__ uint32_t sum_of_waves_before(const uint32_t* totals, int wave)
+{
+    static_assert(kWaves % 4 == 0, "whole 16-byte words");
+    uint32_t s = 0;
+#pragma unroll
+    for(int q = 0; q < kWaves / 4; ++q)
+    {
+        const uint4 v = reinterpret_cast<const uint4*>(totals)[q];
+        s += (4 * q < wave ? v.x : 0u) + (4 * q + 1 < wave ? v.y : 0u) + (4 * q + 2 < wave ? v.z : 0u) +
+             (4 * q + 3 < wave ? v.w : 0u);
+    }
+    return s;
+}
+
 // cov3D = (R S)(R S)^T from scale and (w,x,y,z) quaternion; cpp/rasterizer_kernels.cu:615-659
 __device__ __forceinline__ void cov3d_from_scale_rot(const float* sc, float4 q, float mod, float* out)
 {

@@ -87,7 +87,7 @@ constexpr int kScanItems = 4;
 
 __global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* data, int64_t count, uint32_t* total)
 {
-    __shared__ uint32_t wave_tot[kScanThreads / DSX_WAVE];
+    __shared__ __attribute__((aligned(16))) uint32_t wave_tot[kScanThreads / DSX_WAVE];
     __shared__ uint32_t carry_s;
     __shared__ unsigned long long total64; // the true sum: the 32-bit prefixes wrap silently, the total must not
     const int tid = threadIdx.x;
@@ -116,9 +116,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_u32_kernel(uint32_t* data, 
         if(lane == 63)
             wave_tot[wave] = incl;
         __syncthreads();
-        uint32_t wave_prefix = 0;
-        for(int w = 0; w < wave; ++w)
-            wave_prefix += wave_tot[w];
+        const uint32_t wave_prefix = sum_of_waves_before<kScanThreads / DSX_WAVE>(wave_tot, wave);
         uint32_t run = carry_s + wave_prefix + incl - sum;
 #pragma unroll
         for(int j = 0; j < kScanItems; ++j)

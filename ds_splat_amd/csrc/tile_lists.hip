@@ -214,8 +214,8 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     __shared__ uint16_t s_whist[kSort32Waves][kBins32];
     __shared__ uint32_t s_digit_start[kBins32];
     __shared__ uint32_t s_gbase[kBins32];
-    __shared__ uint32_t s_wave_tot[kBins32 / DSX_WAVE];
-    __shared__ uint32_t s_hist_tot[kBins32 / DSX_WAVE];
+    __shared__ __attribute__((aligned(16))) uint32_t s_wave_tot[kBins32 / DSX_WAVE];
+    __shared__ __attribute__((aligned(16))) uint32_t s_hist_tot[kBins32 / DSX_WAVE];
     __shared__ uint32_t s_tile;
 
     const int tid = threadIdx.x;
@@ -305,12 +305,13 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     __syncthreads();
     if(digit_thread)
     {
-        uint32_t prefix = 0, hprefix = 0;
-        for(int w = 0; w < wave; ++w)
-        {
-            prefix += s_wave_tot[w];
-            hprefix += s_hist_tot[w];
-        }
+        // totals of the digit wavefronts before this one: two 16-byte reads and selects (a loop over
+        // them compiles to dependent 4-byte reads under an exec mask, on every tile's critical path)
+        static_assert(kBins32 / DSX_WAVE == 4, "four digit wavefronts");
+        const uint4 wt = *reinterpret_cast<const uint4*>(s_wave_tot);
+        const uint4 ht = *reinterpret_cast<const uint4*>(s_hist_tot);
+        const uint32_t prefix = (wave > 0 ? wt.x : 0u) + (wave > 1 ? wt.y : 0u) + (wave > 2 ? wt.z : 0u);
+        const uint32_t hprefix = (wave > 0 ? ht.x : 0u) + (wave > 1 ? ht.y : 0u) + (wave > 2 ? ht.z : 0u);
         s_digit_start[tid] = prefix + s_gbase[tid];
         hist_excl += hprefix;
     }
@@ -691,7 +692,7 @@ __global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(int32_t* gri
 {
     extern __shared__ int32_t s_cells[];
     __shared__ uint32_t hist[kMaxPasses32 * kBins32];
-    __shared__ uint32_t wave_tot[kCoverThreads / DSX_WAVE];
+    __shared__ __attribute__((aligned(16))) uint32_t wave_tot[kCoverThreads / DSX_WAVE];
     __shared__ uint32_t s_carry;
     __shared__ int s_last;
     const int tid = threadIdx.x;
@@ -784,9 +785,7 @@ __global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(int32_t* gri
         if(lane == 63)
             wave_tot[wave] = incl;
         __syncthreads();
-        uint32_t prefix = s_carry;
-        for(int w = 0; w < wave; ++w)
-            prefix += wave_tot[w];
+        const uint32_t prefix = s_carry + sum_of_waves_before<kCoverThreads / DSX_WAVE>(wave_tot, wave);
         if(t < tiles)
             ranges[t] = (int32_t)(prefix + incl - cnt);
         __syncthreads();
@@ -971,7 +970,7 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     // per Gaussian of the block: x = first output, y = slot of the rectangle's first tile (0 for
     // negative depths), z = width (0 marks a negative depth: every pair goes to slot 0), w = id
     __shared__ uint4 s_rec[kProjBlock];
-    __shared__ uint32_t wave_tot[kProjBlock / DSX_WAVE];
+    __shared__ __attribute__((aligned(16))) uint32_t wave_tot[kProjBlock / DSX_WAVE];
     __shared__ uint32_t s_mark[kEmitWindows * kProjBlock];
     __shared__ __attribute__((aligned(16))) uint32_t s_wave_max[kEmitWindows][kProjBlock / DSX_WAVE];
     static_assert(kProjBlock == 4 * DSX_WAVE, "four wavefronts per workgroup");
@@ -1038,9 +1037,7 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
         if(lane == 63)
             wave_tot[wave] = incl;
         __syncthreads();
-        uint32_t prefix = 0;
-        for(int w = 0; w < wave; ++w)
-            prefix += wave_tot[w];
+        const uint32_t prefix = sum_of_waves_before<kProjBlock / DSX_WAVE>(wave_tot, wave);
         rec.x = prefix + incl - count;
         s_off[tid] = rec.x;
         s_rec[tid] = rec;
