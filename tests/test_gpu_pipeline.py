@@ -262,6 +262,33 @@ def test_api_precomputed_colors_and_cov3d(oracle):
     assert (radii_a == radii_b).all() and torch.equal(img_a, img_b)
 
 
+def test_api_backward_with_precomputed_inputs():
+    """Gradients on the optional-input paths: cov3D_precomp takes v_cov3d (and the backward reads the
+    covariances that were passed in, not rebuilt ones), colors_precomp takes the colour sums; the
+    other gradients equal those of the scales + rotations + SH run, which the oracle tests pin."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg0", n=5000, width=128, height=96, sh_degree=2)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    cam = stages.camera_from_scene(sc, DEV)
+    _, st = stages.forward(cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
+    o = stages.backward(cam, st, 16, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["v_image"])
+    torch.cuda.synchronize()
+    close = lambda a, b: torch.allclose(a, b.reshape(a.shape), rtol=1e-3, atol=1e-4 * max(1.0, float(b.abs().max())))
+
+    cov = st.cov3d.clone().requires_grad_(True)
+    _, _, leaves = api_run(sc, 2.0, cov3d=cov)
+    assert float(o["v_cov3d"].abs().max()) > 0 and close(cov.grad, o["v_cov3d"])
+    assert close(leaves["means"].grad, o["v_mean3d"]) and close(leaves["shs"].grad, o["v_shs"])
+    assert close(leaves["opac"].grad, o["v_opacity"])
+    assert leaves["scales"].grad is None and leaves["rots"].grad is None
+
+    cols = st.splats[:, 8:11].clone().requires_grad_(True)      # the colours the SH run blended with
+    image_c, _, leaves = api_run(sc, 2.0, colors=cols)
+    assert float(o["v_colors"].abs().max()) > 0 and close(cols.grad, o["v_colors"])
+    assert close(leaves["means"].grad, o["v_mean3d"]) and close(leaves["scales"].grad, o["v_scale"])
+    assert close(leaves["rots"].grad, o["v_quat"]) and leaves["shs"].grad is None
+
+
 def test_forward_core_raw_pointer_entry(oracle):
     """dsx_forward_core: device pointers in, image out (the reference's torch-free entry)."""
     import ctypes as C
