@@ -68,6 +68,20 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.dsx_depth_order(None, 10, None, 0, None) == -1
     assert lib.dsx_sort_flags(-1, 0, 16, 16, None, None, None, None) == -1
     assert lib.dsx_sort_flags(10, 10, 16, 16, None, None, None, None) == 0
+    # with a well-formed camera (its pointers are only compared with null before these checks fail)
+    import ctypes as C
+    cam = _native.Camera(64, 64, 0.5, 0.5, 1.0, 3, 3, 8, 8, 8, 8)
+    ref = C.byref(cam)
+    fake = 16   # any non-null address: nothing is launched
+    # the per-Gaussian backward needs the stored covariances or scales + rotations to rebuild them
+    assert lib.dsx_gaussian_bwd(ref, 10, 16, fake, None, None, fake, None, fake, fake, *([None] * 8), None) == -1
+    # ... and takes either with every output absent (n = 0: nothing to do)
+    assert lib.dsx_gaussian_bwd(ref, 0, 16, fake, None, None, fake, None, fake, fake, *([None] * 8), None) == 0
+    assert lib.dsx_gaussian_bwd(ref, 10, 17, fake, fake, fake, fake, None, fake, fake, *([None] * 8), None) == -1
+    # the forward's first half wants a place for K; the backward its saved tensors
+    assert lib.dsx_forward_project(ref, 10, *([fake] * 7), fake, fake, None, fake, fake, 1 << 20, None, None) == -1
+    assert lib.dsx_backward(ref, 10, 16, fake, fake, fake, fake, None, fake, None, fake, fake, fake, fake, fake, 0,
+                            *([None] * 8), None) == -1
 
 
 def test_python_api_surface():
