@@ -92,8 +92,10 @@ def roofline_entry(name, avg, lps, bound, work, traffic):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # defaults long enough for the clocks to settle (0.15 s of GPU work): with 3 + 20 steps the compute-bound
+    # kernels are still getting faster from launch to launch and the step reads 3 % longer
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
