@@ -414,6 +414,68 @@ def test_full_size_properties_cfg2():
         assert (o[key][radii <= 0] == 0).all()
 
 
+def test_full_size_properties_cfg4_heavy_overlap():
+    """The heavy-overlap shape at full size (1 M large Gaussians, 1080p, K = 858 M pairs: too many for
+    the 64-bit route's buffers and for the CPU oracle in a test): what the lists must satisfy
+    whatever their size.  K equals the sum of the tile counts; every Gaussian appears exactly
+    tiles_touched times; the ranges partition [0, K); inside a tile the pairs are ordered by
+    (depth bits, Gaussian index); every pair of a tile's list covers that tile; the image of an
+    all-white scene telescopes to 1 - final_T; forward and backward outputs are finite."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg4")
+    n = sc["n"]
+    cam = stages.camera_from_scene(sc, DEV)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    image, st = stages.forward(cam, t["means_3d"], t["scales"], t["rotations"], t["opacities"], t["shs"],
+                               prepare_grads=True)
+    torch.cuda.synchronize()
+    k = st.num_keys
+    tiles = st.splats[:, 11].view(torch.int32).to(torch.int64)
+    tiles[-1] = 0                                                    # the last Gaussian never emits
+    assert k == int(tiles.sum().item()) and k > 500_000_000
+    ids = st.sorted_ids.to(torch.int64)
+    assert int(ids.min()) >= 0 and int(ids.max()) < n
+    assert torch.equal(torch.bincount(ids, minlength=n), tiles)
+    r = st.ranges.to(torch.int64)
+    assert int(r[0]) == 0 and int(r[-1]) == k and bool((r[1:] >= r[:-1]).all())
+    # (tile, depth bits) never decreases along the whole array; equal keys keep ascending indices
+    tile_of = torch.repeat_interleave(torch.arange(cam.num_tiles, device=DEV), r[1:] - r[:-1])
+    assert tile_of.numel() == k
+    depth_bits = st.splats[:, 2].view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    key = (tile_of << 32) | depth_bits[ids]
+    assert bool((key[1:] >= key[:-1]).all())
+    same = key[1:] == key[:-1]
+    assert bool((ids[1:][same] > ids[:-1][same]).all())
+    del key, same
+    # each pair's tile lies inside its Gaussian's rectangle (recomputed from centre and radius as the
+    # reference does: truncation, +1 on the upper bound, clamped to the grid)
+    ntx, nty = (cam.width + 15) // 16, (cam.height + 15) // 16
+    cx, cy, d = st.splats[:, 0] / 16, st.splats[:, 1] / 16, st.radii.to(torch.float32) / 16
+    sx = (cx - d).to(torch.int32).clamp(0, ntx)          # cpp/rasterizer_kernels.cu:239-247
+    ex = (cx + d + 1).to(torch.int32).clamp(0, ntx)
+    sy = (cy - d).to(torch.int32).clamp(0, nty)
+    ey = (cy + d + 1).to(torch.int32).clamp(0, nty)
+    assert torch.equal(((ex - sx) * (ey - sy)).to(torch.int64)[:-1] * (st.radii[:-1] > 0), tiles[:-1])
+    step = 997                                                       # a sample of the pairs
+    tt, gg = tile_of[::step], ids[::step]
+    tx, ty = (tt % ntx).to(torch.int32), (tt // ntx).to(torch.int32)
+    assert bool(((tx >= sx[gg]) & (tx < ex[gg]) & (ty >= sy[gg]) & (ty < ey[gg])).all())
+    del tile_of, ids, tt, gg
+    assert bool(torch.isfinite(image).all()) and bool((image >= 0).all())
+    assert bool((st.final_T <= 1).all()) and bool((st.final_T >= 9.9e-5).all())
+    white = st.splats.clone()
+    white[:, 8:11] = 1.0
+    img_w, T_w, _ = stages.blend_fwd(cam, st.ranges, st.sorted_ids, white)
+    assert torch.allclose(img_w, (1 - T_w).unsqueeze(-1).expand(-1, -1, 3), rtol=0, atol=2e-5)
+    assert torch.equal(T_w, st.final_T)
+    o = stages.backward(cam, st, 16, t["means_3d"], t["scales"], t["rotations"], t["v_image"])
+    torch.cuda.synchronize()
+    for name in ("v_mean3d", "v_means2d", "v_shs", "v_opacity", "v_scale", "v_quat"):
+        assert bool(torch.isfinite(o[name]).all()), name
+        assert bool((o[name][st.radii <= 0] == 0).all()), name
+    assert float(o["v_shs"].abs().max()) > 0
+
+
 def test_full_size_cfg2_against_the_openmp_oracle():
     """The headline shape itself (3M Gaussians, 1920x1080, SH3) against the oracle's OpenMP build
     (same source as the serial oracle, loops over Gaussians and tiles in parallel): integers bit
