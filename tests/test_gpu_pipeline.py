@@ -476,14 +476,16 @@ def test_full_size_properties_cfg4_heavy_overlap():
     assert float(o["v_shs"].abs().max()) > 0
 
 
-def test_full_size_cfg2_against_the_openmp_oracle():
-    """The headline shape itself (3M Gaussians, 1920x1080, SH3) against the oracle's OpenMP build
-    (same source as the serial oracle, loops over Gaussians and tiles in parallel): integers bit
-    for bit, image rtol 1e-4 / atol 1e-5 and gradients rtol 1e-3 away from threshold decisions."""
+@pytest.mark.parametrize("workload", ["cfg1", "cfg2"])
+def test_full_size_against_the_openmp_oracle(workload):
+    """The two forward+backward shapes at full size (500 K and the headline 3 M Gaussians, 1920x1080,
+    SH3) against the oracle's OpenMP build (same source as the serial oracle, loops over
+    Gaussians and tiles in parallel): integers bit for bit, image rtol 1e-4 / atol 1e-5 and
+    gradients rtol 1e-3 away from threshold decisions."""
     from oracle.binding import Oracle
     from ds_splat_amd import stages
     omp = Oracle(omp=True)
-    sc = make_scene("cfg2")
+    sc = make_scene(workload)
     n = sc["n"]
     image, radii, leaves = api_run(sc)
     img_o, radii_o, S, B = oracle_run(omp, sc)
