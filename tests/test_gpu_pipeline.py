@@ -476,12 +476,13 @@ def test_full_size_properties_cfg4_heavy_overlap():
     assert float(o["v_shs"].abs().max()) > 0
 
 
-@pytest.mark.parametrize("workload", ["cfg1", "cfg2"])
+@pytest.mark.parametrize("workload", ["cfg1", "cfg2", "cfg4"])
 def test_full_size_against_the_openmp_oracle(workload):
-    """The two forward+backward shapes at full size (500 K and the headline 3 M Gaussians, 1920x1080,
-    SH3) against the oracle's OpenMP build (same source as the serial oracle, loops over
-    Gaussians and tiles in parallel): integers bit for bit, image rtol 1e-4 / atol 1e-5 and
-    gradients rtol 1e-3 away from threshold decisions."""
+    """The three forward+backward shapes at full size (500 K Gaussians, the headline 3 M, and the
+    heavy-overlap 1 M with its 858 M pairs; 1920x1080, SH3) against the oracle's OpenMP build
+    (same source as the serial oracle, loops over Gaussians and tiles in parallel): integers,
+    every sorted id included, bit for bit, image rtol 1e-4 / atol 1e-5 and gradients rtol 1e-3
+    away from threshold decisions."""
     from oracle.binding import Oracle
     from ds_splat_amd import stages
     omp = Oracle(omp=True)
