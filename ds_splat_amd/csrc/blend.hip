@@ -323,43 +323,42 @@ __device__ __forceinline__ float dpp_move(float v)
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
 }
 
-// Sums eight per-lane values over the wavefront as a reduce-scatter: in each of the first
-// three steps a lane keeps half of its values and hands the other half to a partner (inside the
-// quad twice, then to the quad four lanes away), so one value per lane is left for the steps
-// across the row, the rows and the halves.  Lanes 56..63 end up with the eight totals: lane l
-// holds the total of v[4*(l&1) + 2*((l>>1)&1) + ((l>>2)&1)].
+// Sums eight per-lane values over the wavefront as a reduce-scatter.  The first two steps use the
+// lane-swap instructions, which halve two registers into one at a time: across the halves of
+// the wavefront (8 -> 4 registers), across neighbouring rows of 16 (4 -> 2); the third step
+// trades between neighbouring lanes (2 -> 1), and three adds over the lanes that differ in bits
+// 1, 2 and 3 finish the rows.  18 instructions where a select-and-add scheme over all three
+// steps took 32.  Every lane ends up with a total: the one of
+// v[4*(lane&1) + 2*((lane>>4)&1) + (lane>>5)].
+__device__ __forceinline__ float pair_sum_halves(float a, float b)
+{
+    // lanes 0..31 get a summed over the two halves, lanes 32..63 get b
+    const dsx_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r.x) + __uint_as_float(r.y);
+}
+
+__device__ __forceinline__ float pair_sum_rows(float a, float b)
+{
+    // even rows get a summed over each pair of neighbouring rows, odd rows get b
+    const dsx_u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r.x) + __uint_as_float(r.y);
+}
+
 __device__ __forceinline__ float wave_sum8_scatter(const float (&v)[8], int lane)
 {
-    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
-    float r[4];
-#pragma unroll
-    for(int i = 0; i < 4; ++i)
-    {
-        const float keep = b0 ? v[4 + i] : v[i];
-        const float send = b0 ? v[i] : v[4 + i];
-        r[i] = keep + dpp_move<0xB1>(send); // quad_perm [1,0,3,2]
-    }
-    float q[2];
-#pragma unroll
-    for(int i = 0; i < 2; ++i)
-    {
-        const float keep = b1 ? r[2 + i] : r[i];
-        const float send = b1 ? r[i] : r[2 + i];
-        q[i] = keep + dpp_move<0x4E>(send); // quad_perm [2,3,0,1]
-    }
-    const float keep = b2 ? q[1] : q[0];
-    const float send = b2 ? q[0] : q[1];
-    // partner = lane ^ 4: banks 0 and 2 of a row read four lanes up, banks 1 and 3 four lanes down
-    int got = __builtin_amdgcn_update_dpp(0, __float_as_int(send), 0x104, 0xf, 0x5, false); // row_shl:4
-    got = __builtin_amdgcn_update_dpp(got, __float_as_int(send), 0x114, 0xf, 0xa, false);   // row_shr:4
-    float o = keep + __int_as_float(got);
-    o += dpp_move<0x128>(o); // row_ror:8 -> the whole row of 16
-    // across rows the lanes must keep their position inside the row, so the row broadcasts of
-    // the single-value reduction cannot be used: swap rows, then halves
-    const dsx_u32x2 r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(o), __float_as_uint(o), false, false);
-    o = __uint_as_float(r16.x) + __uint_as_float(r16.y);
-    const dsx_u32x2 r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(o), __float_as_uint(o), false, false);
-    o = __uint_as_float(r32.x) + __uint_as_float(r32.y);
+    const float s0 = pair_sum_halves(v[0], v[1]);
+    const float s1 = pair_sum_halves(v[2], v[3]);
+    const float s2 = pair_sum_halves(v[4], v[5]);
+    const float s3 = pair_sum_halves(v[6], v[7]);
+    const float t0 = pair_sum_rows(s0, s1); // v[2 * row parity + half]
+    const float t1 = pair_sum_rows(s2, s3); // v[4 + 2 * row parity + half]
+    const bool odd = lane & 1;
+    const float keep = odd ? t1 : t0;
+    const float send = odd ? t0 : t1;
+    float o = keep + dpp_move<0xB1>(send); // quad_perm [1,0,3,2]: the neighbour's share
+    o = dpp_add<0x4E, 0xf>(o);             // quad_perm [2,3,0,1]: lanes that differ in bit 1
+    o = dpp_add<0x124, 0xf>(o);            // row_ror:4 and
+    o = dpp_add<0x128, 0xf>(o);            // row_ror:8: lanes that differ in bits 2 and 3
     return o;
 }
 
@@ -522,15 +521,14 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             g[4] = -0.5f * B.y * S2;
             const float total = wave_sum8_scatter(g, lane);
             g_blue = wave_sum_to_lane63(g_blue);
-            // lane 63's blue total goes to lane 55 (row_shl:8: a lane reads the one eight up in its
-            // row), so that ONE atomic instruction carries all nine sums, each lane its own address
-            const float blue55 = dpp_move<0x108>(g_blue);
-            if(lane >= 55)
+            // ONE atomic instruction carries all nine sums, each lane its own address: the first
+            // two lanes of every row hold the eight totals of the reduce-scatter (every lane holds
+            // one), lane 63 the ninth
+            if((lane & 14) == 0 || lane == 63)
             {
-                // lane l >= 56 holds the total of g[4*(l&1) + 2*((l>>1)&1) + ((l>>2)&1)]
                 float* rec = grads + (int64_t)s_id[t] * DSX_GRAD_FLOATS;
-                const int slot = lane == 55 ? 8 : 4 * (lane & 1) + 2 * ((lane >> 1) & 1) + ((lane >> 2) & 1);
-                unsafeAtomicAdd(rec + slot, lane == 55 ? blue55 : total);
+                const int slot = lane == 63 ? 8 : 4 * (lane & 1) + 2 * ((lane >> 4) & 1) + (lane >> 5);
+                unsafeAtomicAdd(rec + slot, lane == 63 ? g_blue : total);
             }
         }
     }
