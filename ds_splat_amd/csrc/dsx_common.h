@@ -348,6 +348,26 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v)
     return v;
 }
 
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves only: four shifts
+// inside each row of 16 (lanes without a source add 0), then the row totals are broadcast into
+// the rows behind them.  (A shuffle goes through the LDS crossbar and takes a round trip per step.)
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ uint32_t dpp_add_u32(uint32_t v)
+{
+    return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kCtrl, kRowMask, 0xf, false);
+}
+
+__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t v)
+{
+    v = dpp_add_u32<0x111, 0xf>(v); // row_shr:1
+    v = dpp_add_u32<0x112, 0xf>(v); // row_shr:2
+    v = dpp_add_u32<0x114, 0xf>(v); // row_shr:4
+    v = dpp_add_u32<0x118, 0xf>(v); // row_shr:8
+    v = dpp_add_u32<0x142, 0xa>(v); // row_bcast:15 into rows 1 and 3
+    v = dpp_add_u32<0x143, 0xc>(v); // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 typedef float dsx_v4f __attribute__((ext_vector_type(4)));
 
 // streaming (non-temporal) 16-byte load / store: data that is touched once

@@ -12,16 +12,9 @@ namespace dsx
 // small wave/block primitives
 // ---------------------------------------------------------------------------------------
 
-__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t v, int lane)
+__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t v, int)
 {
-#pragma unroll
-    for(int o = 1; o < DSX_WAVE; o <<= 1)
-    {
-        const uint32_t t = __shfl_up(v, o, DSX_WAVE);
-        if(lane >= o)
-            v += t;
-    }
-    return v;
+    return wave_incl_scan_u32(v);
 }
 
 // lanes of the wavefront that hold the same (up to 9-bit) digit and are valid; call in uniform

@@ -43,16 +43,9 @@ static hipStream_t helper_stream()
     return streams[device];
 }
 
-__device__ __forceinline__ uint32_t wave_incl_scan32(uint32_t v, int lane)
+__device__ __forceinline__ uint32_t wave_incl_scan32(uint32_t v, int)
 {
-#pragma unroll
-    for(int o = 1; o < DSX_WAVE; o <<= 1)
-    {
-        const uint32_t t = __shfl_up(v, o, DSX_WAVE);
-        if(lane >= o)
-            v += t;
-    }
-    return v;
+    return wave_incl_scan_u32(v);
 }
 
 // inclusive max-scan over the 64 lanes with data-parallel-primitive moves only (values >= 0,
