@@ -102,7 +102,7 @@ def main():
     ap.add_argument("--verbose", action="store_true", help="per-kernel table on stderr")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic that scales HBM byte counters) and "
-                         "the library's streaming probe (read / write / copy rates that plain kernels reach here)")
+                         "the streaming probe (read / write / copy rates that plain kernels reach here)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding "
@@ -152,25 +152,26 @@ def main():
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
-        # what plain streaming kernels of this library's access shape reach on this device (1 GiB each)
-        lib = _native.load()
+        # what plain streaming kernels of this library's access shape reach on this device (1 GiB each):
+        # the probe library is measurement tooling, separate from libdsx.so
+        import ctypes as C
+        probe = C.CDLL(os.path.join(ROOT, "ds_splat_amd", "lib", "libdsx_probe.so"))
+        probe.dsxp_stream_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p,
+                                            C.POINTER(C.c_float)]
         stream = torch.cuda.current_stream().cuda_stream
         nbytes = src.numel() * 4
         mixed_bytes = 28 * 16 * 3_000_000   # 10 + 18 arrays of 3 M 16-byte elements: the backward's volume
         sizes = (nbytes, nbytes, nbytes, mixed_bytes, mixed_bytes // 2)
-        for mode in (0, 1, 2, 3, 4):
-            for _ in range(2):
-                _native.check(lib.dsx_stream_probe(src.data_ptr(), dst.data_ptr(), sizes[mode], mode, stream))
-        torch.cuda.synchronize()
-        _native.trace_enable(True)
-        _native.trace_read()
         reps = 5
+        times = []
         for mode in (0, 1, 2, 3, 4):
-            for _ in range(reps):
-                _native.check(lib.dsx_stream_probe(src.data_ptr(), dst.data_ptr(), sizes[mode], mode, stream))
-        torch.cuda.synchronize()
-        times = [ms for name, ms in _native.trace_read() if name == "stream_probe_kernel"]
-        _native.trace_enable(False)
+            for rep in range(2 + reps):
+                ms = C.c_float(0.0)
+                rc = probe.dsxp_stream_probe(src.data_ptr(), dst.data_ptr(), sizes[mode], mode, stream, C.byref(ms))
+                if rc != 0:
+                    raise RuntimeError("dsxp_stream_probe failed with %d" % rc)
+                if rep >= 2:
+                    times.append(float(ms.value))
         per_mode = [min(times[m * reps:(m + 1) * reps]) for m in range(5)]
         stream_ceiling = {"unit": "GB/s", "bytes": nbytes,
                           "read": round(nbytes / per_mode[0] / 1e6, 1), "write": round(nbytes / per_mode[1] / 1e6, 1),

@@ -78,7 +78,7 @@ class TraceEntry(C.Structure):
 
 SIGNATURES["dsx_trace_enable"] = (C.c_int, [C.c_int])
 SIGNATURES["dsx_trace_read"] = (C.c_int, [C.POINTER(TraceEntry), C.c_int])
-SIGNATURES["dsx_stream_probe"] = (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p])
+SIGNATURES["dsx_set_blend_pixels_per_lane"] = (C.c_int, [C.c_int])
 
 _lib = None
 

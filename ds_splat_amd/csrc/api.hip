@@ -597,82 +597,7 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     return rc;
 }
 
-namespace dsx
+extern "C" int dsx_set_blend_pixels_per_lane(int pixels)
 {
-typedef float probe_f4 __attribute__((ext_vector_type(4)));
-__global__ __launch_bounds__(256) void stream_probe_kernel(const probe_f4* __restrict__ src, probe_f4* __restrict__ dst,
-                                                           int64_t count, int mode, float* sink)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if(i >= count)
-        return;
-    if(mode == 1)
-    {
-        const probe_f4 v = {1.f, 2.f, 3.f, 4.f};
-        __builtin_nontemporal_store(v, dst + i);
-        return;
-    }
-    const probe_f4 v = __builtin_nontemporal_load(src + i);
-    if(mode == 2)
-        __builtin_nontemporal_store(v, dst + i);
-    else if(v.x + v.y + v.z + v.w == 12345.678f) // never true for the probe's data: keeps the load alive
-        *sink = 1.f;
-}
-
-// many streams per thread: kReads arrays read and kWrites arrays written, 16 bytes of each
-template <int kReads, int kWrites>
-__global__ __launch_bounds__(256) void stream_probe_mixed_kernel(const probe_f4* __restrict__ src,
-                                                                 probe_f4* __restrict__ dst, int64_t count)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if(i >= count)
-        return;
-    probe_f4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for(int r = 0; r < kReads; ++r)
-        acc += __builtin_nontemporal_load(src + r * count + i);
-#pragma unroll
-    for(int w = 0; w < kWrites; ++w)
-        __builtin_nontemporal_store(acc, dst + w * count + i);
-}
-} // namespace dsx
-
-extern "C" int dsx_stream_probe(const void* src, void* dst, size_t bytes, int mode, void* stream)
-{
-    if(mode < 0 || mode > 4 || (bytes & 15) != 0 || (mode != 1 && !src) || (mode != 0 && !dst))
-        return DSX_ERR_BAD_ARG;
-    if(mode == 0 && !dst)
-        dst = const_cast<void*>(src); // the sink is never written
-    int64_t count = (int64_t)(bytes / 16);
-    if(count == 0)
-        return DSX_OK;
-    if(count >= (1ll << 39))
-        return DSX_ERR_TOO_LARGE;
-    hipStream_t s = as_stream(stream);
-    if(mode >= 3)
-    {
-        // write-heavy mixes like the per-Gaussian backward's: 10 arrays read and 18 written (its
-        // volume per element), or 5 and 9 (closer to its number of arrays); `bytes` is all of it
-        count /= mode == 3 ? 28 : 14;
-        if(count == 0)
-            return DSX_OK;
-        const dim3 grid((unsigned)((count + 255) / 256));
-        DSX_TIMED("stream_probe_kernel", s);
-        if(mode == 3)
-            hipLaunchKernelGGL((dsx::stream_probe_mixed_kernel<10, 18>), grid, dim3(256), 0, s,
-                               static_cast<const dsx::probe_f4*>(src), static_cast<dsx::probe_f4*>(dst), count);
-        else
-            hipLaunchKernelGGL((dsx::stream_probe_mixed_kernel<5, 9>), grid, dim3(256), 0, s,
-                               static_cast<const dsx::probe_f4*>(src), static_cast<dsx::probe_f4*>(dst), count);
-        DSX_LAUNCH_CHECK();
-        return DSX_OK;
-    }
-    {
-        DSX_TIMED("stream_probe_kernel", s);
-        hipLaunchKernelGGL(dsx::stream_probe_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s,
-                           static_cast<const dsx::probe_f4*>(src), static_cast<dsx::probe_f4*>(dst), count, mode,
-                           static_cast<float*>(dst));
-    }
-    DSX_LAUNCH_CHECK();
-    return DSX_OK;
+    return set_blend_pixels_per_lane(pixels);
 }

@@ -3,6 +3,7 @@
 // one float array, so an entry costs two 128-bit and one 32-bit LDS broadcast read.
 #include "dsx_common.h"
 
+#include <atomic>
 #include <cstdlib>
 
 namespace dsx
@@ -74,17 +75,38 @@ __device__ __forceinline__ bool entry_reaches_tile(float mx, float my, float a, 
 // to occupy the chip (8 wavefronts on each of 1024 SIMDs), else 1 (four wavefronts per tile: more
 // instructions in all, but four times as many wavefronts).  Measured crossover (500 K Gaussians,
 // 640x480 to 1920x1080): about 5000 tiles for the forward, 1600 for the backward, whose
-// one-pixel form also quadruples the atomics.  DSX_BLEND_PIXELS_PER_LANE=1|4 in the environment
-// overrides the choice (tests run both forms).
+// one-pixel form also quadruples the atomics.  dsx_set_blend_pixels_per_lane(1 | 4) overrides the
+// choice for the whole process (tests run both forms); DSX_BLEND_PIXELS_PER_LANE=1|4 in the
+// environment gives the override's initial value and is read once.
+static std::atomic<int> g_forced_pixels_per_lane{-1}; // -1: not yet read from the environment, 0: automatic
+
+static int forced_pixels_per_lane()
+{
+    int v = g_forced_pixels_per_lane.load(std::memory_order_relaxed);
+    if(v >= 0)
+        return v;
+    v = 0;
+    if(const char* forced = getenv("DSX_BLEND_PIXELS_PER_LANE"))
+        if((forced[0] == '1' || forced[0] == '4') && forced[1] == 0)
+            v = forced[0] - '0';
+    int expected = -1;
+    g_forced_pixels_per_lane.compare_exchange_strong(expected, v, std::memory_order_relaxed);
+    return g_forced_pixels_per_lane.load(std::memory_order_relaxed);
+}
+
+int set_blend_pixels_per_lane(int pixels)
+{
+    if(pixels != 0 && pixels != 1 && pixels != 4)
+        return DSX_ERR_BAD_ARG;
+    g_forced_pixels_per_lane.store(pixels, std::memory_order_relaxed);
+    return DSX_OK;
+}
+
 static int blend_pixels_per_lane(int num_tiles, int four_from)
 {
-    if(const char* forced = getenv("DSX_BLEND_PIXELS_PER_LANE"))
-    {
-        if(forced[0] == '1' && forced[1] == 0)
-            return 1;
-        if(forced[0] == '4' && forced[1] == 0)
-            return 4;
-    }
+    const int forced = forced_pixels_per_lane();
+    if(forced != 0)
+        return forced;
     return num_tiles >= four_from ? 4 : 1;
 }
 constexpr int kFwdFourPixelsFrom = 5000; // tiles

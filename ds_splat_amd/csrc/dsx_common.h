@@ -259,6 +259,8 @@ int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const f
                         float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d,
                         hipStream_t stream, bool conic_in_grads = false);
 int launch_fill_u32(uint32_t* p, int64_t count, uint32_t value, hipStream_t stream);
+// 1 or 4: force that form of both blend kernels for the whole process; 0: choose by image size
+int set_blend_pixels_per_lane(int pixels);
 
 // Optional per-kernel timing (diagnostics for benchmarks): when switched on through
 // dsx_trace_enable(), every launch is bracketed by two events on the launch stream.

@@ -15,7 +15,6 @@ from dataclasses import dataclass
 import torch
 
 from . import _native
-from . import stages
 
 
 def _check_input(t, name):
@@ -177,15 +176,23 @@ class GaussianRasterizer(torch.nn.Module):
     @property
     def settings_for_cpp_code(self):
         # the reference transposes both matrices on every call (ds_splat/rasterizer.py:147-148);
-        # the result is kept here for as long as the settings' tensors are the same, unmodified ones
+        # the result is kept here for as long as the settings hold the same, unmodified tensors.
+        # The cache entry keeps the tensors themselves (compared with `is`: an address alone could
+        # be a new tensor in a freed one's place) and their version counters; tensors without one
+        # (created under torch.inference_mode) are transposed on every call.
         rs = self._settings
-        key = (id(rs), id(rs.viewmatrix), rs.viewmatrix._version, id(rs.projmatrix), rs.projmatrix._version,
-               id(rs.bg), id(rs.campos), rs.image_height, rs.image_width, rs.tanfovx, rs.tanfovy, rs.scale_modifier,
-               rs.sh_degree, rs.max_sh_degree)
-        if self._native_cache is not None and self._native_cache[0] == key:
-            return self._native_cache[1]
+        try:
+            versions = (rs.viewmatrix._version, rs.projmatrix._version)
+        except RuntimeError:
+            return self._build_native_settings()
+        scalars = (rs.image_height, rs.image_width, rs.tanfovx, rs.tanfovy, rs.scale_modifier, rs.sh_degree,
+                   rs.max_sh_degree, rs.prefiltered, rs.debug)
+        c = self._native_cache
+        if (c is not None and c[0] is rs and c[1] is rs.viewmatrix and c[2] is rs.projmatrix and c[3] is rs.bg
+                and c[4] is rs.campos and c[5] == versions and c[6] == scalars):
+            return c[7]
         s = self._build_native_settings()
-        self._native_cache = (key, s)
+        self._native_cache = (rs, rs.viewmatrix, rs.projmatrix, rs.bg, rs.campos, versions, scalars, s)
         return s
 
     def _build_native_settings(self):

@@ -5,10 +5,14 @@
  * is marked "host".  `stream` is a hipStream_t passed as void* (NULL = the null stream).
  * The library allocates nothing on the device: outputs and workspace are the caller's.
  * All functions return 0 on success or a negative dsx_status; dsx_error_string() explains it.
- * Functions are re-entrant: the compute path keeps no global mutable state, so different
- * streams / devices may be driven concurrently by different host threads (each call uses the
- * current HIP device).  The one exception is the optional per-kernel timing trace
- * (dsx_trace_enable / dsx_trace_read), a process-wide list behind a mutex, off by default.
+ * Functions are re-entrant: different streams / devices may be driven concurrently by different
+ * host threads (each call uses the current HIP device).  Process-wide state, all of it behind
+ * locks or atomics: (1) the optional per-kernel timing trace (dsx_trace_enable / dsx_trace_read),
+ * a list behind a mutex, off by default; (2) one helper stream per device, created on first use
+ * and kept until the process ends: dsx_depth_order / dsx_forward_project fork onto it and join
+ * before they return, so that the tile counting runs beside the depth sort — callers on
+ * different streams of one device share it and their forked parts serialise there; (3) the
+ * blend-kernel form override of dsx_set_blend_pixels_per_lane.
  *
  * What each entry point replaces in the reference (deepsense-ai/ds-splat) is cited as
  * file:line next to it.  Matrices are row-major, math convention (translation in elements
@@ -268,13 +272,12 @@ typedef struct dsx_trace_entry
 int dsx_trace_enable(int on);
 int dsx_trace_read(dsx_trace_entry* out /* host */, int max_entries);
 
-/* Calibration of the HBM roofline: one launch that streams `bytes` (a multiple of 16) with one
- * 16-byte element per thread, the access shape of the per-Gaussian kernels.  mode 0 reads src,
- * 1 writes dst, 2 copies src to dst; modes 3 and 4 move `bytes` in all as 10 arrays read and 18
- * written per thread (src holds 10/28 of `bytes`, dst 18/28), respectively 5 and 9: write-heavy
- * mixes of many streams like the per-Gaussian backward's.  Traced as "stream_probe_kernel".
- * No counterpart in the reference. */
-int dsx_stream_probe(const void* src, void* dst, size_t bytes, int mode, void* stream);
+/* The two blend kernels exist in two forms: one wavefront per tile with four pixels per lane
+ * (images with enough tiles to fill the chip) and four wavefronts per tile with one pixel per
+ * lane.  The library picks by tile count; this forces one form for the whole process (pixels =
+ * 1 or 4) or returns the choice to the library (0).  Results of the forward are bit-identical in
+ * both forms.  For tests, which run both forms at every size.  No counterpart in the reference. */
+int dsx_set_blend_pixels_per_lane(int pixels);
 
 #ifdef __cplusplus
 }

@@ -164,14 +164,14 @@ class Oracle:
         n = means2d.shape[0]
         out = dict(v_xy=np.empty((n, 2), np.float32), v_conic=np.empty((n, 3), np.float32),
                    v_rgb=np.empty((n, 3), np.float32), v_opacity=np.empty((n, 1), np.float32),
-                   g_margin=np.empty(n, np.float32))
+                   g_margin=np.empty(n, np.float32), abs_sums=np.empty((n, 9), np.float32))
         cnt = Counters()
-        self.lib.dsxo_blend_bwd(C.byref(s), C.c_int64(n), _i(np.ascontiguousarray(ranges, np.int32)),
+        self.lib.dsxo_blend_bwd_ex(C.byref(s), C.c_int64(n), _i(np.ascontiguousarray(ranges, np.int32)),
                                 _i(np.ascontiguousarray(sorted_ids, np.int32)), _f(_c32(means2d)), _f(_c32(conic)),
                                 _f(_c32(rgb)), _f(_c32(opacities).reshape(-1)), _f(_c32(final_T)),
                                 _i(np.ascontiguousarray(final_idx, np.int32)), _f(_c32(v_out)), _f(_c32(v_out_alpha)),
                                 _f(out["v_xy"]), _f(out["v_conic"]), _f(out["v_rgb"]), _f(out["v_opacity"]),
-                                _f(out["g_margin"]), C.byref(cnt))
+                                _f(out["g_margin"]), C.byref(cnt), _f(out["abs_sums"]))
         out["counters"] = cnt
         return out
 
@@ -240,12 +240,12 @@ class Oracle:
                  v_shs=np.empty((n, num_bases, 3), np.float32), v_colors=np.empty((n, 3), np.float32),
                  v_opacity=np.empty((n, 1), np.float32), v_scale=np.empty((n, 3), np.float32),
                  v_quat=np.empty((n, 4), np.float32), v_cov3d=np.empty((n, 6), np.float32),
-                 g_margin=np.empty(n, np.float32))
-        self.lib.dsxo_backward(st, C.byref(s), C.c_int64(n), C.c_int32(num_bases), _f(_c32(means3d)),
+                 g_margin=np.empty(n, np.float32), abs_sums=np.empty((n, 9), np.float32))
+        self.lib.dsxo_backward_ex(st, C.byref(s), C.c_int64(n), C.c_int32(num_bases), _f(_c32(means3d)),
                                _f(_c32(scales)), _f(_c32(quats)), _f(_c32(opacities).reshape(-1)),
                                _f(_c32(v_image)), _f(o["v_mean3d"]), _f(o["v_means2d"]), _f(o["v_shs"]),
                                _f(o["v_colors"]), _f(o["v_opacity"]), _f(o["v_scale"]), _f(o["v_quat"]),
-                               _f(o["v_cov3d"]), _f(o["g_margin"]))
+                               _f(o["v_cov3d"]), _f(o["g_margin"]), _f(o["abs_sums"]))
         cnt = Counters()
         self.lib.dsxo_state_get(st, *([None] * 12), C.byref(cnt))
         o["counters"] = cnt
@@ -254,6 +254,46 @@ class Oracle:
     def free(self, st):
         if st is not None:
             self.lib.dsxo_state_free(st)
+
+    def gradient_bounds(self, s, num_bases, means3d, scales, quats, conic, cov3d, radii, abs_sums, rel=1e-3,
+                        floor=1e-7):
+        """Per-element tolerances for the gradients of a backward whose nine screen-space sums were
+        accumulated in another order than the oracle's (float atomics).
+
+        abs_sums[N,9] (from blend_bwd / backward) is, per Gaussian, the sum of the absolute values
+        of the terms of each screen-space sum: a reordered float summation may be off by
+        ``rel * abs_sums + floor`` there.  The outputs of the per-Gaussian backward are linear in
+        those sums; the Jacobian's columns come from running the oracle's projection backward on
+        unit inputs, and the bound of an output element is own = sum_k |J_k| * (rel * abs_sums_k + floor)
+        plus, for the outputs that come out of chains of small matrix products (v_mean3d, v_scale,
+        v_quat, v_cov3d, v_shs), the largest `own` of the same Gaussian's row of that output: an
+        element that is small because its chain cancels carries rounding errors of the size of its
+        neighbours (measured on the GPU against this oracle: up to 4e-3 of `own`, never above 2e-5
+        of the row's largest).  Nothing is scaled by a whole tensor.
+        Returns a dict with the keys of backward()."""
+        n = means3d.shape[0]
+        eps = (rel * np.asarray(abs_sums, np.float64) + floor)          # x y | a b c | opacity | r g b
+        out = dict(v_means2d=np.concatenate([eps[:, 0:2], np.zeros((n, 1))], axis=1), v_opacity=eps[:, 5:6].copy(),
+                   v_colors=eps[:, 6:9].copy())
+        ones = np.ones((n, 3), np.float32)
+        Y = np.abs(self.sh_bwd(s, num_bases, means3d, ones)[:, :, 0].astype(np.float64))   # |Y_b| per Gaussian
+        with_row_max = lambda own: own + own.reshape(n, -1).max(axis=1).reshape((n,) + (1,) * (own.ndim - 1))
+        out["v_shs"] = with_row_max(Y[:, :, None] * eps[:, None, 6:9])
+        acc = None
+        for k in range(5):
+            v_xy = np.zeros((n, 2), np.float32)
+            v_conic = np.zeros((n, 3), np.float32)
+            if k < 2:
+                v_xy[:, k] = 1.0
+            else:
+                v_conic[:, k - 2] = 1.0
+            J = self.project_bwd(s, means3d, scales, quats, conic, cov3d, radii, v_xy, v_conic)
+            if acc is None:
+                acc = {key: np.zeros(J[key].shape, np.float64) for key in ("v_mean3d", "v_scale", "v_quat", "v_cov3d")}
+            for key in acc:
+                acc[key] += np.abs(J[key].astype(np.float64)) * eps[:, k:k + 1]
+        out.update({key: with_row_max(own) for key, own in acc.items()})
+        return out
 
     # ---- float64 instances -----------------------------------------------------------
     def blend_loss_f64(self, width, height, ranges, sorted_ids, xy, conic, rgb, opac, weights, alpha_clamp,

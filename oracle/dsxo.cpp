@@ -589,9 +589,22 @@ extern "C" void dsxo_blend_bwd(const dsxo_settings* s, int64_t n, const int32_t*
                                const float* v_out_alpha, float* v_xy, float* v_conic, float* v_rgb, float* v_opacity,
                                float* g_margin, dsxo_counters* counters)
 {
+    dsxo_blend_bwd_ex(s, n, ranges, sorted_ids, means2d, conic, rgb, opacities, final_T, final_idx, v_out, v_out_alpha,
+                      v_xy, v_conic, v_rgb, v_opacity, g_margin, counters, nullptr);
+}
+
+extern "C" void dsxo_blend_bwd_ex(const dsxo_settings* s, int64_t n, const int32_t* ranges, const int32_t* sorted_ids,
+                                  const float* means2d, const float* conic, const float* rgb, const float* opacities,
+                                  const float* final_T, const int32_t* final_idx, const float* v_out,
+                                  const float* v_out_alpha, float* v_xy, float* v_conic, float* v_rgb,
+                                  float* v_opacity, float* g_margin, dsxo_counters* counters, float* abs_sums)
+{
     const int W = s->image_width, H = s->image_height;
     const int ntx = tiles_x(s), nty = tiles_y(s);
     std::vector<double> acc((size_t)n * 9, 0.0);
+    /* sums of the absolute values of the elementary terms of every accumulation: the scale
+     * against which a differently ordered float summation may be judged */
+    std::vector<double> acc_abs(abs_sums ? (size_t)n * 9 : 0, 0.0);
     if(g_margin)
         for(int64_t i = 0; i < n; ++i)
             g_margin[i] = 1e30f;
@@ -636,6 +649,7 @@ extern "C" void dsxo_blend_bwd(const dsxo_settings* s, int64_t n, const int32_t*
             const float ca = conic[3 * (int64_t)g], cb = conic[3 * (int64_t)g + 1], cc = conic[3 * (int64_t)g + 2];
             const float cr = rgb[3 * (int64_t)g], cg = rgb[3 * (int64_t)g + 1], cbl = rgb[3 * (int64_t)g + 2];
             double l[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+            double la[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
             float gm = 1e30f;
             bool any = false;
             for(int t = 0; t < TILE * TILE; ++t)
@@ -680,6 +694,7 @@ extern "C" void dsxo_blend_bwd(const dsxo_settings* s, int64_t n, const int32_t*
                 v_alpha += -Tfin[t] * ra * bg0 * vo0;
                 v_alpha += -Tfin[t] * ra * bg1 * vo1;
                 v_alpha += -Tfin[t] * ra * bg2 * vo2;
+                const float buf_before[3] = {buf[t][0], buf[t][1], buf[t][2]};
                 buf[t][0] += cr * fac;
                 buf[t][1] += cg * fac;
                 buf[t][2] += cbl * fac;
@@ -690,6 +705,27 @@ extern "C" void dsxo_blend_bwd(const dsxo_settings* s, int64_t n, const int32_t*
                 l[6] += (double)(v_sigma * (ca * dx + cb * dy));
                 l[7] += (double)(v_sigma * (cb * dx + cc * dy));
                 l[8] += (double)(vis * v_alpha);
+                if(abs_sums)
+                {
+                    /* the same sums with every elementary term replaced by its absolute value */
+                    const double aT = fabs((double)Tc), ara = fabs((double)ra), aTf = fabs((double)Tfin[t]) * ara;
+                    const double va = (fabs((double)cr) * aT + fabs((double)buf_before[0]) * ara) * fabs((double)vo0) +
+                                      (fabs((double)cg) * aT + fabs((double)buf_before[1]) * ara) * fabs((double)vo1) +
+                                      (fabs((double)cbl) * aT + fabs((double)buf_before[2]) * ara) * fabs((double)vo2) +
+                                      aTf * (fabs((double)voa) + fabs((double)(bg0 * vo0)) + fabs((double)(bg1 * vo1)) +
+                                             fabs((double)(bg2 * vo2)));
+                    const double vs = fabs((double)opac) * (double)vis * va;
+                    const double adx = fabs((double)dx), ady = fabs((double)dy);
+                    la[0] += fabs((double)(fac * vo0));
+                    la[1] += fabs((double)(fac * vo1));
+                    la[2] += fabs((double)(fac * vo2));
+                    la[3] += 0.5 * vs * adx * adx;
+                    la[4] += vs * adx * ady;
+                    la[5] += 0.5 * vs * ady * ady;
+                    la[6] += vs * (fabs((double)ca) * adx + fabs((double)cb) * ady);
+                    la[7] += vs * (fabs((double)cb) * adx + fabs((double)cc) * ady);
+                    la[8] += (double)vis * va;
+                }
             }
             if(g_margin && gm < 1e30f)
             {
@@ -708,8 +744,34 @@ extern "C" void dsxo_blend_bwd(const dsxo_settings* s, int64_t n, const int32_t*
 #endif
                 a[c] += l[c];
             }
+            if(abs_sums)
+            {
+                double* b = acc_abs.data() + (size_t)g * 9;
+                for(int c = 0; c < 9; ++c)
+                {
+#ifdef _OPENMP
+#pragma omp atomic
+#endif
+                    b[c] += la[c];
+                }
+            }
         }
     }
+    if(abs_sums) /* in the order of the GPU's accumulator record: x y | conic a b c | opacity | r g b */
+        for(int64_t i = 0; i < n; ++i)
+        {
+            const double* b = acc_abs.data() + (size_t)i * 9;
+            float* o = abs_sums + 9 * i;
+            o[0] = (float)b[6];
+            o[1] = (float)b[7];
+            o[2] = (float)b[3];
+            o[3] = (float)b[4];
+            o[4] = (float)b[5];
+            o[5] = (float)b[8];
+            o[6] = (float)b[0];
+            o[7] = (float)b[1];
+            o[8] = (float)b[2];
+        }
     for(int64_t i = 0; i < n; ++i)
     {
         const double* a = acc.data() + (size_t)i * 9;
@@ -1094,10 +1156,20 @@ extern "C" void dsxo_backward(dsxo_state* st, const dsxo_settings* s, int64_t n,
                               const float* v_image, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
                               float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, float* g_margin)
 {
+    dsxo_backward_ex(st, s, n, num_bases, means3d, scales, quats, opacities, v_image, v_mean3d, v_means2d, v_shs,
+                     v_colors, v_opacity, v_scale, v_quat, v_cov3d, g_margin, nullptr);
+}
+
+extern "C" void dsxo_backward_ex(dsxo_state* st, const dsxo_settings* s, int64_t n, int32_t num_bases,
+                                 const float* means3d, const float* scales, const float* quats,
+                                 const float* opacities, const float* v_image, float* v_mean3d, float* v_means2d,
+                                 float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
+                                 float* v_cov3d, float* g_margin, float* abs_sums)
+{
     std::vector<float> v_xy(2 * n), v_conic(3 * n), v_cov2d(3 * n);
-    dsxo_blend_bwd(s, n, st->ranges.data(), st->ids.data(), st->means2d.data(), st->conic.data(), st->rgb.data(),
-                   opacities, st->final_T.data(), st->final_idx.data(), v_image, nullptr, v_xy.data(), v_conic.data(),
-                   v_colors, v_opacity, g_margin, &st->counters);
+    dsxo_blend_bwd_ex(s, n, st->ranges.data(), st->ids.data(), st->means2d.data(), st->conic.data(), st->rgb.data(),
+                      opacities, st->final_T.data(), st->final_idx.data(), v_image, nullptr, v_xy.data(),
+                      v_conic.data(), v_colors, v_opacity, g_margin, &st->counters, abs_sums);
     /* rasterizer_torch.cu:292: v_colors *= clamped_colors (all ones) — identity */
     dsxo_sh_bwd(s, n, num_bases, means3d, v_colors, v_shs);
     dsxo_project_bwd(s, n, means3d, scales, quats, st->conic.data(), st->cov3d.data(), st->radii.data(), v_xy.data(),

@@ -105,6 +105,19 @@ void dsxo_blend_bwd(const dsxo_settings* s, int64_t n, const int32_t* ranges,
                     float* v_xy, float* v_conic, float* v_rgb, float* v_opacity, float* g_margin,
                     dsxo_counters* counters);
 
+/* The same, plus abs_sums[N,9] (may be NULL): for every Gaussian and every one of the nine sums,
+ * in the order x y | conic a b c | opacity | r g b, the sum over pixels of the ABSOLUTE values of
+ * the elementary terms (every product that enters v_alpha taken by its magnitude).  A float
+ * summation in another order, or with other roundings of the terms, may differ from the exact
+ * sum by a small multiple of machine epsilon times this figure: it is the scale that a
+ * tolerance on these gradients has to be relative to. */
+void dsxo_blend_bwd_ex(const dsxo_settings* s, int64_t n, const int32_t* ranges,
+                       const int32_t* sorted_ids, const float* means2d, const float* conic,
+                       const float* rgb, const float* opacities, const float* final_T,
+                       const int32_t* final_idx, const float* v_out, const float* v_out_alpha,
+                       float* v_xy, float* v_conic, float* v_rgb, float* v_opacity, float* g_margin,
+                       dsxo_counters* counters, float* abs_sums);
+
 /* Stage 5b: gsplat/sh.cuh:95-203 with viewdirs = means - campos (rasterizer_torch.cu:291).
  * v_shs[N, num_bases, 3] where num_bases follows rasterizer_torch.cu:224-239 / sh.cuh:18-29;
  * entries above the active degree are zero (gsplat/bindings.cu:38-39). */
@@ -141,6 +154,12 @@ void dsxo_backward(dsxo_state* st, const dsxo_settings* s, int64_t n, int32_t nu
                    const float* opacities, const float* v_image, float* v_mean3d, float* v_means2d,
                    float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
                    float* v_cov3d, float* g_margin);
+/* dsxo_backward with the abs_sums[N,9] of dsxo_blend_bwd_ex (may be NULL) */
+void dsxo_backward_ex(dsxo_state* st, const dsxo_settings* s, int64_t n, int32_t num_bases,
+                      const float* means3d, const float* scales, const float* quats,
+                      const float* opacities, const float* v_image, float* v_mean3d, float* v_means2d,
+                      float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
+                      float* v_cov3d, float* g_margin, float* abs_sums);
 void dsxo_state_free(dsxo_state* st);
 
 /* ---- float64 instances used only for finite-difference pinning of the backward ---- */

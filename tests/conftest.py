@@ -17,3 +17,17 @@ def oracle():
     from oracle.binding import Oracle
 
     return Oracle()
+
+
+@pytest.fixture
+def blend_form():
+    """Returns a function that forces one form of the blend kernels (1 or 4 pixels per lane) for the
+    rest of the test; the library's own choice by image size is restored afterwards."""
+    from ds_splat_amd import _native
+    lib = _native.load()
+
+    def force(pixels_per_lane):
+        _native.check(lib.dsx_set_blend_pixels_per_lane(int(pixels_per_lane)))
+
+    yield force
+    _native.check(lib.dsx_set_blend_pixels_per_lane(0))

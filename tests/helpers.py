@@ -42,3 +42,94 @@ def perspective(tanfovx, tanfovy, znear=0.01, zfar=100.0):
     P[2, 3] = -zfar * znear / (zfar - znear)
     P[3, 2] = 1.0
     return P
+
+
+# Cameras for the GPU parity tests.  "identity" is the benchmark's (view = I, campos = 0, square
+# pixels); the others exercise what the identity hides: the layout of the view matrix in the
+# EWA projection and its backward, campos in the SH view direction, the scale modifier in the
+# covariance and its gradient, fx != fy, and Gaussians behind a rotated camera.
+CAMERAS = {
+    "identity": None,
+    # outside the cloud, rotated about all three axes and translated
+    "rotated": dict(eye=(3.0, 1.5, -2.0), target=(0.2, -0.1, 6.0), up=(0.1, 1.0, 0.05)),
+    # inside the cloud: about half of the Gaussians lie behind the camera
+    "inside": dict(eye=(0.5, -0.3, 5.0), target=(-1.0, 0.5, 9.0), up=(0.0, 1.0, 0.2), scale_modifier=1.3),
+    # non-square pixels (fx != fy) and a shrinking scale modifier
+    "anisotropic": dict(eye=(-2.5, 2.0, -1.0), target=(0.5, 0.0, 7.0), up=(-0.2, 1.0, 0.0), tanfovx=0.62,
+                        tanfovy=0.41, scale_modifier=0.7),
+}
+
+
+def set_camera(sc, camera):
+    """Replaces the camera of a ds_splat_amd.synthetic scene (in place) by CAMERAS[camera]:
+    viewmatrix / projmatrix in the API's transposed convention, campos, tan(fov), scale modifier."""
+    spec = CAMERAS[camera] if isinstance(camera, str) else camera
+    if spec is None:
+        return sc
+    tanfovx = float(spec.get("tanfovx", sc["tanfovx"]))
+    tanfovy = float(spec.get("tanfovy", sc["tanfovy"]))
+    V = look_at_view(spec["eye"], spec["target"], spec.get("up", (0.0, 1.0, 0.0)))
+    full = perspective(tanfovx, tanfovy) @ V
+    sc["tanfovx"], sc["tanfovy"] = tanfovx, tanfovy
+    sc["viewmatrix"] = torch.from_numpy(V.astype(np.float32)).t().contiguous()
+    sc["projmatrix"] = torch.from_numpy(full.astype(np.float32)).t().contiguous()
+    sc["campos"] = torch.tensor(spec["eye"], dtype=torch.float32)
+    sc["scale_modifier"] = float(spec.get("scale_modifier", 1.0))
+    return sc
+
+
+def comparable_gaussians(S, B, width, final_T=None, final_idx=None, slack=8):
+    """Mask of the Gaussians whose gradients two correct implementations must agree on.
+
+    Left out: a Gaussian with a borderline backward decision of its own (g_margin), and every
+    Gaussian in front of a pixel whose FORWARD walk differs between the two: a decision that falls
+    inside the rounding differences of exp (alpha against 1/255, T against 1e-4) may go the other
+    way, the pixel then blends one entry more or less, and the terms of everything in front of it
+    at that pixel shift.  With the GPU's final_T / final_idx (numpy, [H, W]) those pixels are the
+    ones where the two forwards disagree (final_T beyond rtol 1e-4, or another last entry) — the
+    caller asserts separately that this happens only at pixels with a small decision margin;
+    without them, every pixel whose margin is below 1e-5 counts.  The Gaussians left out are the
+    entries of such a pixel's tile list up to the tile's last blended entry (plus `slack`)."""
+    gok = B["g_margin"] > 1e-5
+    ntx = (width + 15) // 16
+    if final_T is None:
+        differs = S["margin"] < 1e-5
+        last_idx = S["final_idx"]
+    else:
+        differs = (np.abs(final_T - S["final_T"]) > 1e-4 * np.abs(S["final_T"])) | (final_idx != S["final_idx"])
+        last_idx = np.maximum(final_idx, S["final_idx"])
+    ys, xs = np.nonzero(differs)
+    tiles = np.unique((ys // 16) * ntx + (xs // 16))
+    if len(tiles):
+        H, W = last_idx.shape
+        nty = (H + 15) // 16
+        pad = np.zeros((nty * 16, ntx * 16), last_idx.dtype)
+        pad[:H, :W] = last_idx
+        last = pad.reshape(nty, 16, ntx, 16).max(axis=(1, 3)).reshape(-1)     # last blended entry per tile
+        r = S["ranges"]
+        for t in tiles.tolist():
+            end = min(int(r[t + 1]), int(last[t]) + 1 + slack)
+            gok[S["sorted_ids"][int(r[t]):end]] = False
+    return gok
+
+
+GRAD_KEYS = (("means", "v_mean3d"), ("means2d", "v_means2d"), ("shs", "v_shs"), ("opac", "v_opacity"),
+             ("scales", "v_scale"), ("rots", "v_quat"))
+
+
+def check_grads_against_bounds(got, B, bounds, mask, what=""):
+    """got: dict key -> numpy array (keys of the oracle's backward()).  Every element of a compared
+    Gaussian must lie within its own bound (Oracle.gradient_bounds: 1e-3 of the summed magnitude of
+    the terms it is made of).  Returns the largest error / bound ratio seen."""
+    worst = 0.0
+    for key, g in got.items():
+        want = B[key][mask].astype(np.float64)
+        err = np.abs(g.reshape(B[key].shape)[mask].astype(np.float64) - want)
+        bound = bounds[key].reshape(B[key].shape)[mask]
+        ratio = err / np.maximum(bound, 1e-300)
+        if ratio.size:
+            i = np.unravel_index(np.argmax(ratio), ratio.shape)
+            worst = max(worst, float(ratio[i]))
+            assert ratio[i] <= 1.0, "%s %s: error %.3e exceeds bound %.3e (want %.6e) at %s" % (
+                what, key, err[i], bound[i], want[i], i)
+    return worst

@@ -26,6 +26,19 @@ def test_library_exports_every_declared_symbol():
         assert getattr(lib, name) is not None
 
 
+def test_probe_library_exports_what_its_header_declares():
+    """include/dsx_probe.h: the benchmark's streaming probe lives in a library of its own."""
+    import ctypes as C
+    text = open(os.path.join(ROOT, "include", "dsx_probe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(dsxp_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["dsxp_stream_probe"]
+    lib = C.CDLL(os.path.join(ROOT, "ds_splat_amd", "lib", "libdsx_probe.so"))
+    for name in names:
+        assert getattr(lib, name) is not None
+    assert lib.dsxp_stream_probe(None, None, C.c_size_t(16), 2, None, None) == -1     # no launch without buffers
+
+
 def test_torch_binding_loads_and_links_the_library():
     from ds_splat_amd import _native
     ext = _native.load_torch_ext()
@@ -95,6 +108,34 @@ def test_python_api_surface():
     sig = list(inspect.signature(GaussianRasterizer.forward).parameters)
     assert sig == ["self", "means_3d", "means_2d", "shs", "colors_precomp", "opacities", "scales", "rotations",
                    "cov_3d_precomp"]
+
+
+def test_native_settings_follow_the_settings_tensors():
+    """The transposed camera matrices are cached per settings object: a replaced or modified matrix
+    must be seen, and matrices made under torch.inference_mode (no version counter) must work."""
+    import torch
+    from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
+    from ds_splat_amd.synthetic import make_scene
+    sc = make_scene("cfg0", n=8, width=32, height=32)
+    s = GaussianRasterizationSettings(32, 32, sc["tanfovx"], sc["tanfovy"], sc["bg"], 1.0, sc["viewmatrix"].clone(),
+                                      sc["projmatrix"].clone(), 0, 3, sc["campos"], False, False)
+    r = GaussianRasterizer(s)
+    a = r.settings_for_cpp_code
+    assert r.settings_for_cpp_code is a                                  # unchanged: cached
+    assert torch.equal(a.view_matrix, s.viewmatrix.t()) and torch.equal(a.proj_matrix, s.projmatrix.t())
+    s.viewmatrix[3, 0] = 5.0                                             # modified in place
+    b = r.settings_for_cpp_code
+    assert b is not a and float(b.view_matrix[0, 3]) == 5.0
+    s.viewmatrix = torch.eye(4) * 2.0                                    # replaced
+    c = r.settings_for_cpp_code
+    assert c is not b and float(c.view_matrix[1, 1]) == 2.0
+    s.scale_modifier = 1.3
+    assert r.settings_for_cpp_code.scale_modifier == 1.3
+    with torch.inference_mode():
+        s.viewmatrix = torch.eye(4) * 3.0
+        s.projmatrix = torch.arange(16, dtype=torch.float32).reshape(4, 4)
+        d = r.settings_for_cpp_code
+    assert float(d.view_matrix[2, 2]) == 3.0 and float(d.proj_matrix[0, 1]) == 4.0
 
 
 def test_scene_dump_round_trip(tmp_path):

@@ -5,7 +5,8 @@ import pytest
 import torch
 
 from ds_splat_amd.synthetic import make_scene
-from helpers import arrays, scene_settings
+from helpers import (GRAD_KEYS, arrays, check_grads_against_bounds, comparable_gaussians, scene_settings,
+                     set_camera)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -16,9 +17,9 @@ def api_run(sc, scale_mul=1.0, backward=True, bg=None, opac_shape=None, colors=N
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
     settings = GaussianRasterizationSettings(
         image_height=sc["height"], image_width=sc["width"], tanfovx=sc["tanfovx"], tanfovy=sc["tanfovy"],
-        bg=t["bg"] if bg is None else torch.tensor(bg, dtype=torch.float32, device=DEV), scale_modifier=1.0,
-        viewmatrix=t["viewmatrix"], projmatrix=t["projmatrix"], sh_degree=sc["sh_degree"], max_sh_degree=3,
-        campos=t["campos"], prefiltered=False, debug=False)
+        bg=t["bg"] if bg is None else torch.tensor(bg, dtype=torch.float32, device=DEV),
+        scale_modifier=sc["scale_modifier"], viewmatrix=t["viewmatrix"], projmatrix=t["projmatrix"],
+        sh_degree=sc["sh_degree"], max_sh_degree=3, campos=t["campos"], prefiltered=False, debug=False)
     opac = t["opacities"] if opac_shape is None else t["opacities"].reshape(opac_shape)
     leaves = dict(means=t["means_3d"].clone(), means2d=torch.zeros_like(t["means_3d"]), shs=t["shs"].clone(),
                   opac=opac.clone(), scales=(t["scales"] * scale_mul).clone(), rots=t["rotations"].clone())
@@ -46,45 +47,70 @@ def oracle_run(oracle, sc, scale_mul=1.0, bg=None, backward=True):
     s = scene_settings(sc, bg=bg)
     img, radii, st = oracle.forward(s, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["shs"])
     S = oracle.state(s, st, sc["n"])
-    B = oracle.backward(s, st, 16, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["v_image"]) \
-        if backward else None
+    B = None
+    if backward:
+        B = oracle.backward(s, st, 16, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["v_image"])
+        # atomics reorder the per-Gaussian sums: every gradient element gets its own tolerance, 1e-4 of
+        # the summed magnitudes of the terms it is made of (no tensor-wide floor; measured errors stay
+        # below 1e-5 of that figure)
+        B["bounds"] = oracle.gradient_bounds(s, 16, A["means_3d"], A["scales"], A["rotations"], S["conic"],
+                                             S["cov3d"], radii, B["abs_sums"], rel=1e-4)
     oracle.free(st)
     return img, radii, S, B
 
 
-def check_grads(leaves, B, ok):
-    pairs = (("means", "v_mean3d"), ("means2d", "v_means2d"), ("shs", "v_shs"), ("opac", "v_opacity"),
-             ("scales", "v_scale"), ("rots", "v_quat"))
-    for leaf, key in pairs:
-        got = leaves[leaf].grad.cpu().numpy().reshape(B[key].shape)[ok]
-        want = B[key][ok]
-        # atomics reorder the per-Gaussian sums: 1e-3 relative, floor at 1e-4 of the tensor's scale
-        scale = max(1.0, float(np.abs(want).max()))
-        np.testing.assert_allclose(got, want, rtol=1e-3, atol=1e-4 * scale, err_msg=key)
+def gpu_forward_state(sc, scale_mul=1.0):
+    """final_T and final_idx of the GPU's forward (numpy): where they differ from the oracle's, a
+    borderline decision went the other way and the pixel's tile list is not compared."""
+    from ds_splat_amd import stages
+    cam = stages.camera_from_scene(sc, DEV)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    _, st = stages.forward(cam, t["means_3d"], t["scales"] * scale_mul, t["rotations"], t["opacities"], t["shs"])
+    torch.cuda.synchronize()
+    return st.final_T.cpu().numpy(), st.final_idx.cpu().numpy(), st
 
 
-@pytest.mark.parametrize("name,n,W,H,deg,scale_mul,bg", [
-    ("cfg0", 16384, 256, 256, 0, 1.0, None),            # workload cfg0 at full size
-    ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9)),
-    ("cfg1", 40000, 480, 270, 3, 1.0, None),            # config 1 distributions, reduced size
-    ("cfg4", 3000, 320, 180, 3, 0.5, None),             # heavy-overlap distributions, reduced size
-    ("cfg2", 30000, 333, 177, 2, 1.5, None),            # ragged image (not a multiple of 16)
+def check_grads(leaves, B, ok, what=""):
+    got = {key: leaves[leaf].grad.cpu().numpy() for leaf, key in GRAD_KEYS}
+    worst = check_grads_against_bounds(got, B, B["bounds"], ok, what)
+    print("%s: gradients of %d of %d Gaussians compared (%.1f %%), largest error / bound = %.3f" % (
+        what, int(ok.sum()), ok.size, 100.0 * ok.mean(), worst))
+    return worst
+
+
+@pytest.mark.parametrize("name,n,W,H,deg,scale_mul,bg,camera", [
+    ("cfg0", 16384, 256, 256, 0, 1.0, None, "identity"),            # workload cfg0 at full size
+    ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9), "identity"),
+    ("cfg1", 40000, 480, 270, 3, 1.0, None, "identity"),            # config 1 distributions, reduced size
+    ("cfg4", 3000, 320, 180, 3, 0.5, None, "identity"),             # heavy-overlap distributions, reduced size
+    ("cfg2", 30000, 333, 177, 2, 1.5, None, "identity"),            # ragged image (not a multiple of 16)
+    # general cameras: rotated + translated (campos != 0 matters at SH degree 3), a camera inside the
+    # cloud (Gaussians behind it) with scale modifier 1.3, non-square pixels with scale modifier 0.7
+    ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9), "rotated"),
+    ("cfg0", 20000, 320, 200, 3, 2.0, None, "inside"),
+    ("cfg1", 40000, 480, 270, 3, 1.5, (0.5, 0.1, 0.3), "anisotropic"),
+    ("cfg4", 3000, 320, 180, 2, 0.5, None, "rotated"),
 ])
 @pytest.mark.parametrize("pixels_per_lane", ["1", "4"])
-def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, bg, pixels_per_lane, monkeypatch):
+def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, bg, camera, pixels_per_lane,
+                                        blend_form):
     # both forms of the blend kernels, whatever the image size would pick
-    monkeypatch.setenv("DSX_BLEND_PIXELS_PER_LANE", pixels_per_lane)
-    sc = make_scene(name, n=n, width=W, height=H, sh_degree=deg)
+    blend_form(pixels_per_lane)
+    sc = set_camera(make_scene(name, n=n, width=W, height=H, sh_degree=deg), camera)
     image, radii, leaves = api_run(sc, scale_mul, bg=bg)
     img_o, radii_o, S, B = oracle_run(oracle, sc, scale_mul, bg=bg)
     assert image.shape == (H, W, 3) and radii.dtype == torch.int32 and radii.shape == (n,)
     assert (radii.cpu().numpy() == radii_o).all()
+    assert (radii_o > 0).sum() > n // 20
     ok = S["margin"] > 1e-4
-    assert ok.mean() > 0.98
+    assert ok.mean() > 0.98, ok.mean()
     np.testing.assert_allclose(image.detach().cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
-    gok = B["g_margin"] > 1e-5
-    assert gok.mean() > 0.97
-    check_grads(leaves, B, gok)
+    T_gpu, idx_gpu, _ = gpu_forward_state(sc, scale_mul)
+    # the two forwards disagree on a pixel's walk only where a decision was borderline
+    assert (S["margin"][(T_gpu != S["final_T"]) & ~np.isclose(T_gpu, S["final_T"], rtol=1e-4, atol=0)] < 1e-4).all()
+    gok = comparable_gaussians(S, B, W, T_gpu, idx_gpu)
+    assert gok.mean() > 0.9, gok.mean()
+    check_grads(leaves, B, gok, "%s %s" % (name, camera))
     assert leaves["opac"].grad.shape == leaves["opac"].shape
     assert (leaves["means2d"].grad[:, 2] == 0).all()
 
@@ -156,12 +182,12 @@ def test_only_the_gradients_asked_for_are_produced():
 
 @pytest.mark.parametrize("pixels_per_lane", ["1", "4"])
 @pytest.mark.parametrize("n", [20000, 20001])
-def test_forward_prepares_the_accumulator_for_one_backward(monkeypatch, pixels_per_lane, n):
+def test_forward_prepares_the_accumulator_for_one_backward(blend_form, pixels_per_lane, n):
     """With prepare_grads the blend forward prepares the backward's accumulator on the side (both kernel
     forms, a Gaussian count that does and does not divide by the wavefronts' shares); a backward on
     it equals one that fills for itself, and a second backward on the same state fills again."""
     from ds_splat_amd import stages
-    monkeypatch.setenv("DSX_BLEND_PIXELS_PER_LANE", pixels_per_lane)
+    blend_form(pixels_per_lane)
     sc = make_scene("cfg1", n=n, width=320, height=200, sh_degree=3)
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
     cam = stages.camera_from_scene(sc, DEV)
@@ -476,6 +502,11 @@ def test_full_size_properties_cfg4_heavy_overlap():
     assert float(o["v_shs"].abs().max()) > 0
 
 
+# share of the VISIBLE Gaussians whose gradients must be comparable at full size (the rest can be
+# reached by a pixel with a borderline forward decision; more of them where lists are long)
+GRADS_COMPARED_FLOOR = {"cfg1": 0.5, "cfg2": 0.5, "cfg4": 0.05}
+
+
 @pytest.mark.parametrize("workload", ["cfg1", "cfg2", "cfg4"])
 def test_full_size_against_the_openmp_oracle(workload):
     """The three forward+backward shapes at full size (500 K Gaussians, the headline 3 M, and the
@@ -492,16 +523,16 @@ def test_full_size_against_the_openmp_oracle(workload):
     img_o, radii_o, S, B = oracle_run(omp, sc)
     assert (radii.cpu().numpy() == radii_o).all()
     ok = S["margin"] > 1e-4
-    assert ok.mean() > 0.97
+    visible = radii_o > 0
+    T_gpu, idx_gpu, st = gpu_forward_state(sc)
+    gok = comparable_gaussians(S, B, sc["width"], T_gpu, idx_gpu)
+    print("%s: %.2f %% of the pixels compared; %d Gaussians visible" % (workload, 100.0 * ok.mean(), int(visible.sum())))
+    assert ok.mean() > 0.97, ok.mean()
     np.testing.assert_allclose(image.detach().cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
-    gok = B["g_margin"] > 1e-5
-    assert gok.mean() > 0.9
-    check_grads(leaves, B, gok)
+    check_grads(leaves, B, gok, workload)
+    # the culled Gaussians compare trivially (all zeros): the floor is on the visible ones
+    assert gok[visible].mean() > GRADS_COMPARED_FLOOR[workload], gok[visible].mean()
     del image, leaves
-    cam = stages.camera_from_scene(sc, DEV)
-    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
-    _, st = stages.forward(cam, t["means_3d"], t["scales"], t["rotations"], t["opacities"], t["shs"])
-    torch.cuda.synchronize()
     assert st.num_keys == S["num_keys"]
     assert (st.ranges.cpu().numpy() == S["ranges"]).all()
     assert (st.sorted_ids.cpu().numpy() == S["sorted_ids"]).all()

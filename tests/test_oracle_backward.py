@@ -282,3 +282,61 @@ def test_full_backward_shapes_and_zero_column(oracle):
     assert B["v_means2d"].shape == (50, 3) and (B["v_means2d"][:, 2] == 0).all()
     assert B["v_opacity"].shape == (50, 1) and B["v_shs"].shape == (50, 16, 3)
     assert np.abs(B["v_mean3d"]).max() > 0 and np.isfinite(B["v_quat"]).all()
+
+
+def test_abs_sums_bound_the_sums_and_equal_them_where_no_term_cancels(oracle):
+    """abs_sums (the scale of the gradient tolerances): never below |sum|; equal to the sum where
+    every term has one sign (v_rgb under a positive upstream gradient); strictly larger where terms
+    cancel (a sign-mixed upstream gradient)."""
+    sc, s, A, S, radii = forward_state(oracle, n=80, W=64, H=48, seed=3)
+    pos = np.abs(RNG.normal(size=(sc["height"], sc["width"], 3))).astype(np.float32)
+    B = oracle.blend_bwd(s, S["ranges"], S["sorted_ids"], S["means2d"], S["conic"], S["rgb"], A["opacities"],
+                         S["final_T"], S["final_idx"], pos)
+    got = np.concatenate([B["v_xy"], B["v_conic"], B["v_opacity"], B["v_rgb"]], axis=1)
+    assert (B["abs_sums"] * (1 + 1e-5) + 1e-30 >= np.abs(got)).all()
+    touched = np.abs(B["v_rgb"]).sum(1) > 0
+    assert touched.sum() > 20
+    np.testing.assert_allclose(B["abs_sums"][:, 6:9], B["v_rgb"], rtol=1e-5, atol=1e-12)
+    mixed = RNG.normal(size=(sc["height"], sc["width"], 3)).astype(np.float32)
+    B2 = oracle.blend_bwd(s, S["ranges"], S["sorted_ids"], S["means2d"], S["conic"], S["rgb"], A["opacities"],
+                          S["final_T"], S["final_idx"], mixed)
+    got2 = np.concatenate([B2["v_xy"], B2["v_conic"], B2["v_opacity"], B2["v_rgb"]], axis=1)
+    assert (B2["abs_sums"] * (1 + 1e-5) + 1e-30 >= np.abs(got2)).all()
+    assert (B2["abs_sums"][touched, 6:9] > 1.05 * np.abs(B2["v_rgb"][touched])).mean() > 0.5
+    # |v_image| as the upstream gradient bounds every channel sum of the sign-mixed run
+    B3 = oracle.blend_bwd(s, S["ranges"], S["sorted_ids"], S["means2d"], S["conic"], S["rgb"], A["opacities"],
+                          S["final_T"], S["final_idx"], np.abs(mixed))
+    np.testing.assert_allclose(B2["abs_sums"][:, 6:9], B3["v_rgb"], rtol=1e-5, atol=1e-12)
+
+
+def test_gradient_bounds_hold_for_perturbed_screen_space_sums(oracle):
+    """gradient_bounds propagates a tolerance on the nine screen-space sums through the (linear)
+    per-Gaussian backward: outputs of inputs perturbed inside the tolerance stay inside the bounds,
+    and a perturbation ten times larger leaves them."""
+    sc = make_scene("cfg0", n=300, width=96, height=64, sh_degree=3, seed=8)
+    A = arrays(sc)
+    V = look_at_view((1.0, 0.5, -1.0), (0.0, 0.0, 6.0))
+    s = make_settings(64, 96, 0.6, 0.45, np.zeros(3), 1.3, V, perspective(0.6, 0.45) @ V, 3, (1.0, 0.5, -1.0))
+    P = oracle.project_fwd(s, A["means_3d"], A["scales"] * 3, A["rotations"], A["shs"])
+    n = 300
+    v = RNG.normal(size=(n, 9)).astype(np.float32)
+    scale = np.abs(v) * 3.0 + 0.1                                          # plays the abs_sums
+    run = lambda u: (oracle.project_bwd(s, A["means_3d"], A["scales"] * 3, A["rotations"], P["conic"], P["cov3d"],
+                                        P["radii"], u[:, 0:2], u[:, 2:5]),
+                     oracle.sh_bwd(s, 16, A["means_3d"], u[:, 6:9]))
+    base, base_sh = run(v)
+    bounds = oracle.gradient_bounds(s, 16, A["means_3d"], A["scales"] * 3, A["rotations"], P["conic"], P["cov3d"],
+                                    P["radii"], scale, rel=1e-3, floor=0.0)
+    sign = np.sign(RNG.normal(size=(n, 9))).astype(np.float32)
+    inside, inside_sh = run(v + 0.9e-3 * scale * sign)
+    outside, _ = run(v + 1e-2 * scale * sign)
+    vis = P["radii"] > 0
+    assert vis.sum() > 50
+    slack = 1e-6   # float rounding of the two runs themselves, relative to the bound's own scale
+    for key in ("v_mean3d", "v_scale", "v_quat", "v_cov3d"):
+        err = np.abs(inside[key].astype(np.float64) - base[key])
+        assert (err <= bounds[key] * (1 + 1e-3) + slack * np.abs(base[key])).all(), key
+        far = np.abs(outside[key].astype(np.float64) - base[key])
+        assert (far[vis] > bounds[key][vis]).mean() > 0.3, key
+    err = np.abs(inside_sh.astype(np.float64) - base_sh)
+    assert (err <= bounds["v_shs"] * (1 + 1e-3) + slack * np.abs(base_sh)).all()
