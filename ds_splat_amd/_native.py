@@ -65,6 +65,7 @@ SIGNATURES = {
     "dsx_forward_project": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P] * 4 + [_P, C.c_size_t, _P, _P]),
     "dsx_forward_finish": (C.c_int, [_CAM, _I64, _I64] + [_P] * 7 + [_P, C.c_size_t, _P, _P]),
     "dsx_backward": (C.c_int, [_CAM, _I64, _I32] + [_P] * 11 + [_P, _I32] + [_P] * 8 + [_P]),
+    "dsx_backward_static": (C.c_int, [_CAM, _I64, _I32] + [_P] * 11 + [_P] * 8 + [_P]),
     "dsx_forward_core": (C.c_int, [_P] * 5 + [_I64] + [_P] * 3 + [_I32, _I32, C.c_float, C.c_float, C.c_float,
                                                                     _I32, _I32, _P, _P]),
 }

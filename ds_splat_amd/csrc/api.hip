@@ -115,6 +115,9 @@ extern "C" const char* dsx_error_string(int status)
         case DSX_ERR_RUNTIME: return "dsx: HIP runtime call failed";
         case DSX_ERR_TOO_LARGE: return "dsx: too many tile keys for 32-bit key indexing (K >= 2^30)";
         case DSX_ERR_WORKSPACE: return "dsx: workspace too small (see dsx_workspace_bytes)";
+        case DSX_ERR_STATIC_LIMIT:
+            return "dsx: more Gaussians than the built-in scratch of dsx_backward_static holds "
+                   "(DSX_STATIC_MAX_GAUSSIANS = 524288); use dsx_backward with a caller-provided accumulator";
         default: return "dsx: unknown status";
     }
 }
@@ -595,6 +598,58 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
         (void)hipFreeAsync(buf2, s);
     (void)hipFreeAsync(buf, s);
     return rc;
+}
+
+// ---- backward without a caller-provided accumulator ---------------------------------------
+// The gradient accumulator of dsx_backward ([n * 12] floats of scratch) lives in a file-scope
+// device array here.  In host code the array's NAME is only a stand-in: each device holds its own
+// copy at its own address, which hipGetSymbolAddress returns; that address is what the kernels get.
+namespace
+{
+constexpr int64_t kStaticMaxGaussians = DSX_STATIC_MAX_GAUSSIANS;
+static __device__ __align__(256) float scratch[kStaticMaxGaussians * DSX_GRAD_FLOATS];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the current device (looked up once per device), or null
+float* static_scratch()
+{
+    int device = -1;
+    if(hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+        return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if(g_scratch_ptr[device] == nullptr)
+    {
+        void* p = nullptr;
+        if(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess)
+            return nullptr;
+        g_scratch_ptr[device] = static_cast<float*>(p);
+    }
+    return g_scratch_ptr[device];
+}
+} // namespace
+
+extern "C" int dsx_backward_static(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+                                   const float* scales, const float* quats, const float* splats,
+                                   const float* cov3d, const int32_t* radii, const int32_t* ranges,
+                                   const int32_t* sorted_ids, const float* final_T, const int32_t* final_idx,
+                                   const float* v_image, float* v_mean3d, float* v_means2d, float* v_shs,
+                                   float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
+                                   float* v_cov3d, void* stream)
+{
+    if(n > kStaticMaxGaussians)
+        return DSX_ERR_STATIC_LIMIT;
+    // (n <= 0 touches no memory: dsx_backward rejects a negative n and returns at n == 0)
+    float* grads = n > 0 ? static_scratch() : nullptr;
+    if(n > 0 && grads == nullptr)
+        return DSX_ERR_RUNTIME;
+    // grads_prepared = 0: the array keeps the last call's sums, so this call clears its n records
+    // itself (a fill kernel with plain stores, which a caller may capture in a graph)
+    return dsx_backward(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, ranges, sorted_ids, final_T,
+                        final_idx, v_image, grads, 0, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat,
+                        v_cov3d, stream);
 }
 
 extern "C" int dsx_set_blend_pixels_per_lane(int pixels)

@@ -12,7 +12,8 @@
  * and kept until the process ends: dsx_depth_order / dsx_forward_project fork onto it and join
  * before they return, so that the tile counting runs beside the depth sort — callers on
  * different streams of one device share it and their forked parts serialise there; (3) the
- * blend-kernel form override of dsx_set_blend_pixels_per_lane.
+ * blend-kernel form override of dsx_set_blend_pixels_per_lane; (4) the device address of the
+ * built-in scratch of dsx_backward_static, looked up once per device.
  *
  * What each entry point replaces in the reference (deepsense-ai/ds-splat) is cited as
  * file:line next to it.  Matrices are row-major, math convention (translation in elements
@@ -33,6 +34,7 @@ extern "C" {
 #define DSX_SPLAT_FLOATS 12    /* projected record, 48 bytes (3 x float4) */
 #define DSX_GRAD_FLOATS 12     /* screen-space gradient accumulator record, 48 bytes */
 #define DSX_PROJ_BLOCK 256     /* Gaussians per workgroup in the per-Gaussian kernels */
+#define DSX_STATIC_MAX_GAUSSIANS 524288 /* largest n of dsx_backward_static (24 MiB of built-in scratch) */
 
 typedef enum dsx_status
 {
@@ -41,7 +43,8 @@ typedef enum dsx_status
     DSX_ERR_LAUNCH = -2,       /* hipGetLastError() after a launch reported a failure       */
     DSX_ERR_RUNTIME = -3,      /* a HIP runtime call (memcpy, sync, event) failed           */
     DSX_ERR_TOO_LARGE = -4,    /* sizes beyond 32-bit indexing of keys (K >= 2^30)          */
-    DSX_ERR_WORKSPACE = -5     /* workspace smaller than dsx_workspace_bytes() asks for     */
+    DSX_ERR_WORKSPACE = -5,    /* workspace smaller than dsx_workspace_bytes() asks for     */
+    DSX_ERR_STATIC_LIMIT = -6  /* n beyond DSX_STATIC_MAX_GAUSSIANS (dsx_backward_static)   */
 } dsx_status;
 
 /* Mirrors TorchRasterizationSettings, cpp/ds_cuda_rasterizer/rasterizer_torch.hpp:7-22.
@@ -244,6 +247,26 @@ int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const floa
                  float* grads, int32_t grads_prepared, float* v_mean3d, float* v_means2d,
                  float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
                  float* v_cov3d, void* stream);
+
+/* dsx_backward for callers that cannot allocate or bring device scratch: code under HIP graph
+ * capture, tight serving or training loops, harnesses that forbid hipMalloc.  No counterpart in
+ * the reference (its backward allocates every temporary through torch).  The same computation and
+ * the same arguments as dsx_backward, except that the [n * 12] gradient accumulator is not an
+ * argument: it is a device array built into the library, DSX_STATIC_MAX_GAUSSIANS records =
+ * 24 MiB, which every GPU the library runs on holds until the process ends.  The call allocates
+ * and frees nothing, on the device or through any library; it returns DSX_ERR_STATIC_LIMIT for
+ * n > DSX_STATIC_MAX_GAUSSIANS.  The array keeps the previous call's sums; each call clears the
+ * n records it uses with a fill kernel (plain stores) before accumulating.  All calls on one GPU
+ * share the one array: calls that overlap on a GPU (two streams, two host threads) race — keep
+ * them on one stream or serialise them.  The array's device address is looked up on the first
+ * call on each device: make that first call outside a graph capture. */
+int dsx_backward_static(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+                        const float* scales, const float* quats, const float* splats,
+                        const float* cov3d, const int32_t* radii, const int32_t* ranges,
+                        const int32_t* sorted_ids, const float* final_T, const int32_t* final_idx,
+                        const float* v_image, float* v_mean3d, float* v_means2d, float* v_shs,
+                        float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
+                        float* v_cov3d, void* stream);
 
 /* Raw-pointer forward-only render, the role of rasterizer_forward_core_deepsense
  * (cpp/ds_cuda_rasterizer/rasterizer_cuda.hpp:4-9, cpp/rasterizer_cuda.cu:128-158) without

@@ -1,0 +1,72 @@
+"""dsx_backward_static (the backward whose gradient accumulator is a device array built into the
+library, for callers that cannot allocate) against dsx_backward on the same forward state, through
+the C ABI: two calls in a row, the second on a smaller scene, so that what the first call left in the
+shared array must not leak into the second."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from ds_splat_amd.synthetic import make_scene
+from helpers import arrays, scene_settings, set_camera
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _backward_both_ways(oracle, n, W, H, camera, seed):
+    from ds_splat_amd import _native, stages
+    lib = _native.load()
+    sc = set_camera(make_scene("cfg1", n=n, width=W, height=H, sh_degree=3, seed=seed), camera)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    scales = (t["scales"] * 2.0).contiguous()
+    cam = stages.camera_from_scene(sc, DEV)
+    _, st = stages.forward(cam, t["means_3d"], scales, t["rotations"], t["opacities"], t["shs"])
+    # the existing entry point, with a caller-provided accumulator
+    ref = stages.backward(cam, st, 16, t["means_3d"], scales, t["rotations"], t["v_image"])
+    # the entry point under test: same arguments, no accumulator
+    out = stages._bwd_outputs(n, 16, torch.device(DEV))
+    p = lambda x: None if x is None else C.c_void_p(x.data_ptr())
+    rc = lib.dsx_backward_static(cam.ref, n, 16, p(t["means_3d"]), p(scales), p(t["rotations"]), p(st.splats), None,
+                                 p(st.radii), p(st.ranges), p(st.sorted_ids), p(st.final_T), p(st.final_idx),
+                                 p(t["v_image"]), p(out["v_mean3d"]), p(out["v_means2d"]), p(out["v_shs"]),
+                                 p(out["v_colors"]), p(out["v_opacity"]), p(out["v_scale"]), p(out["v_quat"]),
+                                 p(out["v_cov3d"]), C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, _native.load().dsx_error_string(rc)
+    torch.cuda.synchronize()
+    # tolerances per element from the oracle: 1e-4 of the summed magnitudes of the terms of each sum
+    # (both runs add them with float atomics, in an order of their own)
+    A = arrays(sc)
+    s = scene_settings(sc)
+    _, radii, ost = oracle.forward(s, A["means_3d"], A["scales"] * 2.0, A["rotations"], A["opacities"], A["shs"])
+    S = oracle.state(s, ost, n)
+    B = oracle.backward(s, ost, 16, A["means_3d"], A["scales"] * 2.0, A["rotations"], A["opacities"], A["v_image"])
+    oracle.free(ost)
+    bounds = oracle.gradient_bounds(s, 16, A["means_3d"], A["scales"] * 2.0, A["rotations"], S["conic"], S["cov3d"],
+                                    radii, B["abs_sums"], rel=1e-4)
+    assert st.num_keys == S["num_keys"] > 3 * n
+    worst = 0.0
+    for key in ("v_mean3d", "v_means2d", "v_shs", "v_colors", "v_opacity", "v_scale", "v_quat", "v_cov3d"):
+        a, b = ref[key].cpu().numpy().astype(np.float64), out[key].cpu().numpy().astype(np.float64)
+        assert np.isfinite(b).all() and np.abs(a).max() > 0, key
+        ratio = np.abs(a - b) / (bounds[key].reshape(a.shape) + 1e-300)
+        assert ratio.max() <= 1.0, "%s: static and caller-scratch backward differ by %.3e of the bound" % (
+            key, ratio.max())
+        worst = max(worst, float(ratio.max()))
+    return worst
+
+
+def test_backward_static_matches_backward_twice_in_a_row(oracle):
+    first = _backward_both_ways(oracle, 30000, 640, 360, "rotated", seed=71)
+    second = _backward_both_ways(oracle, 7000, 320, 200, "identity", seed=72)      # smaller: stale sums must be gone
+    print("dsx_backward_static vs dsx_backward: largest difference / bound = %.4f, %.4f" % (first, second))
+
+
+def test_backward_static_rejects_more_gaussians_than_its_scratch_holds():
+    from ds_splat_amd import _native
+    lib = _native.load()
+    cam = _native.Camera(64, 64, 0.5, 0.5, 1.0, 3, 3, 8, 8, 8, 8)
+    fake = 16
+    rc = lib.dsx_backward_static(C.byref(cam), 524288 + 1, 16, *([fake] * 11), *([None] * 8), None)
+    assert rc == -6 and b"524288" in lib.dsx_error_string(rc)
