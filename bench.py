@@ -99,6 +99,8 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--list-bin", type=int, default=0, choices=(0, 1, 2, 4),
+                    help="tiles per side of the bins the tile lists are built for (0: the library's choice)")
     ap.add_argument("--verbose", action="store_true", help="per-kernel table on stderr")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic that scales HBM byte counters) and "
@@ -116,7 +118,7 @@ def main():
     from ds_splat_amd import _native
     from ds_splat_amd.synthetic import WORKLOADS, make_scene
 
-    _native.load()
+    _native.check(_native.load().dsx_set_list_bin(args.list_bin))
     spec = WORKLOADS[args.workload]
     dev = torch.device("cuda:0")
     sc = make_scene(spec, n=args.n)

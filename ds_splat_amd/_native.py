@@ -80,6 +80,9 @@ class TraceEntry(C.Structure):
 SIGNATURES["dsx_trace_enable"] = (C.c_int, [C.c_int])
 SIGNATURES["dsx_trace_read"] = (C.c_int, [C.POINTER(TraceEntry), C.c_int])
 SIGNATURES["dsx_set_blend_pixels_per_lane"] = (C.c_int, [C.c_int])
+SIGNATURES["dsx_list_bin"] = (_I32, [_I32, _I32])
+SIGNATURES["dsx_set_list_bin"] = (C.c_int, [C.c_int])
+SIGNATURES["dsx_ranges_count"] = (_I64, [_I32, _I32])
 
 _lib = None
 

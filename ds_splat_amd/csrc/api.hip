@@ -145,7 +145,22 @@ extern "C" int32_t dsx_sort_passes(int32_t num_tiles)
 extern "C" size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height)
 {
     (void)n;
-    return lists_workspace(k < 0 ? 0 : k, dsx_num_tiles(width, height)).bytes;
+    return lists_workspace(k < 0 ? 0 : k, list_grid(width, height).lists()).bytes;
+}
+
+extern "C" int32_t dsx_list_bin(int32_t width, int32_t height)
+{
+    return 1 << list_grid(width, height).shift;
+}
+
+extern "C" int dsx_set_list_bin(int tiles_per_side)
+{
+    return set_list_bin(tiles_per_side);
+}
+
+extern "C" int64_t dsx_ranges_count(int32_t width, int32_t height)
+{
+    return ranges_layout(list_grid(width < 0 ? 0 : width, height < 0 ? 0 : height)).count;
 }
 
 extern "C" size_t dsx_sort_workspace_bytes(int64_t k, int32_t num_tiles)
@@ -371,7 +386,7 @@ extern "C" int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t heigh
         *partition_flag = nullptr;
         if(workspace && k > 0)
         {
-            const int tiles = dsx_num_tiles(width, height);
+            const int tiles = list_grid(width, height).lists();
             const ListsWorkspace lw = lists_workspace(k, tiles);
             const Sort32Workspace w = sort32_workspace(k, slot_bits(tiles), kListSortTile);
             *partition_flag =
@@ -394,7 +409,7 @@ extern "C" int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const
     {
         if(!order || !sorted_ids || !workspace)
             return DSX_ERR_BAD_ARG;
-        if(workspace_bytes < lists_workspace(k, dsx_num_tiles(cam->image_width, cam->image_height)).bytes)
+        if(workspace_bytes < lists_workspace(k, list_grid(cam->image_width, cam->image_height).lists()).bytes)
             return DSX_ERR_WORKSPACE;
     }
     return launch_tile_lists(*cam, n, k, order, sorted_ids, ranges, workspace, as_stream(stream));
@@ -507,7 +522,8 @@ extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, c
     if(rc)
         return rc;
     return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream), depth_flag,
-                            partition_flag, n > 0 ? grads_to_prepare : nullptr, n);
+                            partition_flag, n > 0 ? grads_to_prepare : nullptr, n,
+                            list_grid(cam->image_width, cam->image_height).shift ? ranges : nullptr);
 }
 
 extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
@@ -526,7 +542,8 @@ extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases,
     if(!ranges || !final_T || !final_idx || !v_image || !grads || !splats)
         return DSX_ERR_BAD_ARG;
     int rc = launch_blend_bwd(*cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
-                              as_stream(stream), grads_prepared != 0);
+                              as_stream(stream), grads_prepared != 0,
+                              list_grid(cam->image_width, cam->image_height).shift ? ranges : nullptr);
     if(rc)
         return rc;
     return gaussian_bwd_checked(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
@@ -567,7 +584,7 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     o_cov3d = align(o_radii + (size_t)n * 4);
     o_bs = align(o_cov3d + (size_t)n * 24);
     o_ranges = align(o_bs + (size_t)nb * 4);
-    o_T = align(o_ranges + (size_t)(num_tiles + 1) * 4);
+    o_T = align(o_ranges + (size_t)dsx_ranges_count(image_width, image_height) * 4);
     o_idx = align(o_T + (size_t)P * 4);
     o_order = align(o_idx + (size_t)P * 4);
     const size_t order_bytes = order_layout(n, image_width, image_height).bytes;
@@ -583,7 +600,7 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     char* buf2 = nullptr;
     if(rc == DSX_OK)
     {
-        const size_t ws = lists_workspace(k, num_tiles).bytes;
+        const size_t ws = lists_workspace(k, list_grid(image_width, image_height).lists()).bytes;
         const size_t o_ids = align(ws);
         if(hipMallocAsync(reinterpret_cast<void**>(&buf2), o_ids + (size_t)k * 4 + 256, s) != hipSuccess)
             rc = DSX_ERR_RUNTIME;

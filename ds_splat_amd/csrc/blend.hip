@@ -109,6 +109,74 @@ static int blend_pixels_per_lane(int num_tiles, int four_from)
         return forced;
     return num_tiles >= four_from ? 4 : 1;
 }
+// Binned tile lists (see ListGrid): what a blend kernel needs to find a tile's entries in its
+// bin's list.  fine[t] .. fine[t + 1] is the tile's range in the reference's fully sorted key
+// array: its length says how many entries of the bin list belong to the tile, and its start turns
+// "the i-th entry of the tile" into the index that the reference's final_idx holds.
+struct BinLists
+{
+    const int32_t* fine;      // int32[tiles + 1]
+    const int32_t* last_tile; // highest occupied tile (-1: none)
+    const int32_t* bins;      // int32[bins + 1]
+    int32_t* walk;            // int32[tiles * 8]: per tile and band, (last blended position in the bin list, its index in the tile's list)
+    int shift, nbx, nty;
+};
+
+// Where tile `tile` finds its entries.  The reference never records the end of the LAST run of
+// its sorted keys (cpp/rasterizer_kernels.cu:313-322, cpp/rasterizer_torch.cu:31-39), so the pairs
+// of the highest occupied tile are walked by the image's last tile instead, and by nobody if that
+// is another tile; with no tile occupied at all, the last tile walks the pairs of negative depth
+// (slot 0, positions [0, bins[0])), every one of them.  The per-tile ranges carry those rules;
+// here they decide whose pairs (src) the tile takes out of which bin's list.
+struct TileSource
+{
+    int start, end; // positions in sorted_ids to scan
+    int count;      // entries among them that belong to the tile
+    int fine_base;  // index of the tile's first entry in the fully sorted key array
+    int sx, sy;     // the tile whose rectangle membership selects the entries; sx < 0: every entry belongs
+};
+__device__ __forceinline__ TileSource tile_source(const BinLists& L, int tile, int ntx)
+{
+    TileSource t;
+    t.fine_base = L.fine[tile];
+    t.count = L.fine[tile + 1] - t.fine_base;
+    t.start = t.end = 0;
+    t.sx = t.sy = 0;
+    if(t.count <= 0)
+        return t;
+    int src = tile;
+    if(tile == ntx * L.nty - 1)
+        src = *L.last_tile;
+    if(src < 0)
+    {
+        t.sx = -1;
+        t.end = L.bins[0];
+        return t;
+    }
+    t.sx = src % ntx;
+    t.sy = src / ntx;
+    const int bin = (t.sy >> L.shift) * L.nbx + (t.sx >> L.shift);
+    t.start = L.bins[bin];
+    t.end = L.bins[bin + 1];
+    return t;
+}
+
+// does the entry's tile rectangle (recomputed from the splat record exactly as the projection
+// computed it) contain the source tile?
+__device__ __forceinline__ bool entry_in_tile(const TileSource& t, float px, float py, float radius_bits, int ntx, int nty)
+{
+    if(t.sx < 0)
+        return true;
+    const TileRect r = tile_rect(px, py, __float_as_int(radius_bits), ntx, nty);
+    return t.sx >= r.sx && t.sx < r.ex && t.sy >= r.sy && t.sy < r.ey;
+}
+
+// number of set bits of a wavefront mask below this lane
+__device__ __forceinline__ int bits_below_lane(uint64_t mask)
+{
+    return (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
 constexpr int kFwdFourPixelsFrom = 5000; // tiles
 constexpr int kBwdFourPixelsFrom = 1600;
 
@@ -125,7 +193,10 @@ constexpr int kBwdFourPixelsFrom = 1600;
 constexpr int kFwdBatch = 128; // sorted entries staged in LDS per round (two per lane)
 
 // 8 wavefronts per SIMD (at most 64 VGPRs): all tiles of a 1080p image are resident at once
-template <int kFwdPix>
+// kBinned: the entries come out of the list of the tile's bin (BinLists); an entry belongs to the
+// tile if its tile rectangle contains it, and final_idx still receives the reference's index (the
+// tile's range start plus the entry's rank among the tile's own entries).
+template <int kFwdPix, bool kBinned>
 __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))) void blend_fwd_kernel(const int32_t* __restrict__ ranges,
                                                              const int32_t* __restrict__ ids,
                                                              const float4* __restrict__ splats,
@@ -133,7 +204,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                                                              int32_t* __restrict__ final_idx, int W, int H, int ntx,
                                                              const uint32_t* __restrict__ sort_flag_a,
                                                              const uint32_t* __restrict__ sort_flag_b,
-                                                             float4* __restrict__ prep, int64_t prep_count)
+                                                             float4* __restrict__ prep, int64_t prep_count,
+                                                             const BinLists lists)
 {
     __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic a, conic b
     __shared__ float4 s_b[kFwdBatch]; // conic c, opacity, red, green
@@ -151,8 +223,21 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     const float box_x0 = (float)(tx * kTile) + 0.5f, box_y0 = (float)(ty * kTile + 4 * band) + 0.5f;
     const float span_y = kFwdPix == 4 ? 15.0f : 3.0f;
 
-    const int start = ranges[tile];
-    const int end = ranges[tile + 1];
+    int start, end;
+    TileSource src;
+    if(kBinned)
+    {
+        src = tile_source(lists, tile, ntx);
+        start = src.start;
+        end = src.end;
+    }
+    else
+    {
+        start = ranges[tile];
+        end = ranges[tile + 1];
+    }
+    int seen = 0;     // entries of the tile's own list met so far (binned lists)
+    int pos_hi = -1;  // position of the last entry that any pixel blended (binned lists)
 
     // A pixel that has stopped (or lies outside the image) gets NaN as its row coordinate: its
     // exponent is then NaN, the test `power < 0` fails whatever the entry holds, and the loop
@@ -177,14 +262,19 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     {
         if(alive == 0)
             break;
+        if(kBinned && seen >= src.count) // the bin's list goes on, the tile's own has ended
+            break;
         __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
         uint64_t todo[kFwdBatch / DSX_WAVE]; // entries of this round that can touch the tile
+        uint64_t members[kFwdBatch / DSX_WAVE]; // entries of this round that belong to the tile (binned lists)
+        int seen_before[kFwdBatch / DSX_WAVE];  // entries of the tile's own list before each half of the round
 #pragma unroll
         for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
         {
             const int slot = h * DSX_WAVE + lane;
             const int e = b + slot;
             bool useful = false;
+            bool member = false;
             if(e < end)
             {
                 const int g = ids[e];
@@ -193,9 +283,16 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                 s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
                 s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
-                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
+                member = !kBinned || entry_in_tile(src, q0.x, q0.y, q0.w, ntx, lists.nty);
+                useful = member && entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
             }
             todo[h] = __ballot(useful);
+            if(kBinned)
+            {
+                members[h] = __ballot(member);
+                seen_before[h] = seen;
+                seen += __popcll(members[h]);
+            }
         }
         __syncthreads();
 #pragma unroll
@@ -206,11 +303,18 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             {
                 if(alive == 0)
                     break;
-                const int i = h * DSX_WAVE + __builtin_ctzll(mask);
+                const int bit = __builtin_ctzll(mask);
+                const int i = h * DSX_WAVE + bit;
                 mask &= mask - 1;
                 const float4 A = s_a[i];
                 const float4 B = s_b[i];
                 const float C = s_c[i];
+                // what final_idx records for this entry: its position in the sorted key array
+                // (binned lists: the tile's range start plus the entry's rank among the tile's own
+                // entries, counted on the scalar unit from the round's membership mask)
+                const int entry_index =
+                    kBinned ? src.fine_base + seen_before[h] + __popcll(members[h] & ((1ull << bit) - 1ull)) : b + i;
+                uint64_t m_applied = 0;
                 const ExponentX ex = exponent_x(A.z, A.w, pxf - A.x);
 #pragma unroll
                 for(int p = 0; p < kFwdPix; ++p)
@@ -232,10 +336,14 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                     cg[p] += vis * B.w;
                     cb[p] += vis * C;
                     T[p] = apply ? Tn : T[p];
-                    last[p] = apply ? b + i : last[p];
+                    last[p] = apply ? entry_index : last[p];
                     pyf[p] = stop ? __builtin_nanf("") : pyf[p];
                     alive -= __popcll(m_stop);
+                    if(kBinned)
+                        m_applied |= m_pass & ~m_low;
                 }
+                if(kBinned)
+                    pos_hi = m_applied ? b + i : pos_hi; // (scalar unit)
             }
         }
     }
@@ -262,6 +370,29 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             final_idx[pix] = last[p];
         }
     }
+    if(kBinned)
+    {
+        // for the backward: where this wavefront's walk ended, as a position in the bin's list and
+        // as an index in the sorted key array (-1, -1 if it blended nothing).  The four-pixel form
+        // speaks for the whole tile and marks the other three bands as empty.
+        int top = -1;
+#pragma unroll
+        for(int p = 0; p < kFwdPix; ++p)
+            top = max(top, last[p]);
+#pragma unroll
+        for(int o = 32; o > 0; o >>= 1)
+            top = max(top, __shfl_xor(top, o, DSX_WAVE));
+        if(pos_hi < 0)
+            top = -1;
+        int32_t* w = lists.walk + (int64_t)tile * 8;
+        if(kFwdPix == 4)
+        {
+            if(lane < 8)
+                w[lane] = lane == 0 ? pos_hi : (lane == 1 ? top : -1);
+        }
+        else if(lane < 2)
+            w[2 * band + lane] = lane == 0 ? pos_hi : top;
+    }
     // A side job for the memory system, which this kernel leaves idle: every wavefront prepares
     // its share of the backward's gradient accumulator, twelve floats per Gaussian: the nine sums
     // zeroed and, in the three spare places, the conic, which the per-Gaussian backward then has
@@ -285,10 +416,12 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     }
 }
 
+// lists: null when ranges / sorted_ids are the per-tile lists (the stage entry point), else the
+// `ranges` buffer of binned lists in ranges_layout() (the kernel also writes its `walk` part)
 int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids, const float* splats,
                      float* image, float* final_T, int32_t* final_idx, hipStream_t stream,
                      const uint32_t* sort_flag_a, const uint32_t* sort_flag_b, float* prepare_grads,
-                     int64_t num_gaussians)
+                     int64_t num_gaussians, int32_t* lists)
 {
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
     if(ntx * nty == 0)
@@ -297,16 +430,39 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
         return DSX_ERR_BAD_ARG;
     float4* prep = reinterpret_cast<float4*>(prepare_grads);
     const int64_t prep_count = prepare_grads ? num_gaussians : 0;
+    BinLists L = {};
+    if(lists)
+    {
+        const ListGrid lg = list_grid(cam.image_width, cam.image_height);
+        if(lg.shift == 0)
+            return DSX_ERR_BAD_ARG;
+        const RangesLayout rl = ranges_layout(lg);
+        L.fine = lists + rl.fine;
+        L.last_tile = lists + rl.last_tile;
+        L.bins = lists + rl.bins;
+        L.walk = lists + rl.walk;
+        L.shift = lg.shift;
+        L.nbx = lg.nbx;
+        L.nty = nty;
+    }
     {
         DSX_TIMED("blend_fwd_kernel", stream);
-        if(blend_pixels_per_lane(ntx * nty, kFwdFourPixelsFrom) == 4)
-            hipLaunchKernelGGL(blend_fwd_kernel<4>, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
-                               reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                               cam.image_height, ntx, sort_flag_a, sort_flag_b, prep, prep_count);
+        const bool four = blend_pixels_per_lane(ntx * nty, kFwdFourPixelsFrom) == 4;
+        const dim3 grid(four ? ntx * nty : 4 * ntx * nty);
+        const float4* sp = reinterpret_cast<const float4*>(splats);
+#define DSX_LAUNCH_FWD(PIX, BINNED)                                                                              \
+    hipLaunchKernelGGL((blend_fwd_kernel<PIX, BINNED>), grid, dim3(DSX_WAVE), 0, stream, ranges, sorted_ids, sp,   \
+                       image, final_T, final_idx, cam.image_width, cam.image_height, ntx, sort_flag_a,            \
+                       sort_flag_b, prep, prep_count, L)
+        if(four && lists)
+            DSX_LAUNCH_FWD(4, true);
+        else if(four)
+            DSX_LAUNCH_FWD(4, false);
+        else if(lists)
+            DSX_LAUNCH_FWD(1, true);
         else
-            hipLaunchKernelGGL(blend_fwd_kernel<1>, dim3(4 * ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
-                               reinterpret_cast<const float4*>(splats), image, final_T, final_idx, cam.image_width,
-                               cam.image_height, ntx, sort_flag_a, sort_flag_b, prep, prep_count);
+            DSX_LAUNCH_FWD(1, false);
+#undef DSX_LAUNCH_FWD
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;
@@ -392,11 +548,14 @@ constexpr int kBwdBatch = 128; // sorted entries staged in LDS per round (two pe
 // (tile, entry).  Compared with four wavefronts of one pixel per lane this does one
 // cross-lane reduction per entry instead of four and needs no LDS accumulators or barriers.
 // (kBwdPix = 1: four wavefronts per tile with one band of four rows each, as in the forward)
-template <int kBwdPix>
+// kBinned: the entries come out of the list of the tile's bin; the forward left, per tile and band,
+// the bin-list position where its walk ended and that entry's index in the sorted key array, from
+// which every entry met on the way down gets its own index (final_idx is compared with those).
+template <int kBwdPix, bool kBinned>
 __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const int32_t* __restrict__ ranges, const int32_t* __restrict__ ids, const float4* __restrict__ splats,
     const float* __restrict__ final_T, const int32_t* __restrict__ final_idx, const float* __restrict__ v_image,
-    const float* __restrict__ bg, float* grads, int W, int H, int ntx)
+    const float* __restrict__ bg, float* grads, int W, int H, int ntx, const BinLists lists)
 {
     __shared__ float4 s_a[kBwdBatch]; // pixel x, pixel y, conic a, conic b
     __shared__ float4 s_b[kBwdBatch]; // conic c, opacity, red, green
@@ -439,25 +598,48 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
         m = max(m, bin_final[p]);
     }
 
-    const int start = ranges[tile];
-    const int end = ranges[tile + 1];
-
-    // last entry any pixel of this tile blended
+    int start, hi;
+    TileSource src;
+    int index_hi = 0; // index (in the sorted key array) of the entry at position hi (binned lists)
+    int above = 0;    // entries of the tile's own list met so far, from the top (binned lists)
+    if(kBinned)
+    {
+        // the forward's walk of this tile ended at position hi of the bin's list, on the entry
+        // with index index_hi (the larger of the four bands' figures: both grow together)
+        src = tile_source(lists, tile, ntx);
+        start = src.start;
+        const int32_t* w = lists.walk + (int64_t)tile * 8;
+        hi = max(max(w[0], w[2]), max(w[4], w[6]));
+        index_hi = max(max(w[1], w[3]), max(w[5], w[7]));
+        if(src.count <= 0)
+            hi = -1;
+    }
+    else
+    {
+        start = ranges[tile];
+        const int end = ranges[tile + 1];
+        // last entry any pixel of this tile blended
 #pragma unroll
-    for(int o = 32; o > 0; o >>= 1)
-        m = max(m, __shfl_xor(m, o, DSX_WAVE));
-    const int hi = min(end - 1, m);
+        for(int o = 32; o > 0; o >>= 1)
+            m = max(m, __shfl_xor(m, o, DSX_WAVE));
+        hi = min(end - 1, m);
+    }
 
     for(int top = hi; top >= start; top -= kBwdBatch)
     {
+        if(kBinned && index_hi - above < src.fine_base) // every entry of the tile's own list has been met
+            break;
         __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
         uint64_t todo[kBwdBatch / DSX_WAVE]; // entries of this round that can touch the tile
+        uint64_t members[kBwdBatch / DSX_WAVE]; // entries of this round that belong to the tile (binned lists)
+        int above_before[kBwdBatch / DSX_WAVE]; // entries of the tile's own list above each half of the round
 #pragma unroll
         for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
         {
             const int slot = h * DSX_WAVE + lane;
             const int e = top - slot;
             bool useful = false;
+            bool member = false;
             if(e >= start)
             {
                 const int g = ids[e];
@@ -467,17 +649,28 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
                 s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
                 s_id[slot] = g;
-                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
+                member = !kBinned || entry_in_tile(src, q0.x, q0.y, q0.w, ntx, lists.nty);
+                useful = member && entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
             }
             todo[h] = __ballot(useful);
+            if(kBinned)
+            {
+                members[h] = __ballot(member);
+                above_before[h] = above;
+                above += __popcll(members[h]);
+            }
         }
         __syncthreads();
 #pragma unroll
         for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
         for(uint64_t mask = todo[h]; mask != 0; mask &= mask - 1)
         {
-            const int t = h * DSX_WAVE + __builtin_ctzll(mask);
-            const int idx = top - t;
+            const int bit = __builtin_ctzll(mask);
+            const int t = h * DSX_WAVE + bit;
+            // binned lists: lower slots are higher positions, so the entry's index is the top one's
+            // less the tile's entries met above it (scalar unit)
+            const int idx =
+                kBinned ? index_hi - above_before[h] - __popcll(members[h] & ((1ull << bit) - 1ull)) : top - t;
             const float4 A = s_a[t];
             const float4 B = s_b[t];
             // the exponent exactly as the forward computed it (pixel - mean); sigma = -exponent
@@ -556,9 +749,10 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     }
 }
 
+// lists: as for launch_blend_fwd (null: ranges / sorted_ids are per-tile lists)
 int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, const int32_t* sorted_ids,
                      const float* splats, const float* final_T, const int32_t* final_idx, const float* v_image,
-                     float* grads, hipStream_t stream, bool grads_prepared)
+                     float* grads, hipStream_t stream, bool grads_prepared, const int32_t* lists)
 {
     if(!grads_prepared)
         if(int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(grads), n * DSX_GRAD_FLOATS, 0u, stream))
@@ -566,16 +760,38 @@ int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, co
     const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
     if(ntx * nty == 0 || n == 0)
         return DSX_OK;
+    BinLists L = {};
+    if(lists)
+    {
+        const ListGrid lg = list_grid(cam.image_width, cam.image_height);
+        if(lg.shift == 0)
+            return DSX_ERR_BAD_ARG;
+        const RangesLayout rl = ranges_layout(lg);
+        L.fine = lists + rl.fine;
+        L.last_tile = lists + rl.last_tile;
+        L.bins = lists + rl.bins;
+        L.walk = const_cast<int32_t*>(lists) + rl.walk;
+        L.shift = lg.shift;
+        L.nbx = lg.nbx;
+        L.nty = nty;
+    }
     {
         DSX_TIMED("blend_bwd_kernel", stream);
-        if(blend_pixels_per_lane(ntx * nty, kBwdFourPixelsFrom) == 4)
-            hipLaunchKernelGGL(blend_bwd_kernel<4>, dim3(ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
-                               reinterpret_cast<const float4*>(splats), final_T, final_idx, v_image, cam.bg, grads,
-                               cam.image_width, cam.image_height, ntx);
+        const bool four = blend_pixels_per_lane(ntx * nty, kBwdFourPixelsFrom) == 4;
+        const dim3 grid(four ? ntx * nty : 4 * ntx * nty);
+        const float4* sp = reinterpret_cast<const float4*>(splats);
+#define DSX_LAUNCH_BWD(PIX, BINNED)                                                                              \
+    hipLaunchKernelGGL((blend_bwd_kernel<PIX, BINNED>), grid, dim3(DSX_WAVE), 0, stream, ranges, sorted_ids, sp,   \
+                       final_T, final_idx, v_image, cam.bg, grads, cam.image_width, cam.image_height, ntx, L)
+        if(four && lists)
+            DSX_LAUNCH_BWD(4, true);
+        else if(four)
+            DSX_LAUNCH_BWD(4, false);
+        else if(lists)
+            DSX_LAUNCH_BWD(1, true);
         else
-            hipLaunchKernelGGL(blend_bwd_kernel<1>, dim3(4 * ntx * nty), dim3(DSX_WAVE), 0, stream, ranges, sorted_ids,
-                               reinterpret_cast<const float4*>(splats), final_T, final_idx, v_image, cam.bg, grads,
-                               cam.image_width, cam.image_height, ntx);
+            DSX_LAUNCH_BWD(1, false);
+#undef DSX_LAUNCH_BWD
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;

@@ -170,6 +170,50 @@ inline int slot_bits(int num_tiles)
     return b;
 }
 
+// The tile lists are built per BIN of (1 << shift) x (1 << shift) tiles: a Gaussian enters the list
+// of every bin that its tile rectangle touches, once, and a blend tile walks its bin's list and
+// keeps the entries whose rectangle contains the tile itself.  shift = 0: one list per tile, the
+// reference's own lists.  Larger bins mean fewer pairs to emit and to partition (a Gaussian that
+// covers 11 tiles touches 2 or 3 bins of 4 x 4) and longer lists to filter in the blend.
+struct ListGrid
+{
+    int shift;    // log2 of the bin's side in tiles
+    int ntx, nty; // tiles of the image
+    int nbx, nby; // bins of the image
+    int tiles() const { return ntx * nty; }
+    int bins() const { return nbx * nby; }
+    // what the partition sorts by: bins when the lists are binned, tiles when they are not
+    int lists() const { return shift ? bins() : tiles(); }
+};
+ListGrid list_grid(int image_width, int image_height);
+// 0: choose by image size; 1, 2, 4: bins of that many tiles a side, for the whole process
+int set_list_bin(int tiles_per_side);
+
+// Layout of the `ranges` buffer of the forward (int32 words):
+//   fine[tiles + 1]   ranges of the per-tile lists as the reference defines them (the index of a
+//                     tile's first pair in the fully sorted key array; the last word is the
+//                     number of pairs)
+// and, when the lists are binned,
+//   last_tile[1]      highest tile that holds a pair of non-negative depth, -1 if none
+//   bins[bins + 1]    ranges of the bin lists inside sorted_ids
+//   walk[tiles * 8]   written by the blend forward for the backward: per tile and band of four
+//                     rows, the position in the bin list of the last entry any of its pixels
+//                     blended, and that entry's index in the per-tile list
+struct RangesLayout
+{
+    int fine, last_tile, bins, walk, count;
+};
+inline RangesLayout ranges_layout(const ListGrid& g)
+{
+    RangesLayout r;
+    r.fine = 0;
+    r.last_tile = g.tiles() + 1;
+    r.bins = r.last_tile + 1;
+    r.walk = r.bins + g.bins() + 1;
+    r.count = g.shift ? r.walk + g.tiles() * 8 : g.tiles() + 1;
+    return r;
+}
+
 // Workspace of one 32-bit sort of `count` pairs (offsets relative to its base, 256-byte aligned).
 struct Sort32Workspace
 {
@@ -194,8 +238,9 @@ struct OrderLayout
     size_t block_sums; // uint32[blocks + 1] tile counts of 256 consecutive Gaussians IN DEPTH ORDER, scanned
     size_t slot_hist;  // uint32[kMaxPasses32 * 256] digit histograms of the tile slots of all pairs
     size_t cover;      // int32[(ntx + 1) * (nty + 1) + 1] pairs per tile (corner grid, then its 2-D prefix sum)
-    size_t key_count;  // uint64     number of pairs of the scene (summed by the corner-grid kernel)
-    size_t ranges;     // int32[tiles + 1] the tile ranges, ready before the pairs exist
+    size_t bin_cover;  // int32[(nbx + 1) * (nby + 1) + 1] the same per bin (binned lists only)
+    size_t key_count;  // uint64[2]  pairs of the per-tile lists, pairs of the bin lists (summed by the corner-grid kernel)
+    size_t ranges;     // int32[...] ranges_layout() without its `walk` part, ready before the pairs exist
     size_t sort;       // Sort32Workspace
     size_t bytes;
 };
@@ -247,11 +292,11 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
                      const float* splats, float* image, float* final_T, int32_t* final_idx,
                      hipStream_t stream,
                      const uint32_t* sort_flag_a = nullptr, const uint32_t* sort_flag_b = nullptr,
-                     float* prepare_grads = nullptr, int64_t num_gaussians = 0);
+                     float* prepare_grads = nullptr, int64_t num_gaussians = 0, int32_t* lists = nullptr);
 int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges,
                      const int32_t* sorted_ids, const float* splats, const float* final_T,
                      const int32_t* final_idx, const float* v_image, float* grads,
-                     hipStream_t stream, bool grads_prepared = false);
+                     hipStream_t stream, bool grads_prepared = false, const int32_t* lists = nullptr);
 int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d,
                         const float* scales, const float* quats, const float* splats,
                         const float* cov3d, const int32_t* radii, const float* grads,

@@ -12,6 +12,7 @@
 // once and moved twice, instead of 12 bytes moved five times.
 #include "dsx_common.h"
 
+#include <atomic>
 #include <mutex>
 
 namespace dsx
@@ -41,6 +42,32 @@ static hipStream_t helper_stream()
             (void)hipGetLastError();
     }
     return streams[device];
+}
+
+// Bin size of the tile lists: 4 x 4 tiles from 256 tiles on (a Gaussian's rectangle then touches a
+// few bins instead of a dozen tiles, and emission and partition shrink accordingly), one list per
+// tile below (nothing to gain on a handful of tiles).  set_list_bin overrides it for the process.
+static std::atomic<int> g_list_bin{0};
+
+int set_list_bin(int tiles_per_side)
+{
+    if(tiles_per_side != 0 && tiles_per_side != 1 && tiles_per_side != 2 && tiles_per_side != 4)
+        return DSX_ERR_BAD_ARG;
+    g_list_bin.store(tiles_per_side, std::memory_order_relaxed);
+    return DSX_OK;
+}
+
+ListGrid list_grid(int image_width, int image_height)
+{
+    ListGrid g;
+    g.ntx = tiles_x(image_width);
+    g.nty = tiles_y(image_height);
+    const int forced = g_list_bin.load(std::memory_order_relaxed);
+    const int side = forced ? forced : (g.ntx * g.nty >= 256 ? 4 : 1);
+    g.shift = side == 4 ? 2 : (side == 2 ? 1 : 0);
+    g.nbx = (g.ntx + side - 1) / side;
+    g.nby = (g.nty + side - 1) / side;
+    return g;
 }
 
 __device__ __forceinline__ uint32_t wave_incl_scan32(uint32_t v, int)
@@ -565,13 +592,17 @@ OrderLayout order_layout(int64_t n, int image_width, int image_height)
     off = align(off + (size_t)kMaxPasses32 * kBins32 * 4);
     o.sort = off;
     off = align(off + sort32_workspace(n, 32, sort32_tile_keys(n)).bytes);
+    const ListGrid g = list_grid(image_width, image_height);
     o.cover = off;
-    off += (size_t)((tiles_x(image_width) + 1) * (tiles_y(image_height) + 1) + 1) * 4;
+    off += (size_t)((g.ntx + 1) * (g.nty + 1) + 1) * 4;
+    o.bin_cover = off;
+    if(g.shift)
+        off += (size_t)((g.nbx + 1) * (g.nby + 1) + 1) * 4;
     off = (off + 7) & ~(size_t)7;
-    o.key_count = off; // inside the region that is zeroed with the corner grid
-    off = align(off + 8);
+    o.key_count = off; // inside the region that is zeroed with the corner grids
+    off = align(off + 16);
     o.ranges = off;
-    off += (size_t)(tiles_x(image_width) * tiles_y(image_height) + 1) * 4;
+    off += (size_t)(ranges_layout(g).count - (g.shift ? g.tiles() * 8 : 0)) * 4;
     o.bytes = align(off);
     return o;
 }
@@ -581,17 +612,46 @@ __device__ __forceinline__ uint32_t rect_count(uint2 r)
     return (r.y & 0xffffu) * ((r.y >> 16) & 0x7fffu);
 }
 
+// The bins a tile rectangle touches: first bin (x, y) and extent, for a rectangle that is not empty.
+struct BinRect
+{
+    uint32_t bx, by, bw, bh;
+};
+__device__ __forceinline__ BinRect bin_rect(uint2 r, int shift)
+{
+    const uint32_t sx = r.x & 0xffffu, sy = r.x >> 16;
+    const uint32_t w = r.y & 0xffffu, h = (r.y >> 16) & 0x7fffu;
+    BinRect b;
+    b.bx = sx >> shift;
+    b.by = sy >> shift;
+    b.bw = ((sx + w - 1u) >> shift) - b.bx + 1u;
+    b.bh = ((sy + h - 1u) >> shift) - b.by + 1u;
+    return b;
+}
+// Pairs a Gaussian contributes to the lists: one per bin its rectangle touches (shift = 0: one
+// per tile).  A Gaussian with a negative depth is in no bin list; its pairs all sit in slot 0,
+// as many as the per-tile lists have, so that slot 0 is the same list whatever the bin size.
+__device__ __forceinline__ uint32_t list_count(uint2 r, int shift)
+{
+    const uint32_t fine = rect_count(r);
+    if(shift == 0 || fine == 0 || (r.y >> 31))
+        return fine;
+    const BinRect b = bin_rect(r, shift);
+    return b.bw * b.bh;
+}
+
 // Tile count of each run of 256 Gaussians taken in depth order (the last pass of the depth sort
 // has already put the rectangles into that order).
 __global__ __launch_bounds__(kProjBlock) void ordered_block_sums_kernel(const uint2* __restrict__ rects_sorted,
-                                                                       int64_t n, uint32_t* __restrict__ block_sums)
+                                                                       int64_t n, int shift,
+                                                                       uint32_t* __restrict__ block_sums)
 {
     __shared__ uint32_t wave_sums[kProjBlock / DSX_WAVE];
     const int tid = threadIdx.x;
     const int64_t p = (int64_t)blockIdx.x * kProjBlock + tid;
     uint32_t count = 0;
     if(p < n)
-        count = rect_count(rects_sorted[p]);
+        count = list_count(rects_sorted[p], shift);
     const uint32_t ws = wave_sum_u32(count);
     if((tid & 63) == 0)
         wave_sums[tid >> 6] = ws;
@@ -611,19 +671,27 @@ constexpr int kCoverBlocks = 128;
 constexpr int kCoverLdsCells = 14 * 1024;      // grids up to this many cells (56 KB) are held in LDS as they are
 constexpr int kCoverLdsCellsLarge = 38 * 1024; // up to 152 KB of the CU's 160 KB, once the kernels are allowed it
 
+// shift > 0: the same for the bins, into a second grid right behind the first (bin_grid); the
+// pairs of the bin lists are summed into key_count[1].
 __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* __restrict__ rects, int64_t n, int ntx,
-                                                                   int nty, int use_lds, int32_t* __restrict__ grid,
+                                                                   int nty, int shift, int nbx, int nby, int use_lds,
+                                                                   int32_t* __restrict__ grid,
+                                                                   int32_t* __restrict__ bin_grid,
                                                                    unsigned long long* __restrict__ key_count)
 {
     extern __shared__ int32_t s_grid[];
     const int tid = threadIdx.x;
-    unsigned long long pairs = 0; // tiles of this thread's rectangles: summed over the launch this is K
+    unsigned long long pairs = 0;     // tiles of this thread's rectangles: summed over the launch this is K
+    unsigned long long bin_pairs = 0; // the same for the bin lists
     const int pitch = ntx + 1;
     const int cells = pitch * (nty + 1) + 1;
+    const int bpitch = nbx + 1;
+    const int bcells = shift ? bpitch * (nby + 1) + 1 : 0;
     int32_t* acc = use_lds ? s_grid : grid;
+    int32_t* bacc = use_lds ? s_grid + cells : bin_grid;
     if(use_lds)
     {
-        for(int j = tid; j < cells; j += kCoverThreads)
+        for(int j = tid; j < cells + bcells; j += kCoverThreads)
             s_grid[j] = 0;
         __syncthreads();
     }
@@ -637,6 +705,11 @@ __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* 
         if(r.y >> 31)
         {
             atomicAdd(&acc[cells - 1], w * h);
+            if(shift)
+            {
+                atomicAdd(&bacc[bcells - 1], w * h);
+                bin_pairs += (unsigned long long)(w * h);
+            }
             continue;
         }
         const int sx = (int)(r.x & 0xffffu), sy = (int)(r.x >> 16);
@@ -644,6 +717,15 @@ __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* 
         atomicAdd(&acc[sy * pitch + sx + w], -1);
         atomicAdd(&acc[(sy + h) * pitch + sx], -1);
         atomicAdd(&acc[(sy + h) * pitch + sx + w], 1);
+        if(shift)
+        {
+            const BinRect b = bin_rect(r, shift);
+            bin_pairs += (unsigned long long)(b.bw * b.bh);
+            atomicAdd(&bacc[b.by * bpitch + b.bx], 1);
+            atomicAdd(&bacc[b.by * bpitch + b.bx + b.bw], -1);
+            atomicAdd(&bacc[(b.by + b.bh) * bpitch + b.bx], -1);
+            atomicAdd(&bacc[(b.by + b.bh) * bpitch + b.bx + b.bw], 1);
+        }
     }
     if(use_lds)
     {
@@ -651,23 +733,32 @@ __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* 
         for(int j = tid; j < cells; j += kCoverThreads)
             if(s_grid[j])
                 atomicAdd(&grid[j], s_grid[j]);
+        for(int j = tid; j < bcells; j += kCoverThreads)
+            if(s_grid[cells + j])
+                atomicAdd(&bin_grid[j], s_grid[cells + j]);
     }
     // the number of pairs of the whole scene (64 bits: it is compared with the 2^30 limit, not wrapped)
     // (one atomic per workgroup: atomics on one address serialise in the L2)
-    __shared__ unsigned long long s_pairs[kCoverThreads / DSX_WAVE];
+    __shared__ unsigned long long s_pairs[2][kCoverThreads / DSX_WAVE];
 #pragma unroll
     for(int o = 32; o > 0; o >>= 1)
+    {
         pairs += __shfl_xor(pairs, o, DSX_WAVE);
+        bin_pairs += __shfl_xor(bin_pairs, o, DSX_WAVE);
+    }
     if((tid & 63) == 0)
-        s_pairs[tid >> 6] = pairs;
+    {
+        s_pairs[0][tid >> 6] = pairs;
+        s_pairs[1][tid >> 6] = bin_pairs;
+    }
     __syncthreads();
-    if(tid == 0)
+    if(tid < 2)
     {
         unsigned long long total = 0;
         for(int w = 0; w < kCoverThreads / DSX_WAVE; ++w)
-            total += s_pairs[w];
+            total += s_pairs[tid][w];
         if(total)
-            atomicAdd(key_count, total);
+            atomicAdd(key_count + tid, total);
     }
 }
 
@@ -678,11 +769,33 @@ __global__ __launch_bounds__(kCoverThreads) void tile_cover_kernel(const uint2* 
 //    (cpp/rasterizer_kernels.cu:313-322, cpp/rasterizer_torch.cu:31-39): the boundary after
 //    the LAST run is never recorded, so tiles above the highest occupied tile inherit the
 //    START of that run (all zero when no tile is occupied), and ranges[num_tiles] = K.
-__global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(int32_t* grid, int ntx, int nty, int use_lds,
-                                                                    const Digits32 plan,
-                                                                    uint32_t* __restrict__ slot_hist,
-                                                                    int32_t* __restrict__ ranges)
+// Binned lists: workgroup 0 does the above for the tiles (no histograms: nothing is partitioned by
+// tile then) and also records the highest occupied tile; workgroup 1 takes the bins' grid, whose
+// ranges are plain prefix sums (the reference's two rules are rules about tiles) and whose
+// histograms drive the partition.
+struct CountsJob
 {
+    int32_t* grid;
+    int ntx, nty;
+    int plain;           // 1: ranges are plain prefix sums, no rule about the last run
+    uint32_t* slot_hist; // may be null
+    int32_t* ranges;
+    int32_t* last;       // may be null: receives the highest occupied tile, -1 if none
+    Digits32 plan;
+};
+struct CountsJobs
+{
+    CountsJob job[2];
+};
+
+__global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(const CountsJobs jobs, int use_lds)
+{
+    const CountsJob& J = jobs.job[blockIdx.x];
+    int32_t* const grid = J.grid;
+    const int ntx = J.ntx, nty = J.nty;
+    const Digits32& plan = J.plan;
+    uint32_t* const slot_hist = J.slot_hist;
+    int32_t* const ranges = J.ranges;
     extern __shared__ int32_t s_cells[];
     __shared__ uint32_t hist[kMaxPasses32 * kBins32];
     __shared__ __attribute__((aligned(16))) uint32_t wave_tot[kCoverThreads / DSX_WAVE];
@@ -749,7 +862,7 @@ __global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(int32_t* gri
         // after a wavefront sum; same-address LDS atomics would serialise)
         {
             const uint32_t slot = (uint32_t)t + 1u;
-            for(int p = 0; p < plan.passes; ++p)
+            for(int p = 0; slot_hist && p < plan.passes; ++p)
             {
                 const uint32_t d = (slot >> plan.shift[p]) & plan.mask[p];
                 if(plan.shift[p] == 0)
@@ -789,19 +902,25 @@ __global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(int32_t* gri
     __threadfence_block();
     __syncthreads();
     const int last = s_last;
-    const int32_t tail = last >= 0 ? ranges[last] : 0;
-    for(int t = tid; t < tiles; t += kCoverThreads)
-        if(t > last)
-            ranges[t] = tail;
+    if(!J.plain)
+    {
+        const int32_t tail = last >= 0 ? ranges[last] : 0;
+        for(int t = tid; t < tiles; t += kCoverThreads)
+            if(t > last)
+                ranges[t] = tail;
+    }
     if(tid == 0)
     {
         ranges[tiles] = (int32_t)s_carry; // K
+        if(J.last)
+            *J.last = last;
         for(int p = 0; p < plan.passes; ++p)
             atomicAdd(&hist[p * kBins32], negatives);
     }
     __syncthreads();
-    for(int j = tid; j < kMaxPasses32 * kBins32; j += kCoverThreads)
-        slot_hist[j] = hist[j];
+    if(slot_hist)
+        for(int j = tid; j < kMaxPasses32 * kBins32; j += kCoverThreads)
+            slot_hist[j] = hist[j];
 }
 
 // order: the buffer of order_layout(n) whose depth_keys and rects the projection has written
@@ -859,17 +978,22 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
     bool k_copy_ok = true;
     {
         hipStream_t cs = side ? side : stream;
-        const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
+        const ListGrid lg = list_grid(cam.image_width, cam.image_height);
+        const RangesLayout rl = ranges_layout(lg);
+        const int ntx = lg.ntx, nty = lg.nty;
         const int cells = (ntx + 1) * (nty + 1) + 1;
+        const int bcells = lg.shift ? (lg.nbx + 1) * (lg.nby + 1) + 1 : 0;
         int32_t* grid = reinterpret_cast<int32_t*>(base + o.cover);
-        // The corner grid is privatised in LDS whenever it fits (a 4K image has 32 776 cells =
+        int32_t* bin_grid = reinterpret_cast<int32_t*>(base + o.bin_cover);
+        int32_t* ranges = reinterpret_cast<int32_t*>(base + o.ranges);
+        // The corner grids are privatised in LDS whenever they fit (a 4K image has 32 776 cells =
         // 128 KB: one workgroup per CU); beyond 64 KB a kernel needs its limit raised first.
         // Global atomics are the fallback: correct for any grid, but 24 M same-line atomics
         // at 6 M Gaussians cost 0.6 ms and stall the sort passes that run beside them.
-        int use_lds = cells <= kCoverLdsCells ? 1 : 0;
-        if(!use_lds && cells <= kCoverLdsCellsLarge)
+        int use_lds = cells + bcells <= kCoverLdsCells ? 1 : 0;
+        if(!use_lds && cells + bcells <= kCoverLdsCellsLarge)
         {
-            const int bytes = cells * 4;
+            const int bytes = (cells + bcells) * 4;
             use_lds = hipFuncSetAttribute(reinterpret_cast<const void*>(tile_cover_kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess &&
                               hipFuncSetAttribute(reinterpret_cast<const void*>(tile_counts_kernel),
@@ -883,18 +1007,42 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
         {
             DSX_TIMED("tile_cover_kernel", cs);
             hipLaunchKernelGGL(tile_cover_kernel, dim3((unsigned)min((int64_t)kCoverBlocks, want)), dim3(kCoverThreads),
-                               use_lds ? (size_t)cells * 4 : 0, cs, reinterpret_cast<const uint2*>(base + o.rects), n,
-                               ntx, nty, use_lds, grid, reinterpret_cast<unsigned long long*>(base + o.key_count));
+                               use_lds ? (size_t)(cells + bcells) * 4 : 0, cs,
+                               reinterpret_cast<const uint2*>(base + o.rects), n, ntx, nty, lg.shift, lg.nbx, lg.nby,
+                               use_lds, grid, bin_grid, reinterpret_cast<unsigned long long*>(base + o.key_count));
         }
+        // the pairs of the lists that will be built: per bin when the lists are binned
         if(k_host)
-            k_copy_ok = hipMemcpyAsync(k_host, base + o.key_count, 8, hipMemcpyDeviceToHost, cs) == hipSuccess &&
+            k_copy_ok = hipMemcpyAsync(k_host, base + o.key_count + (lg.shift ? 8 : 0), 8, hipMemcpyDeviceToHost,
+                                       cs) == hipSuccess &&
                         hipEventRecord(k_copied, cs) == hipSuccess;
         {
+            CountsJobs jobs;
+            CountsJob& fine = jobs.job[0];
+            fine.grid = grid;
+            fine.ntx = ntx;
+            fine.nty = nty;
+            fine.plain = 0;
+            fine.plan = digits32(slot_bits(lg.tiles()));
+            fine.slot_hist = lg.shift ? nullptr : reinterpret_cast<uint32_t*>(base + o.slot_hist);
+            fine.ranges = ranges + rl.fine;
+            fine.last = lg.shift ? ranges + rl.last_tile : nullptr;
+            jobs.job[1] = fine;
+            if(lg.shift)
+            {
+                CountsJob& bins = jobs.job[1];
+                bins.grid = bin_grid;
+                bins.ntx = lg.nbx;
+                bins.nty = lg.nby;
+                bins.plain = 1;
+                bins.plan = digits32(slot_bits(lg.bins()));
+                bins.slot_hist = reinterpret_cast<uint32_t*>(base + o.slot_hist);
+                bins.ranges = ranges + rl.bins;
+                bins.last = nullptr;
+            }
             DSX_TIMED("tile_counts_kernel", cs);
-            hipLaunchKernelGGL(tile_counts_kernel, dim3(1), dim3(kCoverThreads), use_lds ? (size_t)cells * 4 : 0, cs,
-                               grid, ntx, nty, use_lds, digits32(slot_bits(ntx * nty)),
-                               reinterpret_cast<uint32_t*>(base + o.slot_hist),
-                               reinterpret_cast<int32_t*>(base + o.ranges));
+            hipLaunchKernelGGL(tile_counts_kernel, dim3(lg.shift ? 2 : 1), dim3(kCoverThreads),
+                               use_lds ? (size_t)cells * 4 : 0, cs, jobs, use_lds);
         }
     }
     bool joined = true;
@@ -928,7 +1076,8 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
     {
         DSX_TIMED("ordered_block_sums_kernel", stream);
         hipLaunchKernelGGL(ordered_block_sums_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
-                           reinterpret_cast<const uint2*>(base + o.rects_sorted), n, block_sums);
+                           reinterpret_cast<const uint2*>(base + o.rects_sorted), n,
+                           list_grid(cam.image_width, cam.image_height).shift, block_sums);
     }
     if(hipGetLastError() != hipSuccess)
         return finish(DSX_ERR_LAUNCH);
@@ -952,7 +1101,7 @@ template <typename SlotT>
 __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t* __restrict__ order,
                                                                   const uint2* __restrict__ rects_sorted,
                                                                   const uint32_t* __restrict__ block_offsets,
-                                                                  int64_t n, int64_t k, int ntx,
+                                                                  int64_t n, int64_t k, int ntx, int shift,
                                                                   SlotT* __restrict__ slots, int32_t* __restrict__ ids,
                                                                   const int32_t* __restrict__ ranges_in,
                                                                   int32_t* __restrict__ ranges_out, int range_count,
@@ -1017,12 +1166,20 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
         uint4 rec = make_uint4(0u, 0u, 0u, 0u);
         if(p < n)
         {
+            // (ntx: lists per row, i.e. bins per row when the lists are binned)
             const uint32_t g = order[p];
             const uint2 r = rects_sorted[p];
-            count = rect_count(r);
-            const uint32_t w = r.y & 0xffffu;
+            count = list_count(r, shift);
             const bool negative = (r.y >> 31) != 0;
-            rec.y = negative ? 0u : (r.x >> 16) * (uint32_t)ntx + (r.x & 0xffffu) + 1u;
+            uint32_t first_x = r.x & 0xffffu, first_y = r.x >> 16, w = r.y & 0xffffu;
+            if(shift && count && !negative)
+            {
+                const BinRect b = bin_rect(r, shift);
+                first_x = b.bx;
+                first_y = b.by;
+                w = b.bw;
+            }
+            rec.y = negative ? 0u : first_y * (uint32_t)ntx + first_x + 1u;
             rec.z = negative ? 0u : w;
             rec.w = g;
         }
@@ -1144,16 +1301,24 @@ ListsWorkspace lists_workspace(int64_t k, int num_tiles)
     return w;
 }
 
+// num_tiles: lists that the pairs are partitioned into (tiles, or bins when the lists are binned)
 template <typename SlotT>
 static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_tiles, const void* order,
                            int32_t* sorted_ids, int32_t* ranges, void* workspace, hipStream_t stream)
 {
     const OrderLayout o = order_layout(n, cam.image_width, cam.image_height);
     const char* obase = static_cast<const char*>(order);
+    const ListGrid lg = list_grid(cam.image_width, cam.image_height);
+    const RangesLayout rl = ranges_layout(lg);
+    // what the depth order left ready: everything but the part that the blend forward writes
+    const int ready_words = lg.shift ? rl.walk : rl.count;
     if(k <= 0)
     {
-        // no pairs: the ranges are all zero
-        return launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), num_tiles + 1, 0u, stream);
+        // no pairs: the ranges are all zero (and no tile is occupied)
+        int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), ready_words, 0u, stream);
+        if(rc == DSX_OK && lg.shift)
+            rc = launch_fill_u32(reinterpret_cast<uint32_t*>(ranges) + rl.last_tile, 1, 0xffffffffu, stream);
+        return rc;
     }
     const ListsWorkspace w = lists_workspace(k, num_tiles);
     const int bits = slot_bits(num_tiles);
@@ -1176,9 +1341,9 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
         hipLaunchKernelGGL(emit_ordered_kernel<SlotT>, dim3((unsigned)((k + chunk - 1) / chunk)), dim3(kProjBlock),
                            0, stream, reinterpret_cast<const uint32_t*>(obase + o.ids_a),
                            reinterpret_cast<const uint2*>(obase + o.rects_sorted),
-                           reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k, tiles_x(cam.image_width),
-                           slots_a, reinterpret_cast<int32_t*>(vals_a),
-                           reinterpret_cast<const int32_t*>(obase + o.ranges), ranges, num_tiles + 1,
+                           reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k,
+                           lg.shift ? lg.nbx : lg.ntx, lg.shift, slots_a, reinterpret_cast<int32_t*>(vals_a),
+                           reinterpret_cast<const int32_t*>(obase + o.ranges), ranges, ready_words,
                            reinterpret_cast<uint32_t*>(base + w.sort + sw.hist), (int64_t)(sw.bytes / 4), chunk);
     }
     DSX_LAUNCH_CHECK();
@@ -1194,11 +1359,13 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
     return vo == ids_final ? DSX_OK : DSX_ERR_RUNTIME;
 }
 
-// order: buffer of order_layout(n) after launch_depth_order.  Writes sorted_ids[k], ranges[T+1].
+// order: buffer of order_layout(n) after launch_depth_order.  Writes sorted_ids[k] and the ready part
+// of ranges (ranges_layout: per-tile ranges and, for binned lists, the last occupied tile and the
+// bins' ranges).
 int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
                       int32_t* ranges, void* workspace, hipStream_t stream)
 {
-    const int num_tiles = tiles_x(cam.image_width) * tiles_y(cam.image_height);
+    const int num_tiles = list_grid(cam.image_width, cam.image_height).lists();
     if(k >= (1ll << 30))
         return DSX_ERR_TOO_LARGE;
     if(n <= 0)

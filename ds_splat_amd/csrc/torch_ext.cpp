@@ -69,7 +69,7 @@ at::Tensor& pinned_key_count()
 
 } // namespace
 
-// image[H,W,3], radii[N], splats[N,12], sorted_ids[K], ranges[T+1], final_T[H,W], final_idx[H,W]
+// image[H,W,3], radii[N], splats[N,12], sorted_ids[K], ranges[dsx_ranges_count], final_T[H,W], final_idx[H,W]
 // (the 3-D covariances are not kept: the backward rebuilds them from scales and rotations, or
 // reads cov3d_precomp) and, when prepare_backward is set, the backward's gradient accumulator
 // [N,12], which the blend kernel prepares on the side: sums zeroed, conics in the spare places
@@ -105,9 +105,8 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
                               splats.data_ptr<float>(), radii.data_ptr<int32_t>(), nullptr, bs, order.data_ptr(),
                               order_bytes, k_host.data_ptr<int64_t>(), s));
     const int64_t k = *k_host.data_ptr<int64_t>();
-    const int64_t tiles = dsx_num_tiles((int32_t)width, (int32_t)height);
     at::Tensor sorted_ids = at::empty({k}, i32);
-    at::Tensor ranges = at::empty({tiles + 1}, i32);
+    at::Tensor ranges = at::empty({dsx_ranges_count((int32_t)width, (int32_t)height)}, i32);
     at::Tensor image = at::empty({height, width, 3}, f32);
     at::Tensor final_T = at::empty({height, width}, f32);
     at::Tensor final_idx = at::empty({height, width}, i32);

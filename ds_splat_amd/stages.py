@@ -91,9 +91,15 @@ def new_order(cam, n, device):
 
 def depth_order(cam, n, order):
     """Sorts the Gaussians of a projected `order` buffer by depth bits (stable).  Returns views
-    (depth order int32[n], scanned tile counts of its 256-Gaussian blocks int32[blocks + 1])."""
+    (depth order int32[n], scanned pair counts of its 256-Gaussian blocks int32[blocks + 1]; pairs
+    per bin when the lists are binned)."""
     lib = N.load()
     N.check(lib.dsx_depth_order(cam.ref, n, _ptr(order), order.numel(), _stream()))
+    return depth_order_view(n, order)
+
+
+def depth_order_view(n, order):
+    lib = N.load()
     p_order, p_off = C.c_void_p(), C.c_void_p()
     N.check(lib.dsx_order_view(n, _ptr(order), C.byref(p_order), C.byref(p_off)))
     base = order.data_ptr()
@@ -103,16 +109,46 @@ def depth_order(cam, n, order):
     return as_i32[o0:o0 + n], as_i32[o1:o1 + int(lib.dsx_num_blocks(n)) + 1]
 
 
-def tile_lists(cam, n, k, order, return_flags=False):
+def list_bin(cam):
+    """Tiles per side of the bins that the tile lists of this image size are built for (1: per tile)."""
+    return int(N.load().dsx_list_bin(cam.width, cam.height))
+
+
+def key_count(cam, n, order):
+    """Number of pairs of the lists that dsx_tile_lists will build from a depth-ordered `order`
+    buffer (per bin when the lists are binned): the last scanned block offset."""
+    _, offsets = depth_order_view(n, order)
+    return int(offsets[-1].item())
+
+
+def split_lists(cam, lists):
+    """The parts of a `ranges` buffer (dsx_ranges_count words): dict with 'fine' [T+1] and, for
+    binned lists, 'last_tile' (int tensor [1]), 'bins' [bins+1] and 'walk' [T, 4, 2]."""
+    t = cam.num_tiles
+    out = {"fine": lists[:t + 1]}
+    b = list_bin(cam)
+    if b > 1:
+        nbx, nby = (((cam.width + 15) // 16) + b - 1) // b, (((cam.height + 15) // 16) + b - 1) // b
+        out["last_tile"] = lists[t + 1:t + 2]
+        out["bins"] = lists[t + 2:t + 2 + nbx * nby + 1]
+        out["walk"] = lists[t + 3 + nbx * nby:].view(t, 4, 2)
+    return out
+
+
+def tile_lists(cam, n, k, order, return_flags=False, return_lists=False):
     """(sorted_ids[k], ranges[T+1]) from a depth-ordered `order` buffer; with return_flags also
-    the two give-up flags of the chained scans (depth sort, tile partition) as Python ints."""
+    the two give-up flags of the chained scans (depth sort, tile partition) as Python ints.
+    The ranges are the per-tile ranges as the reference defines them whatever the bin size;
+    sorted_ids holds the per-tile lists only with bins of one tile.  return_lists: the whole
+    `ranges` buffer (see split_lists) instead of its first T+1 words."""
     lib = N.load()
     dev = order.device
     sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
-    ranges = torch.empty((cam.num_tiles + 1,), dtype=torch.int32, device=dev)
+    lists = torch.empty((int(lib.dsx_ranges_count(cam.width, cam.height)),), dtype=torch.int32, device=dev)
     nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
-    N.check(lib.dsx_tile_lists(cam.ref, n, k, _ptr(order), _ptr(sorted_ids), _ptr(ranges), _ptr(ws), nbytes, _stream()))
+    N.check(lib.dsx_tile_lists(cam.ref, n, k, _ptr(order), _ptr(sorted_ids), _ptr(lists), _ptr(ws), nbytes, _stream()))
+    ranges = lists if return_lists else lists[:cam.num_tiles + 1]
     if not return_flags:
         return sorted_ids, ranges
     p_a, p_b = C.c_void_p(), C.c_void_p()
@@ -217,7 +253,8 @@ def _pinned_i64():
 class ForwardState:
     """What the forward keeps for the backward (the reference saves the analogous tensors
     on the autograd context, ds_splat/rasterizer.py:47-64)."""
-    __slots__ = ("splats", "radii", "cov3d", "sorted_ids", "ranges", "final_T", "final_idx", "num_keys", "grads")
+    __slots__ = ("splats", "radii", "cov3d", "sorted_ids", "lists", "ranges", "final_T", "final_idx", "num_keys",
+                 "grads")
 
 
 def sort_flag_indices(cam, n, k, order, workspace):
@@ -258,7 +295,9 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     if after_project is not None:
         after_project(order, n, k)
     st.sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
-    st.ranges = torch.empty((cam.num_tiles + 1,), dtype=torch.int32, device=dev)
+    # the whole `ranges` buffer, and its first T+1 words: the per-tile ranges as the reference defines them
+    st.lists = torch.empty((int(lib.dsx_ranges_count(cam.width, cam.height)),), dtype=torch.int32, device=dev)
+    st.ranges = st.lists[:cam.num_tiles + 1]
     image = torch.empty((cam.height, cam.width, 3), dtype=torch.float32, device=dev)
     st.final_T = torch.empty((cam.height, cam.width), dtype=torch.float32, device=dev)
     st.final_idx = torch.empty((cam.height, cam.width), dtype=torch.int32, device=dev)
@@ -266,7 +305,7 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
     st.grads = torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=dev) if prepare_grads else None
     N.check(lib.dsx_forward_finish(cam.ref, n, k, _ptr(st.splats), _ptr(order), _ptr(st.sorted_ids),
-                                   _ptr(st.ranges), _ptr(image), _ptr(st.final_T), _ptr(st.final_idx), _ptr(ws),
+                                   _ptr(st.lists), _ptr(image), _ptr(st.final_T), _ptr(st.final_idx), _ptr(ws),
                                    nbytes, _ptr(st.grads), stream))
     return image, st
 
@@ -281,7 +320,7 @@ def backward(cam, st, num_bases, means3d, scales, quats, v_image):
     grads = st.grads if prepared else torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=dev)
     st.grads = None
     N.check(lib.dsx_backward(cam.ref, n, num_bases, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(st.splats),
-                             _ptr(st.cov3d), _ptr(st.radii), _ptr(st.ranges), _ptr(st.sorted_ids), _ptr(st.final_T),
+                             _ptr(st.cov3d), _ptr(st.radii), _ptr(st.lists), _ptr(st.sorted_ids), _ptr(st.final_T),
                              _ptr(st.final_idx), _ptr(v_image), _ptr(grads), int(prepared), _ptr(o["v_mean3d"]),
                              _ptr(o["v_means2d"]), _ptr(o["v_shs"]), _ptr(o["v_colors"]), _ptr(o["v_opacity"]),
                              _ptr(o["v_scale"]), _ptr(o["v_quat"]), _ptr(o["v_cov3d"]), _stream()))

@@ -84,6 +84,22 @@ int64_t dsx_num_blocks(int64_t n);
 /* tiles of an image, and radix passes the sort runs for that many tiles */
 int32_t dsx_num_tiles(int32_t width, int32_t height);
 int32_t dsx_sort_passes(int32_t num_tiles);
+/* The tile lists of the whole forward (dsx_forward_project / dsx_forward_finish / dsx_backward,
+ * dsx_depth_order / dsx_tile_lists) are built per BIN of b x b tiles, b = 1, 2 or 4: a Gaussian
+ * enters the list of every bin that its tile rectangle touches, and a blend tile walks its bin's
+ * list and keeps the entries whose rectangle contains the tile.  With b = 1 the lists are the
+ * reference's own (sorted_ids is the value array of its sorted keys, bit for bit); with b > 1 the
+ * same entries reach every pixel in the same order, final_idx holds the same indices, and emission
+ * and partition handle a fraction of the pairs.  dsx_list_bin says which b the library uses for an
+ * image size (4 from 256 tiles on, else 1); dsx_set_list_bin forces one for the whole process
+ * (0: back to the library's choice) — not between the two halves of a forward or between a
+ * forward and its backward.  dsx_ranges_count: int32 words of the `ranges` buffer of those entry
+ * points: tiles + 1 words of per-tile ranges as the reference defines them and, for b > 1, the
+ * highest occupied tile, the bins' ranges and 8 words per tile that the blend forward leaves for
+ * the backward.  No counterpart in the reference. */
+int32_t dsx_list_bin(int32_t width, int32_t height);
+int dsx_set_list_bin(int tiles_per_side);
+int64_t dsx_ranges_count(int32_t width, int32_t height);
 /* bytes of `workspace` dsx_forward_finish / dsx_tile_lists need for k keys */
 size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height);
 /* bytes of `workspace` dsx_sort_pairs needs for k keys, and dsx_sort_pairs_u32 for count pairs */

@@ -31,3 +31,17 @@ def blend_form():
 
     yield force
     _native.check(lib.dsx_set_blend_pixels_per_lane(0))
+
+
+@pytest.fixture
+def list_bin():
+    """Returns a function that forces the bin size of the tile lists (1, 2 or 4 tiles a side; 0: the
+    library's choice) for the rest of the test; the library's own choice is restored afterwards."""
+    from ds_splat_amd import _native
+    lib = _native.load()
+
+    def force(tiles_per_side):
+        _native.check(lib.dsx_set_list_bin(int(tiles_per_side)))
+
+    yield force
+    _native.check(lib.dsx_set_list_bin(0))

@@ -133,3 +133,51 @@ def check_grads_against_bounds(got, B, bounds, mask, what=""):
             assert ratio[i] <= 1.0, "%s %s: error %.3e exceeds bound %.3e (want %.6e) at %s" % (
                 what, key, err[i], bound[i], want[i], i)
     return worst
+
+
+def tile_rects(S, radii, width, height):
+    """Tile rectangles [sx, ex) x [sy, ey) of every Gaussian from the oracle's pixel means and radii,
+    in float32 as cpp/rasterizer_kernels.cu:233-250 computes them (truncation, +1 on the upper
+    bound, clamped to the grid).  Checked by the caller against the oracle's own tile counts."""
+    ntx, nty = (width + 15) // 16, (height + 15) // 16
+    f = np.float32
+    cx, cy = S["means2d"][:, 0].astype(f) / f(16), S["means2d"][:, 1].astype(f) / f(16)
+    d = radii.astype(f) / f(16)
+    trunc = lambda v: np.clip(np.nan_to_num(v, nan=0.0, posinf=2.0e9, neginf=-2.0e9), -2.0e9, 2.0e9).astype(np.int64)
+    sx = np.clip(trunc(cx - d), 0, ntx)
+    ex = np.clip(trunc((cx + d) + f(1)), 0, ntx)
+    sy = np.clip(trunc(cy - d), 0, nty)
+    ey = np.clip(trunc((cy + d) + f(1)), 0, nty)
+    return sx, ex, sy, ey
+
+
+def expected_bin_lists(S, radii, width, height, bin_side):
+    """What binned tile lists must hold, from the oracle's stage-1 results: (ids, bin_ranges,
+    last_tile).  Slot 0 (positions [0, bin_ranges[0])) is the oracle's own list of pairs with a
+    negative depth; the list of a bin holds every Gaussian of non-negative depth (the last Gaussian
+    excepted: it never emits) whose tile rectangle touches the bin, once, by (depth bits, index)."""
+    n = len(radii)
+    ntx, nty = (width + 15) // 16, (height + 15) // 16
+    nbx, nby = (ntx + bin_side - 1) // bin_side, (nty + bin_side - 1) // bin_side
+    sx, ex, sy, ey = tile_rects(S, radii, width, height)
+    counts = (ex - sx) * (ey - sy) * (radii > 0)
+    assert (counts == S["tiles_touched"]).all()            # the helper agrees with the oracle's rectangles
+    bits = S["means2d"][:, 2].copy().view(np.uint32)
+    emits = (counts > 0)
+    emits[n - 1] = False
+    pos = emits & ((bits >> 31) == 0)
+    negatives = int(counts[emits & ~pos].sum())        # pairs of negative depth: they sort first
+    order = np.lexsort((np.arange(n), bits))                # by depth bits, then index
+    order = order[pos[order]]
+    per_bin = [[] for _ in range(nbx * nby)]
+    for g in order.tolist():
+        for by in range(sy[g] // bin_side, (ey[g] - 1) // bin_side + 1):
+            for bx in range(sx[g] // bin_side, (ex[g] - 1) // bin_side + 1):
+                per_bin[by * nbx + bx].append(g)
+    ids = [S["sorted_ids"][:negatives].astype(np.int64)]
+    ranges = [negatives]
+    for lst in per_bin:
+        ids.append(np.asarray(lst, np.int64))
+        ranges.append(ranges[-1] + len(lst))
+    last_rows = np.where(pos, (ey - 1) * ntx + (ex - 1), -1)
+    return np.concatenate(ids), np.asarray(ranges, np.int64), int(last_rows.max()) if n else -1

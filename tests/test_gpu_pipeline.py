@@ -78,24 +78,27 @@ def check_grads(leaves, B, ok, what=""):
     return worst
 
 
-@pytest.mark.parametrize("name,n,W,H,deg,scale_mul,bg,camera", [
-    ("cfg0", 16384, 256, 256, 0, 1.0, None, "identity"),            # workload cfg0 at full size
-    ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9), "identity"),
-    ("cfg1", 40000, 480, 270, 3, 1.0, None, "identity"),            # config 1 distributions, reduced size
-    ("cfg4", 3000, 320, 180, 3, 0.5, None, "identity"),             # heavy-overlap distributions, reduced size
-    ("cfg2", 30000, 333, 177, 2, 1.5, None, "identity"),            # ragged image (not a multiple of 16)
+# (bins: tiles per side of the bins the tile lists are built for; 0 = the library's choice by image size)
+@pytest.mark.parametrize("name,n,W,H,deg,scale_mul,bg,camera,bins", [
+    ("cfg0", 16384, 256, 256, 0, 1.0, None, "identity", 0),            # workload cfg0 at full size
+    ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9), "identity", 1),
+    ("cfg1", 40000, 480, 270, 3, 1.0, None, "identity", 4),            # config 1 distributions, reduced size
+    ("cfg4", 3000, 320, 180, 3, 0.5, None, "identity", 2),             # heavy-overlap distributions, reduced size
+    ("cfg2", 30000, 333, 177, 2, 1.5, None, "identity", 4),            # ragged image (not a multiple of 16)
     # general cameras: rotated + translated (campos != 0 matters at SH degree 3), a camera inside the
     # cloud (Gaussians behind it) with scale modifier 1.3, non-square pixels with scale modifier 0.7
-    ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9), "rotated"),
-    ("cfg0", 20000, 320, 200, 3, 2.0, None, "inside"),
-    ("cfg1", 40000, 480, 270, 3, 1.5, (0.5, 0.1, 0.3), "anisotropic"),
-    ("cfg4", 3000, 320, 180, 2, 0.5, None, "rotated"),
+    ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9), "rotated", 2),
+    ("cfg0", 20000, 320, 200, 3, 2.0, None, "inside", 4),
+    ("cfg1", 40000, 480, 270, 3, 1.5, (0.5, 0.1, 0.3), "anisotropic", 1),
+    ("cfg4", 3000, 320, 180, 2, 0.5, None, "rotated", 4),
+    ("cfg1", 40000, 1000, 520, 3, 2.0, (0.1, 0.2, 0.3), "rotated", 0),  # 63 x 33 tiles: ragged against the bins
 ])
 @pytest.mark.parametrize("pixels_per_lane", ["1", "4"])
-def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, bg, camera, pixels_per_lane,
-                                        blend_form):
+def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, bg, camera, bins, pixels_per_lane,
+                                        blend_form, list_bin):
     # both forms of the blend kernels, whatever the image size would pick
     blend_form(pixels_per_lane)
+    list_bin(bins)
     sc = set_camera(make_scene(name, n=n, width=W, height=H, sh_degree=deg), camera)
     image, radii, leaves = api_run(sc, scale_mul, bg=bg)
     img_o, radii_o, S, B = oracle_run(oracle, sc, scale_mul, bg=bg)
@@ -106,6 +109,8 @@ def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, b
     assert ok.mean() > 0.98, ok.mean()
     np.testing.assert_allclose(image.detach().cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
     T_gpu, idx_gpu, _ = gpu_forward_state(sc, scale_mul)
+    # final_idx holds the reference's indices whatever the bin size of the lists
+    assert (idx_gpu[ok] == S["final_idx"][ok]).all()
     # the two forwards disagree on a pixel's walk only where a decision was borderline
     assert (S["margin"][(T_gpu != S["final_T"]) & ~np.isclose(T_gpu, S["final_T"], rtol=1e-4, atol=0)] < 1e-4).all()
     gok = comparable_gaussians(S, B, W, T_gpu, idx_gpu)
@@ -115,17 +120,25 @@ def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, b
     assert (leaves["means2d"].grad[:, 2] == 0).all()
 
 
-def test_api_internal_integers_bit_exact(oracle):
-    """sorted order (stable tie-break) and tile ranges of the whole forward, bit for bit."""
+@pytest.mark.parametrize("bins", [1, 2, 4])
+def test_api_internal_integers_bit_exact(oracle, list_bin, bins):
+    """Tile ranges, tile counts, radii and last blended index of the whole forward, bit for bit,
+    whatever the bin size of the lists; with one list per tile also the sorted order itself
+    (stable tie-break) and the number of keys."""
     from ds_splat_amd import stages
+    list_bin(bins)
     sc = make_scene("cfg1", n=50000, width=640, height=360, sh_degree=1)
     cam = stages.camera_from_scene(sc, DEV)
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
     image, st = stages.forward(cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
     torch.cuda.synchronize()
     img_o, radii_o, S, _ = oracle_run(oracle, sc, 2.0, backward=False)
-    assert st.num_keys == S["num_keys"] > 100000
-    assert (st.sorted_ids.cpu().numpy() == S["sorted_ids"]).all()
+    assert S["num_keys"] > 100000
+    if bins == 1:
+        assert st.num_keys == S["num_keys"]
+        assert (st.sorted_ids.cpu().numpy() == S["sorted_ids"]).all()
+    else:
+        assert 0 < st.num_keys < S["num_keys"] // 2
     assert (st.ranges.cpu().numpy() == S["ranges"]).all()
     assert (st.radii.cpu().numpy() == radii_o).all()
     sp = st.splats.cpu().numpy()
@@ -342,11 +355,12 @@ def test_forward_core_raw_pointer_entry(oracle):
     ("cfg2", 300, 16, 16, 1.0),             # one tile
     ("cfg4", 100_000, 1920, 1080, 1.0),     # ~850 tiles per Gaussian
 ])
-def test_forward_lists_equal_the_64_bit_route(name, n, W, H, scale_mul):
-    """The whole forward's sorted ids and ranges (depth order + tile partition) against the
-    reference-shaped route (64-bit keys, radix sort, ranges from keys) at shapes the oracle is
-    too slow for."""
+def test_forward_lists_equal_the_64_bit_route(list_bin, name, n, W, H, scale_mul):
+    """The whole forward's sorted ids and ranges (depth order + tile partition, one list per tile)
+    against the reference-shaped route (64-bit keys, radix sort, ranges from keys) at shapes the
+    oracle is too slow for."""
     from ds_splat_amd import stages
+    list_bin(1)
     sc = make_scene(name, n=n, width=W, height=H)
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
     cam = stages.camera_from_scene(sc, DEV)
@@ -366,9 +380,10 @@ def test_forward_lists_equal_the_64_bit_route(name, n, W, H, scale_mul):
 
 
 # ------------------------------------------------------------------------- properties at full size
-def test_full_size_properties_cfg2():
-    """3M Gaussians, 1920x1080, SH3 (the headline shape): properties that need no oracle."""
+def test_full_size_properties_cfg2(list_bin):
+    """3M Gaussians, 1920x1080, SH3 (the headline shape): properties that need no oracle (one list per tile)."""
     from ds_splat_amd import stages
+    list_bin(1)
     sc = make_scene("cfg2")
     n = sc["n"]
     cam = stages.camera_from_scene(sc, DEV)
@@ -440,14 +455,15 @@ def test_full_size_properties_cfg2():
         assert (o[key][radii <= 0] == 0).all()
 
 
-def test_full_size_properties_cfg4_heavy_overlap():
+def test_full_size_properties_cfg4_heavy_overlap(list_bin):
     """The heavy-overlap shape at full size (1 M large Gaussians, 1080p, K = 858 M pairs: too many for
     the 64-bit route's buffers and for the CPU oracle in a test): what the lists must satisfy
     whatever their size.  K equals the sum of the tile counts; every Gaussian appears exactly
     tiles_touched times; the ranges partition [0, K); inside a tile the pairs are ordered by
     (depth bits, Gaussian index); every pair of a tile's list covers that tile; the image of an
-    all-white scene telescopes to 1 - final_T; forward and backward outputs are finite."""
+    all-white scene telescopes to 1 - final_T; forward and backward outputs are finite.  (One list per tile.)"""
     from ds_splat_amd import stages
+    list_bin(1)
     sc = make_scene("cfg4")
     n = sc["n"]
     cam = stages.camera_from_scene(sc, DEV)
@@ -508,7 +524,7 @@ GRADS_COMPARED_FLOOR = {"cfg1": 0.5, "cfg2": 0.5, "cfg4": 0.05}
 
 
 @pytest.mark.parametrize("workload", ["cfg1", "cfg2", "cfg4"])
-def test_full_size_against_the_openmp_oracle(workload):
+def test_full_size_against_the_openmp_oracle(workload, list_bin):
     """The three forward+backward shapes at full size (500 K Gaussians, the headline 3 M, and the
     heavy-overlap 1 M with its 858 M pairs; 1920x1080, SH3) against the oracle's OpenMP build
     (same source as the serial oracle, loops over Gaussians and tiles in parallel): integers,
@@ -518,7 +534,6 @@ def test_full_size_against_the_openmp_oracle(workload):
     from ds_splat_amd import stages
     omp = Oracle(omp=True)
     sc = make_scene(workload)
-    n = sc["n"]
     image, radii, leaves = api_run(sc)
     img_o, radii_o, S, B = oracle_run(omp, sc)
     assert (radii.cpu().numpy() == radii_o).all()
@@ -533,18 +548,31 @@ def test_full_size_against_the_openmp_oracle(workload):
     # the culled Gaussians compare trivially (all zeros): the floor is on the visible ones
     assert gok[visible].mean() > GRADS_COMPARED_FLOOR[workload], gok[visible].mean()
     del image, leaves
+    # the API ran with the library's own bin size for the lists: ranges and last blended indices
+    # are the reference's whatever that is ...
+    assert (st.ranges.cpu().numpy() == S["ranges"]).all()
+    assert (st.final_idx.cpu().numpy()[ok] == S["final_idx"][ok]).all()
+    print("%s: lists of %d x %d tiles, %d pairs instead of %d" % (
+        workload, stages.list_bin(stages.camera_from_scene(sc, DEV)), stages.list_bin(stages.camera_from_scene(sc, DEV)),
+        st.num_keys, S["num_keys"]))
+    del st
+    # ... and with one list per tile the sorted order itself is the reference's
+    list_bin(1)
+    _, _, st = gpu_forward_state(sc)
     assert st.num_keys == S["num_keys"]
     assert (st.ranges.cpu().numpy() == S["ranges"]).all()
     assert (st.sorted_ids.cpu().numpy() == S["sorted_ids"]).all()
     assert (st.final_idx.cpu().numpy()[ok] == S["final_idx"][ok]).all()
 
 
-def test_full_size_forward_cfg3_4k():
+@pytest.mark.parametrize("bins", [1, 0])
+def test_full_size_forward_cfg3_4k(list_bin, bins):
     """6M Gaussians at 3840x2160 (forward only): runs, sorted, deterministic, and equal to the
-    oracle's OpenMP build: radii, key count, ranges and the 36 M sorted ids bit for bit, the image
-    rtol 1e-4 / atol 1e-5 away from threshold decisions."""
+    oracle's OpenMP build: radii, ranges (and, with one list per tile, the key count and the 36 M
+    sorted ids) bit for bit, the image rtol 1e-4 / atol 1e-5 away from threshold decisions."""
     from oracle.binding import Oracle
     from ds_splat_amd import stages
+    list_bin(bins)
     sc = make_scene("cfg3")
     cam = stages.camera_from_scene(sc, DEV)
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
@@ -553,14 +581,17 @@ def test_full_size_forward_cfg3_4k():
     torch.cuda.synchronize()
     assert st.num_keys == st2.num_keys > 1_000_000
     assert torch.equal(st.sorted_ids, st2.sorted_ids) and torch.equal(image, image2)
-    assert (st.ranges[1:] >= st.ranges[:-1]).all() and int(st.ranges[-1]) == st.num_keys
+    assert (st.ranges[1:] >= st.ranges[:-1]).all() and (bins != 1 or int(st.ranges[-1]) == st.num_keys)
     assert torch.isfinite(image).all()
     del image2, st2
     img_o, radii_o, S, _ = oracle_run(Oracle(omp=True), sc, backward=False)
-    assert (st.radii.cpu().numpy() == radii_o).all() and st.num_keys == S["num_keys"]
+    assert (st.radii.cpu().numpy() == radii_o).all()
     assert (st.ranges.cpu().numpy() == S["ranges"]).all()
-    assert (st.sorted_ids.cpu().numpy() == S["sorted_ids"]).all()
+    if bins == 1:
+        assert st.num_keys == S["num_keys"]
+        assert (st.sorted_ids.cpu().numpy() == S["sorted_ids"]).all()
     ok = S["margin"] > 1e-4
+    assert (st.final_idx.cpu().numpy()[ok] == S["final_idx"][ok]).all()
     assert ok.mean() > 0.97
     np.testing.assert_allclose(image.cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
 

