@@ -28,23 +28,27 @@ FWD_PAIR_FLOPS, FWD_REJECT_FLOPS = 25, 15
 BWD_PAIR_FLOPS, BWD_REJECT_FLOPS = 72, 15
 
 
-# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counters (two rocprofv3 --pmc runs of this
-# script with --copy-probe, each counter scaled by its reading for the 1 GiB copy; summary in
-# profiles/cfg2_hbm_traffic_per_kernel.md).  Counters cannot be read from inside this process, so
-# the figures are quoted here and only reported when workload and key count are the profiled ones.
-MEASURED_TRAFFIC = {
-    ("cfg2", 32604809): {
-        "project_fwd_kernel": 857.7e6, "hist32_kernel": 13.3e6, "onesweep32_kernel<sort>": 103.4e6,
-        "ordered_block_sums_kernel": 24.4e6, "emit_ordered_kernel": 248.5e6,
-        "onesweep32_kernel<tile partition>": 376.3e6, "gaussian_bwd_kernel": 1020.2e6,
-        "blend_fwd_kernel": 329.5e6, "blend_bwd_kernel": 143.5e6,
-    },
-}
+def measured_traffic(workload, num_keys):
+    """HBM bytes per launch of every kernel from the FETCH_SIZE / WRITE_SIZE counters: the figures of
+    profiles/<workload>_hbm_traffic_per_kernel.json, which bench_profiles.py writes from two
+    rocprofv3 --pmc runs of this script (counters cannot be read from inside the process).  They are
+    reported only for the workload and pair count they were taken at; the record carries the
+    commit they were measured on.  Returns (dict kernel -> bytes, source description) or ({}, None)."""
+    path = os.path.join(ROOT, "profiles", "%s_hbm_traffic_per_kernel.json" % workload)
+    if not os.path.exists(path):
+        return {}, None
+    with open(path) as f:
+        rec = json.load(f)
+    if int(rec.get("num_keys", -1)) != int(num_keys):
+        return {}, None
+    return rec.get("kernels", {}), {"file": os.path.relpath(path, ROOT), "commit": rec.get("commit"),
+                                    "scale_fetch": rec.get("scale_fetch"), "scale_write": rec.get("scale_write")}
 
 
-def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, counters):
-    """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch."""
-    slot_bytes = 2 if tiles + 1 <= 65535 else 4
+def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters):
+    """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch.
+    k: pairs of the tile lists as built (per bin of tiles); lists: how many lists they are partitioned into."""
+    slot_bytes = 2 if lists + 1 <= 65535 else 4
     if kernel == "project_fwd_kernel":
         # inputs 44 + 12c bytes, outputs radii + splat record + depth key + tile rectangle (the 3-D
         # covariance is not stored on this path: the backward rebuilds it)
@@ -63,7 +67,7 @@ def algorithmic_work(kernel, n, k, pixels, tiles, coeffs, counters):
         return "hbm", 12 * n + (slot_bytes + 4) * k, "B"
     if kernel == "onesweep32_kernel<tile partition>":
         # tile partition: slot + id in and out, except that the last pass writes no slots (average per launch)
-        passes = 1 if tiles + 1 <= 256 else (2 if tiles + 1 <= 65536 else 3)
+        passes = 1 if lists + 1 <= 256 else (2 if lists + 1 <= 65536 else 3)
         return "hbm", (2 * (slot_bytes + 4) * passes - slot_bytes) * k / passes, "B"
     if kernel == "blend_fwd_kernel" and counters is not None:
         rej = counters.pairs_fwd - counters.pairs_fwd_applied
@@ -191,6 +195,19 @@ def main():
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
 
+    # what a step costs the host: the duration of the call with the GPU idle when it starts (kernel
+    # enqueues, allocations, and the one blocking wait for the pair count in the middle of the
+    # forward, which includes the projection's run time).  Outside the timed region.
+    host_steps = min(args.steps, 20)
+    host_ms = 0.0
+    for _ in range(host_steps):
+        torch.cuda.synchronize()
+        h0 = time.perf_counter()
+        step()
+        host_ms += (time.perf_counter() - h0) * 1e3
+    torch.cuda.synchronize()
+    host_ms_per_step = host_ms / host_steps
+
     # the same K steps again with an event pair around every kernel launch (on the launch stream):
     # per-kernel averages for the roofline.  The event packets cost about 0.15 ms per step, so this
     # pass is not the one `value` comes from; its own wall time is reported beside it.
@@ -218,6 +235,9 @@ def main():
     torch.cuda.synchronize()
     k = st.num_keys
     tiles = cam.num_tiles
+    list_bin = stages.list_bin(cam)
+    lists = (((W + 15) // 16 + list_bin - 1) // list_bin) * (((H + 15) // 16 + list_bin - 1) // list_bin)
+    k_per_tile = int(st.ranges[-1].item())      # pairs of the per-tile lists (the reference's K)
 
     # ---- CPU baseline: the oracle's OpenMP build on the host cores, same inputs -----------------
     cpu_baseline = None
@@ -229,23 +249,36 @@ def main():
                           sc["viewmatrix"].t().contiguous().numpy(), sc["projmatrix"].t().contiguous().numpy(),
                           sc["sh_degree"], sc["campos"].numpy())
         A = {kk: v.numpy() for kk, v in sc.items() if isinstance(v, torch.Tensor)}
-        c0 = time.perf_counter()
-        img_o, radii_o, ost = O.forward(s, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["shs"])
-        c1 = time.perf_counter()
-        if do_backward:
-            B = O.backward(s, ost, 16, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["v_image"])
-            counters = B["counters"]
-        else:
-            counters = O.state(s, ost, n)["counters"]
-        c2 = time.perf_counter()
-        k_cpu = int(O.lib.dsxo_state_num_keys(ost))
-        O.free(ost)
-        cpu_ms = (c2 - c0) * 1e3
+        # one warm-up iteration (first touch of ~2 GB of vectors), then the median of the timed ones;
+        # fewer timed iterations for the workloads whose iteration takes many seconds
+        timed = 3 if spec.name in ("cfg0", "cfg1", "cfg2") else 1
+        runs = []
+        k_cpu = -1
+        for it in range(1 + timed):
+            c0 = time.perf_counter()
+            img_o, radii_o, ost = O.forward(s, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["shs"])
+            c1 = time.perf_counter()
+            if do_backward:
+                B = O.backward(s, ost, 16, A["means_3d"], A["scales"], A["rotations"], A["opacities"], A["v_image"])
+                counters = B["counters"]
+                del B
+            else:
+                counters = O.state(s, ost, n)["counters"]
+            c2 = time.perf_counter()
+            k_cpu = int(O.lib.dsxo_state_num_keys(ost))
+            O.free(ost)
+            if it > 0:
+                runs.append(((c2 - c0) * 1e3, (c1 - c0) * 1e3, (c2 - c1) * 1e3))
+        runs.sort()
+        cpu_ms, fwd_ms, bwd_ms = runs[len(runs) // 2]
         cpu_baseline = {
             "value": round(cpu_ms, 1), "unit": "ms/iter", "cores": O.num_threads(), "kind": "port",
-            "sample": "1 iteration of the full %s workload (forward %.0f ms%s), C++ oracle built -O3 -fopenmp"
-                      % (spec.name, (c1 - c0) * 1e3, (", backward %.0f ms" % ((c2 - c1) * 1e3)) if do_backward else ""),
-            "keys_match_gpu": bool(k_cpu == k),
+            "iterations": timed, "warmup_iterations": 1,
+            "sample": "median of %d iteration%s of the full %s workload after 1 warm-up (forward %.0f ms%s), "
+                      "C++ oracle built -O3 -fopenmp" % (timed, "" if timed == 1 else "s", spec.name, fwd_ms,
+                                                         (", backward %.0f ms" % bwd_ms) if do_backward else ""),
+            "all_iterations_ms": [round(r[0], 1) for r in runs],
+            "keys_match_gpu": bool(k_cpu == k_per_tile),
         }
 
     # ---- roofline of the dominant kernel (and of the dominant HBM-bound one, if that is another) ----
@@ -253,10 +286,10 @@ def main():
     for name, (tot, cnt) in per_kernel.items():
         launches_per_step = cnt / args.steps
         avg = tot / cnt
-        bound, work, unit = algorithmic_work(name, n, k, W * H, tiles, coeffs, counters)
+        bound, work, unit = algorithmic_work(name, n, k, W * H, lists, coeffs, counters)
         table.append((tot / args.steps, name, avg, launches_per_step, bound, work, unit))
     table.sort(reverse=True)
-    measured = MEASURED_TRAFFIC.get((spec.name, int(k)), {}) if args.n is None else {}
+    measured, traffic_source = measured_traffic(spec.name, k) if args.n is None else ({}, None)
     roofline = None
     roofline_hbm = None
     for ms_step, name, avg, lps, bound, work, unit in table:
@@ -291,9 +324,16 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: %d Gaussians, %dx%d, SH degree %d, %s" %
                                (spec.name, n, W, H, sc["sh_degree"], "forward+backward" if do_backward else "forward"),
-                   "num_keys": int(k), "tiles": int(tiles)},
+                   "num_keys": int(k), "num_keys_per_tile_lists": k_per_tile, "tiles": int(tiles),
+                   "list_bin_tiles": list_bin, "lists": int(lists)},
         "mpix_per_s": round(W * H / (ms_per_step * 1e-3) / 1e6, 1),
         "ms_per_step_with_kernel_events": round(ms_per_step_traced, 4),
+        # the host's share of a step (enqueue + the wait for the pair count) and the device's (sum of the
+        # kernels' own times): the step is host-bound when the first is not hidden behind the second
+        "host_ms_per_step": round(host_ms_per_step, 4),
+        "kernels_sum_ms_per_step": round(sum(r[0] for r in table), 4),
+        "host_bound": bool(sum(r[0] for r in table) < 0.9 * ms_per_step),
+        "traffic_source": traffic_source,
         "kernels_ms_per_step": {name: round(ms_step, 4) for ms_step, name, *_ in table},
         "roofline": roofline,
         "roofline_hbm": roofline_hbm,
