@@ -91,7 +91,7 @@ int32_t dsx_sort_passes(int32_t num_tiles);
  * reference's own (sorted_ids is the value array of its sorted keys, bit for bit); with b > 1 the
  * same entries reach every pixel in the same order, final_idx holds the same indices, and emission
  * and partition handle a fraction of the pairs.  dsx_list_bin says which b the library uses for an
- * image size (4 from 256 tiles on, else 1); dsx_set_list_bin forces one for the whole process
+ * image size (4 from 2048 tiles on, else 1); dsx_set_list_bin forces one for the whole process
  * (0: back to the library's choice) — not between the two halves of a forward or between a
  * forward and its backward.  dsx_ranges_count: int32 words of the `ranges` buffer of those entry
  * points: tiles + 1 words of per-tile ranges as the reference defines them and, for b > 1, the

@@ -60,10 +60,10 @@ def test_host_helpers():
     assert (1 << 20) * 8 < lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080) < (1 << 20) * 9
     assert lib.dsx_set_list_bin(1) == 0
     assert (1 << 20) * 12 < lib.dsx_workspace_bytes(0, 1 << 20, 16400, 1040) < (1 << 20) * 13
-    # bins of the tile lists: 4 x 4 tiles from 256 tiles on, unless forced; the `ranges` buffer grows with them
+    # bins of the tile lists: 4 x 4 tiles from 2048 tiles on, unless forced; the `ranges` buffer grows with them
     assert lib.dsx_list_bin(1920, 1080) == 1 and lib.dsx_ranges_count(1920, 1080) == 8160 + 1
     assert lib.dsx_set_list_bin(0) == 0 and lib.dsx_set_list_bin(3) == -1
-    assert lib.dsx_list_bin(1920, 1080) == 4 and lib.dsx_list_bin(255, 255) == 4 and lib.dsx_list_bin(240, 240) == 1
+    assert lib.dsx_list_bin(1920, 1080) == 4 and lib.dsx_list_bin(1024, 512) == 4 and lib.dsx_list_bin(1024, 496) == 1
     assert lib.dsx_ranges_count(1920, 1080) == (8160 + 1) + 1 + (30 * 17 + 1) + 8 * 8160
     assert lib.dsx_ranges_count(240, 240) == 225 + 1
     assert lib.dsx_sort_workspace_bytes(1 << 20, 8160) > (1 << 20) * 12
