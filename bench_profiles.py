@@ -51,7 +51,7 @@ SQ_CMD = ("rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU 
 
 def short_name(kernel):
     """'void dsx::blend_fwd_kernel<4, true>(...)' -> 'blend_fwd_kernel<4, true>'"""
-    name = re.sub(r"^void ", "", kernel)
+    name = re.sub(r"^void ", "", kernel).replace("(anonymous namespace)::", "")
     depth, cut = 0, len(name)
     for i, ch in enumerate(name):           # the argument list starts at the first '(' outside <>
         if ch == "<":
@@ -61,7 +61,7 @@ def short_name(kernel):
         elif ch == "(" and depth == 0:
             cut = i
             break
-    return name[:cut].replace("dsx::", "").replace("(anonymous namespace)::", "")
+    return name[:cut].replace("dsx::", "")
 
 
 def trace_name(short):
