@@ -258,6 +258,15 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
         last[p] = 0;
     }
 
+    // the Gaussian ids of a round are fetched one round ahead: the gather of the splat records then
+    // waits for one memory round trip instead of two in a row
+    int g_ahead[kFwdBatch / DSX_WAVE];
+#pragma unroll
+    for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
+    {
+        const int e = start + h * DSX_WAVE + lane;
+        g_ahead[h] = e < end ? ids[e] : 0;
+    }
     for(int b = start; b < end; b += kFwdBatch)
     {
         if(alive == 0)
@@ -275,9 +284,10 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             const int e = b + slot;
             bool useful = false;
             bool member = false;
+            const int g = g_ahead[h];
+            g_ahead[h] = e + kFwdBatch < end ? ids[e + kFwdBatch] : 0;
             if(e < end)
             {
-                const int g = ids[e];
                 const float4* rec = splats + 3 * (int64_t)g;
                 const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
                 s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
@@ -625,6 +635,14 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
         hi = min(end - 1, m);
     }
 
+    // (ids one round ahead, as in the forward)
+    int g_ahead[kBwdBatch / DSX_WAVE];
+#pragma unroll
+    for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
+    {
+        const int e = hi - (h * DSX_WAVE + lane);
+        g_ahead[h] = e >= start ? ids[e] : 0;
+    }
     for(int top = hi; top >= start; top -= kBwdBatch)
     {
         if(kBinned && index_hi - above < src.fine_base) // every entry of the tile's own list has been met
@@ -640,9 +658,10 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             const int e = top - slot;
             bool useful = false;
             bool member = false;
+            const int g = g_ahead[h];
+            g_ahead[h] = e - kBwdBatch >= start ? ids[e - kBwdBatch] : 0;
             if(e >= start)
             {
-                const int g = ids[e];
                 const float4* rec = splats + 3 * (int64_t)g;
                 const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
                 s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
