@@ -302,7 +302,14 @@ int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const f
                         const float* cov3d, const int32_t* radii, const float* grads,
                         float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
                         float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d,
-                        hipStream_t stream, bool conic_in_grads = false);
+                        hipStream_t stream, bool conic_in_grads = false, bool outputs_cleared = false);
+// zeros in every output of launch_gaussian_bwd that is not null (it writes only the Gaussians that
+// have something to propagate; outputs_cleared tells it that this has been done)
+int launch_zero_outputs(int64_t n, int num_bases, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
+                        float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, hipStream_t stream);
+// the device's helper stream (default priority, made on first use, kept until the process ends;
+// shared by every caller thread), or nullptr when none can be made
+hipStream_t helper_stream();
 int launch_fill_u32(uint32_t* p, int64_t count, uint32_t value, hipStream_t stream);
 // 1 or 4: force that form of both blend kernels for the whole process; 0: choose by image size
 int set_blend_pixels_per_lane(int pixels);

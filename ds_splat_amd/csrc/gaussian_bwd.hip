@@ -1,8 +1,13 @@
 // Stages 5b + 5c for gfx950, fused: per-Gaussian backward of the SH colour (v_shs) and of the
 // projection (mean, scale, rotation, cov3D) from the screen-space gradients accumulated by the
-// blend backward.  One thread per Gaussian; the 192-byte v_shs rows are assembled in LDS per
-// wavefront and written with 16-byte coalesced stores.  Every output element is written
-// exactly once (zeros for culled Gaussians), so no output needs clearing beforehand.
+// blend backward.  Every output is linear in a Gaussian's nine accumulated sums, so a Gaussian
+// whose sums are all zero (culled, hidden behind others, or outside every tile that still had
+// light to give: the large majority of a dense scene) has all-zero gradients.  The outputs are
+// therefore cleared by a plain fill (zero_outputs_kernel, which the whole backward runs on a
+// second stream beside the blend kernel, whose work leaves the memory system idle), and this
+// kernel reads the 48-byte accumulator rows of a chunk of Gaussians, packs the ones with a
+// non-zero sum in LDS, and works on those only: one thread per such Gaussian, the 192-byte
+// v_shs rows assembled in LDS per wavefront and written with 16-byte stores.
 // Math follows cpp/gsplat/backward.cu:216-393, cpp/gsplat/helpers.cuh:68-220 and
 // cpp/gsplat/sh.cuh:95-186 of the reference; matrices below are indexed [row][col].
 #include "dsx_common.h"
@@ -78,289 +83,424 @@ __device__ __forceinline__ int sh_basis(int deg, float3 d, float* Y)
     return 16;
 }
 
+constexpr int kBwdChunk = 1024;                       // Gaussians per workgroup
+constexpr int kBwdPerThread = kBwdChunk / kProjBlock; // accumulator rows a thread tests
+
+// does any of the nine sums of an accumulator row differ from zero? (a NaN does)
+__device__ __forceinline__ bool any_sum(const float4& g0, const float4& g1, const float4& g2)
+{
+    return g0.x != 0.f || g0.y != 0.f || g0.z != 0.f || g0.w != 0.f || g1.x != 0.f || g1.y != 0.f || g1.z != 0.f ||
+           g1.w != 0.f || g2.x != 0.f;
+}
+
 __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const GaussianBwdParams p)
 {
     __shared__ float sh_lds[4][64 * kShPitchB];
+    __shared__ uint16_t s_list[kBwdChunk];                 // the chunk's Gaussians with work, in index order
+    __shared__ int s_count[kBwdPerThread * 4 + 1];         // per (row of the test, wavefront): how many
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int64_t i = (int64_t)blockIdx.x * kProjBlock + tid;
-    const bool live = i < p.n;
+    const int64_t chunk0 = (int64_t)blockIdx.x * kBwdChunk;
 
-    float v_rgb[3] = {0.f, 0.f, 0.f};
-    float3 mean = make_float3(0.f, 0.f, 0.f);
-    if(live)
+    // ---- which Gaussians of the chunk have anything to propagate ------------------------------
+    uint64_t mask[kBwdPerThread];
+#pragma unroll
+    for(int j = 0; j < kBwdPerThread; ++j)
     {
-        const float4 g0 = p.grads[3 * i], g1 = p.grads[3 * i + 1], g2 = p.grads[3 * i + 2];
-        const float v_x = g0.x, v_y = g0.y;
-        const float vc[3] = {g0.z, g0.w, g1.x};
-        const float v_o = g1.y;
-        v_rgb[0] = g1.z;
-        v_rgb[1] = g1.w;
-        v_rgb[2] = g2.x;
-        mean = make_float3(p.means3d[3 * i], p.means3d[3 * i + 1], p.means3d[3 * i + 2]);
-
-        // straight copies: screen-space mean gradient (z column zero), colour and opacity
-        // (every output is optional: a null pointer means that the caller has no use for it)
-        if(p.v_means2d)
-        {
-            p.v_means2d[3 * i] = v_x;
-            p.v_means2d[3 * i + 1] = v_y;
-            p.v_means2d[3 * i + 2] = 0.f;
-        }
-        if(p.v_colors)
-        {
-            p.v_colors[3 * i] = v_rgb[0];
-            p.v_colors[3 * i + 1] = v_rgb[1];
-            p.v_colors[3 * i + 2] = v_rgb[2];
-        }
-        if(p.v_opacity)
-            p.v_opacity[i] = v_o;
-
-        float vm[3] = {0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f};
-        float vc3[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if(p.radii[i] > 0)
-        {
-            const float* V = p.view;
-            const float R[3][3] = {{V[0], V[1], V[2]}, {V[4], V[5], V[6]}, {V[8], V[9], V[10]}};
-            const float t[3] = {R[0][0] * mean.x + R[0][1] * mean.y + R[0][2] * mean.z + V[3],
-                                R[1][0] * mean.x + R[1][1] * mean.y + R[1][2] * mean.z + V[7],
-                                R[2][0] * mean.x + R[2][1] * mean.y + R[2][2] * mean.z + V[11]};
-            // pixel mean -> view position -> world position
-            {
-                const float rw = 1.f / (t[2] + 1e-6f);
-                const float vpx = p.fx * v_x, vpy = p.fy * v_y;
-                const float vv[3] = {vpx * rw, vpy * rw, -(vpx * t[0] + vpy * t[1]) * rw * rw};
-#pragma unroll
-                for(int c = 0; c < 3; ++c)
-                    vm[c] = R[0][c] * vv[0] + R[1][c] * vv[1] + R[2][c] * vv[2];
-            }
-            // conic -> cov2d:  v_Sigma = -X G X, X = conic, G = symmetrised v_conic
-            float v_cov2d[3];
-            {
-                // the conic: behind the sums when the forward prepared the accumulator, else from the splat record
-                float4 q1;
-                if(p.conic_in_grads)
-                    q1 = make_float4(g2.y, g2.z, g2.w, 0.f);
-                else
-                    q1 = p.splats[3 * i + 1];
-                const float X[2][2] = {{q1.x, q1.y}, {q1.y, q1.z}};
-                const float G[2][2] = {{vc[0], 0.5f * vc[1]}, {0.5f * vc[1], vc[2]}};
-                float M[2][2], N[2][2];
-#pragma unroll
-                for(int r = 0; r < 2; ++r)
-#pragma unroll
-                    for(int c = 0; c < 2; ++c)
-                        M[r][c] = X[r][0] * G[0][c] + X[r][1] * G[1][c];
-#pragma unroll
-                for(int r = 0; r < 2; ++r)
-#pragma unroll
-                    for(int c = 0; c < 2; ++c)
-                        N[r][c] = M[r][0] * X[0][c] + M[r][1] * X[1][c];
-                v_cov2d[0] = -N[0][0];
-                v_cov2d[1] = -(N[0][1] + N[1][0]);
-                v_cov2d[2] = -N[1][1];
-            }
-            // EWA projection: cov2d = T Sigma T^T, T = J R (unclamped t, rz = 1/t.z)
-            {
-                const float rz = 1.f / t[2];
-                const float rz2 = rz * rz;
-                const float J[2][3] = {{p.fx * rz, 0.f, -p.fx * t[0] * rz2}, {0.f, p.fy * rz, -p.fy * t[1] * rz2}};
-                float T[2][3];
-#pragma unroll
-                for(int r = 0; r < 2; ++r)
-#pragma unroll
-                    for(int c = 0; c < 3; ++c)
-                        T[r][c] = J[r][0] * R[0][c] + J[r][1] * R[1][c] + J[r][2] * R[2][c];
-                // the covariance the forward projected: stored by it, or rebuilt here from scale and
-                // rotation with the forward's own routine (same bits; 24 bytes per Gaussian less to
-                // write there and to read here)
-                float c3[6];
-                if(p.cov3d)
-                {
-                    const float2* cs = reinterpret_cast<const float2*>(p.cov3d + 6 * i);
-                    const float2 c01 = cs[0], c23 = cs[1], c45 = cs[2];
-                    c3[0] = c01.x, c3[1] = c01.y, c3[2] = c23.x, c3[3] = c23.y, c3[4] = c45.x, c3[5] = c45.y;
-                }
-                else
-                {
-                    const float sc[3] = {p.scales[3 * i], p.scales[3 * i + 1], p.scales[3 * i + 2]};
-                    cov3d_from_scale_rot(sc, reinterpret_cast<const float4*>(p.quats)[i], p.glob, c3);
-                }
-                const float S[3][3] = {{c3[0], c3[1], c3[2]}, {c3[1], c3[3], c3[4]}, {c3[2], c3[4], c3[5]}};
-                const float Gc[2][2] = {{v_cov2d[0], 0.5f * v_cov2d[1]}, {0.5f * v_cov2d[1], v_cov2d[2]}};
-                // GT = Gc T (2x3)
-                float GT[2][3];
-#pragma unroll
-                for(int r = 0; r < 2; ++r)
-#pragma unroll
-                    for(int c = 0; c < 3; ++c)
-                        GT[r][c] = Gc[r][0] * T[0][c] + Gc[r][1] * T[1][c];
-                // v_Sigma = T^T Gc T (3x3)
-                float vS[3][3];
-#pragma unroll
-                for(int r = 0; r < 3; ++r)
-#pragma unroll
-                    for(int c = 0; c < 3; ++c)
-                        vS[r][c] = T[0][r] * GT[0][c] + T[1][r] * GT[1][c];
-                vc3[0] = vS[0][0];
-                vc3[1] = vS[0][1] + vS[1][0];
-                vc3[2] = vS[0][2] + vS[2][0];
-                vc3[3] = vS[1][1];
-                vc3[4] = vS[1][2] + vS[2][1];
-                vc3[5] = vS[2][2];
-                // v_T = Gc T Sigma^T + Gc^T T Sigma  (2x3); v_J = v_T R^T (2x3)
-                float vT[2][3];
-#pragma unroll
-                for(int r = 0; r < 2; ++r)
-#pragma unroll
-                    for(int c = 0; c < 3; ++c)
-                    {
-                        const float a = GT[r][0] * S[c][0] + GT[r][1] * S[c][1] + GT[r][2] * S[c][2];
-                        const float b = GT[r][0] * S[0][c] + GT[r][1] * S[1][c] + GT[r][2] * S[2][c];
-                        vT[r][c] = a + b;
-                    }
-                float vJ[2][3];
-#pragma unroll
-                for(int r = 0; r < 2; ++r)
-#pragma unroll
-                    for(int c = 0; c < 3; ++c)
-                        vJ[r][c] = vT[r][0] * R[c][0] + vT[r][1] * R[c][1] + vT[r][2] * R[c][2];
-                const float rz3 = rz2 * rz;
-                const float vt[3] = {-p.fx * rz2 * vJ[0][2], -p.fy * rz2 * vJ[1][2],
-                                     -p.fx * rz2 * vJ[0][0] + 2.f * p.fx * t[0] * rz3 * vJ[0][2] -
-                                         p.fy * rz2 * vJ[1][1] + 2.f * p.fy * t[1] * rz3 * vJ[1][2]};
-#pragma unroll
-                for(int c = 0; c < 3; ++c)
-                    vm[c] += vt[0] * R[0][c] + vt[1] * R[1][c] + vt[2] * R[2][c];
-            }
-            // cov3d = (Rq S)(Rq S)^T -> scale, quaternion (raw quaternion, no normalisation)
-            if(p.scales != nullptr)
-            {
-                const float vV[3][3] = {{vc3[0], 0.5f * vc3[1], 0.5f * vc3[2]},
-                                        {0.5f * vc3[1], vc3[3], 0.5f * vc3[4]},
-                                        {0.5f * vc3[2], 0.5f * vc3[4], vc3[5]}};
-                const float4 q = reinterpret_cast<const float4*>(p.quats)[i];
-                const float w = q.x, x = q.y, y = q.z, z = q.w;
-                const float Rq[3][3] = {
-                    {1.f - 2.f * (y * y + z * z), 2.f * (x * y - w * z), 2.f * (x * z + w * y)},
-                    {2.f * (x * y + w * z), 1.f - 2.f * (x * x + z * z), 2.f * (y * z - w * x)},
-                    {2.f * (x * z - w * y), 2.f * (y * z + w * x), 1.f - 2.f * (x * x + y * y)}};
-                const float s[3] = {p.glob * p.scales[3 * i], p.glob * p.scales[3 * i + 1],
-                                    p.glob * p.scales[3 * i + 2]};
-                float M[3][3], vM[3][3], vR[3][3];
-#pragma unroll
-                for(int r = 0; r < 3; ++r)
-#pragma unroll
-                    for(int c = 0; c < 3; ++c)
-                        M[r][c] = Rq[r][c] * s[c];
-                mat3_mul(vV, M, vM);
-#pragma unroll
-                for(int r = 0; r < 3; ++r)
-#pragma unroll
-                    for(int c = 0; c < 3; ++c)
-                        vM[r][c] *= 2.f;
-#pragma unroll
-                for(int c = 0; c < 3; ++c)
-                    vs[c] = (Rq[0][c] * vM[0][c] + Rq[1][c] * vM[1][c] + Rq[2][c] * vM[2][c]) * p.glob;
-#pragma unroll
-                for(int r = 0; r < 3; ++r)
-#pragma unroll
-                    for(int c = 0; c < 3; ++c)
-                        vR[r][c] = vM[r][c] * s[c];
-                vq[0] = 2.f * (x * (vR[2][1] - vR[1][2]) + y * (vR[0][2] - vR[2][0]) + z * (vR[1][0] - vR[0][1]));
-                vq[1] = 2.f * (-2.f * x * (vR[1][1] + vR[2][2]) + y * (vR[1][0] + vR[0][1]) +
-                               z * (vR[2][0] + vR[0][2]) + w * (vR[2][1] - vR[1][2]));
-                vq[2] = 2.f * (x * (vR[1][0] + vR[0][1]) - 2.f * y * (vR[0][0] + vR[2][2]) +
-                               z * (vR[2][1] + vR[1][2]) + w * (vR[0][2] - vR[2][0]));
-                vq[3] = 2.f * (x * (vR[2][0] + vR[0][2]) + y * (vR[2][1] + vR[1][2]) -
-                               2.f * z * (vR[0][0] + vR[1][1]) + w * (vR[1][0] - vR[0][1]));
-            }
-        }
-        if(p.v_mean3d)
-#pragma unroll
-            for(int c = 0; c < 3; ++c)
-                p.v_mean3d[3 * i + c] = vm[c];
-        if(p.v_scale)
-#pragma unroll
-            for(int c = 0; c < 3; ++c)
-                p.v_scale[3 * i + c] = vs[c];
-        if(p.v_quat)
-            reinterpret_cast<float4*>(p.v_quat)[i] = make_float4(vq[0], vq[1], vq[2], vq[3]);
-        if(p.v_cov3d)
-        {
-            float2* o = reinterpret_cast<float2*>(p.v_cov3d + 6 * i);
-            o[0] = make_float2(vc3[0], vc3[1]);
-            o[1] = make_float2(vc3[2], vc3[3]);
-            o[2] = make_float2(vc3[4], vc3[5]);
-        }
-    }
-
-    // ---- v_shs[b][c] = Y_b(dir) * v_rgb[c], zero above the active degree -------------------
-    if(p.v_shs == nullptr)
-        return;
-    const int row_floats = p.num_bases * 3;
-    float* rows = sh_lds[wave];
-    if(live)
-    {
-        float Y[16];
-        const float3 d = make_float3(mean.x - p.campos[0], mean.y - p.campos[1], mean.z - p.campos[2]);
-        const int nb = min(sh_basis(p.sh_degree, d, Y), p.num_bases);
-        float* r = rows + lane * kShPitchB;
-#pragma unroll
-        for(int b = 0; b < 16; ++b)
-        {
-            if(b < p.num_bases)
-            {
-                const float yb = b < nb ? Y[b] : 0.f;
-                r[3 * b] = b < nb ? yb * v_rgb[0] : 0.f;
-                r[3 * b + 1] = b < nb ? yb * v_rgb[1] : 0.f;
-                r[3 * b + 2] = b < nb ? yb * v_rgb[2] : 0.f;
-            }
-        }
+        const int64_t i = chunk0 + j * kProjBlock + tid;
+        bool work = false;
+        if(i < p.n)
+            work = any_sum(p.grads[3 * i], p.grads[3 * i + 1], p.grads[3 * i + 2]);
+        mask[j] = __ballot(work);
+        if(lane == 0)
+            s_count[j * 4 + wave] = __popcll(mask[j]);
     }
     __syncthreads();
-    const int64_t row0 = (int64_t)blockIdx.x * kProjBlock + wave * 64;
-    const int nrows = (int)max((int64_t)0, min((int64_t)64, p.n - row0));
-    if(row_floats == 48 && ((uintptr_t)p.v_shs & 15) == 0)
-    {
-        float4* dst = reinterpret_cast<float4*>(p.v_shs + row0 * 48);
-        const int chunks = nrows * 12;
+    int total = 0; // Gaussians with work in the rows before row j, then in the whole chunk
 #pragma unroll
-        for(int j = 0; j < 12; ++j)
+    for(int j = 0; j < kBwdPerThread; ++j)
+    {
+        int before = 0, row_total = 0; // ... in front of this wavefront's 64 of row j, and in row j
+#pragma unroll
+        for(int w = 0; w < 4; ++w)
         {
-            const int e = j * 64 + lane;
-            if(e < chunks)
+            const int c = s_count[j * 4 + w];
+            before += w < wave ? c : 0;
+            row_total += c;
+        }
+        if((mask[j] >> lane) & 1)
+            s_list[total + before + __popcll(mask[j] & ((1ull << lane) - 1ull))] = (uint16_t)(j * kProjBlock + tid);
+        total += row_total;
+    }
+    __syncthreads();
+
+    const int row_floats = p.num_bases * 3;
+    float* rows = sh_lds[wave];
+    for(int first = 0; first < total; first += kProjBlock)
+    {
+        const bool live = first + tid < total;
+        const int64_t i = live ? chunk0 + s_list[first + tid] : 0;
+
+        float v_rgb[3] = {0.f, 0.f, 0.f};
+        float3 mean = make_float3(0.f, 0.f, 0.f);
+        if(live)
+        {
+            const float4 g0 = p.grads[3 * i], g1 = p.grads[3 * i + 1], g2 = p.grads[3 * i + 2];
+            const float v_x = g0.x, v_y = g0.y;
+            const float vc[3] = {g0.z, g0.w, g1.x};
+            const float v_o = g1.y;
+            v_rgb[0] = g1.z;
+            v_rgb[1] = g1.w;
+            v_rgb[2] = g2.x;
+            mean = make_float3(p.means3d[3 * i], p.means3d[3 * i + 1], p.means3d[3 * i + 2]);
+
+            // straight copies: screen-space mean gradient (z column zero), colour and opacity
+            // (every output is optional: a null pointer means that the caller has no use for it)
+            if(p.v_means2d)
             {
-                const int row = e / 12;
-                const int c4 = e - row * 12;
-                const float* s = rows + row * kShPitchB + c4 * 4;
-                nt_store_f4(dst + e, make_float4(s[0], s[1], s[2], s[3]));
+                p.v_means2d[3 * i] = v_x;
+                p.v_means2d[3 * i + 1] = v_y;
+                p.v_means2d[3 * i + 2] = 0.f;
+            }
+            if(p.v_colors)
+            {
+                p.v_colors[3 * i] = v_rgb[0];
+                p.v_colors[3 * i + 1] = v_rgb[1];
+                p.v_colors[3 * i + 2] = v_rgb[2];
+            }
+            if(p.v_opacity)
+                p.v_opacity[i] = v_o;
+
+            float vm[3] = {0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f};
+            float vc3[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if(p.radii[i] > 0)
+            {
+                const float* V = p.view;
+                const float R[3][3] = {{V[0], V[1], V[2]}, {V[4], V[5], V[6]}, {V[8], V[9], V[10]}};
+                const float t[3] = {R[0][0] * mean.x + R[0][1] * mean.y + R[0][2] * mean.z + V[3],
+                                    R[1][0] * mean.x + R[1][1] * mean.y + R[1][2] * mean.z + V[7],
+                                    R[2][0] * mean.x + R[2][1] * mean.y + R[2][2] * mean.z + V[11]};
+                // pixel mean -> view position -> world position
+                {
+                    const float rw = 1.f / (t[2] + 1e-6f);
+                    const float vpx = p.fx * v_x, vpy = p.fy * v_y;
+                    const float vv[3] = {vpx * rw, vpy * rw, -(vpx * t[0] + vpy * t[1]) * rw * rw};
+#pragma unroll
+                    for(int c = 0; c < 3; ++c)
+                        vm[c] = R[0][c] * vv[0] + R[1][c] * vv[1] + R[2][c] * vv[2];
+                }
+                // conic -> cov2d:  v_Sigma = -X G X, X = conic, G = symmetrised v_conic
+                float v_cov2d[3];
+                {
+                    // the conic: behind the sums when the forward prepared the accumulator, else from the splat record
+                    float4 q1;
+                    if(p.conic_in_grads)
+                        q1 = make_float4(g2.y, g2.z, g2.w, 0.f);
+                    else
+                        q1 = p.splats[3 * i + 1];
+                    const float X[2][2] = {{q1.x, q1.y}, {q1.y, q1.z}};
+                    const float G[2][2] = {{vc[0], 0.5f * vc[1]}, {0.5f * vc[1], vc[2]}};
+                    float M[2][2], N[2][2];
+#pragma unroll
+                    for(int r = 0; r < 2; ++r)
+#pragma unroll
+                        for(int c = 0; c < 2; ++c)
+                            M[r][c] = X[r][0] * G[0][c] + X[r][1] * G[1][c];
+#pragma unroll
+                    for(int r = 0; r < 2; ++r)
+#pragma unroll
+                        for(int c = 0; c < 2; ++c)
+                            N[r][c] = M[r][0] * X[0][c] + M[r][1] * X[1][c];
+                    v_cov2d[0] = -N[0][0];
+                    v_cov2d[1] = -(N[0][1] + N[1][0]);
+                    v_cov2d[2] = -N[1][1];
+                }
+                // EWA projection: cov2d = T Sigma T^T, T = J R (unclamped t, rz = 1/t.z)
+                {
+                    const float rz = 1.f / t[2];
+                    const float rz2 = rz * rz;
+                    const float J[2][3] = {{p.fx * rz, 0.f, -p.fx * t[0] * rz2}, {0.f, p.fy * rz, -p.fy * t[1] * rz2}};
+                    float T[2][3];
+#pragma unroll
+                    for(int r = 0; r < 2; ++r)
+#pragma unroll
+                        for(int c = 0; c < 3; ++c)
+                            T[r][c] = J[r][0] * R[0][c] + J[r][1] * R[1][c] + J[r][2] * R[2][c];
+                    // the covariance the forward projected: stored by it, or rebuilt here from scale and
+                    // rotation with the forward's own routine (same bits; 24 bytes per Gaussian less to
+                    // write there and to read here)
+                    float c3[6];
+                    if(p.cov3d)
+                    {
+                        const float2* cs = reinterpret_cast<const float2*>(p.cov3d + 6 * i);
+                        const float2 c01 = cs[0], c23 = cs[1], c45 = cs[2];
+                        c3[0] = c01.x, c3[1] = c01.y, c3[2] = c23.x, c3[3] = c23.y, c3[4] = c45.x, c3[5] = c45.y;
+                    }
+                    else
+                    {
+                        const float sc[3] = {p.scales[3 * i], p.scales[3 * i + 1], p.scales[3 * i + 2]};
+                        cov3d_from_scale_rot(sc, reinterpret_cast<const float4*>(p.quats)[i], p.glob, c3);
+                    }
+                    const float S[3][3] = {{c3[0], c3[1], c3[2]}, {c3[1], c3[3], c3[4]}, {c3[2], c3[4], c3[5]}};
+                    const float Gc[2][2] = {{v_cov2d[0], 0.5f * v_cov2d[1]}, {0.5f * v_cov2d[1], v_cov2d[2]}};
+                    // GT = Gc T (2x3)
+                    float GT[2][3];
+#pragma unroll
+                    for(int r = 0; r < 2; ++r)
+#pragma unroll
+                        for(int c = 0; c < 3; ++c)
+                            GT[r][c] = Gc[r][0] * T[0][c] + Gc[r][1] * T[1][c];
+                    // v_Sigma = T^T Gc T (3x3)
+                    float vS[3][3];
+#pragma unroll
+                    for(int r = 0; r < 3; ++r)
+#pragma unroll
+                        for(int c = 0; c < 3; ++c)
+                            vS[r][c] = T[0][r] * GT[0][c] + T[1][r] * GT[1][c];
+                    vc3[0] = vS[0][0];
+                    vc3[1] = vS[0][1] + vS[1][0];
+                    vc3[2] = vS[0][2] + vS[2][0];
+                    vc3[3] = vS[1][1];
+                    vc3[4] = vS[1][2] + vS[2][1];
+                    vc3[5] = vS[2][2];
+                    // v_T = Gc T Sigma^T + Gc^T T Sigma  (2x3); v_J = v_T R^T (2x3)
+                    float vT[2][3];
+#pragma unroll
+                    for(int r = 0; r < 2; ++r)
+#pragma unroll
+                        for(int c = 0; c < 3; ++c)
+                        {
+                            const float a = GT[r][0] * S[c][0] + GT[r][1] * S[c][1] + GT[r][2] * S[c][2];
+                            const float b = GT[r][0] * S[0][c] + GT[r][1] * S[1][c] + GT[r][2] * S[2][c];
+                            vT[r][c] = a + b;
+                        }
+                    float vJ[2][3];
+#pragma unroll
+                    for(int r = 0; r < 2; ++r)
+#pragma unroll
+                        for(int c = 0; c < 3; ++c)
+                            vJ[r][c] = vT[r][0] * R[c][0] + vT[r][1] * R[c][1] + vT[r][2] * R[c][2];
+                    const float rz3 = rz2 * rz;
+                    const float vt[3] = {-p.fx * rz2 * vJ[0][2], -p.fy * rz2 * vJ[1][2],
+                                         -p.fx * rz2 * vJ[0][0] + 2.f * p.fx * t[0] * rz3 * vJ[0][2] -
+                                             p.fy * rz2 * vJ[1][1] + 2.f * p.fy * t[1] * rz3 * vJ[1][2]};
+#pragma unroll
+                    for(int c = 0; c < 3; ++c)
+                        vm[c] += vt[0] * R[0][c] + vt[1] * R[1][c] + vt[2] * R[2][c];
+                }
+                // cov3d = (Rq S)(Rq S)^T -> scale, quaternion (raw quaternion, no normalisation)
+                if(p.scales != nullptr)
+                {
+                    const float vV[3][3] = {{vc3[0], 0.5f * vc3[1], 0.5f * vc3[2]},
+                                            {0.5f * vc3[1], vc3[3], 0.5f * vc3[4]},
+                                            {0.5f * vc3[2], 0.5f * vc3[4], vc3[5]}};
+                    const float4 q = reinterpret_cast<const float4*>(p.quats)[i];
+                    const float w = q.x, x = q.y, y = q.z, z = q.w;
+                    const float Rq[3][3] = {
+                        {1.f - 2.f * (y * y + z * z), 2.f * (x * y - w * z), 2.f * (x * z + w * y)},
+                        {2.f * (x * y + w * z), 1.f - 2.f * (x * x + z * z), 2.f * (y * z - w * x)},
+                        {2.f * (x * z - w * y), 2.f * (y * z + w * x), 1.f - 2.f * (x * x + y * y)}};
+                    const float s[3] = {p.glob * p.scales[3 * i], p.glob * p.scales[3 * i + 1],
+                                        p.glob * p.scales[3 * i + 2]};
+                    float M[3][3], vM[3][3], vR[3][3];
+#pragma unroll
+                    for(int r = 0; r < 3; ++r)
+#pragma unroll
+                        for(int c = 0; c < 3; ++c)
+                            M[r][c] = Rq[r][c] * s[c];
+                    mat3_mul(vV, M, vM);
+#pragma unroll
+                    for(int r = 0; r < 3; ++r)
+#pragma unroll
+                        for(int c = 0; c < 3; ++c)
+                            vM[r][c] *= 2.f;
+#pragma unroll
+                    for(int c = 0; c < 3; ++c)
+                        vs[c] = (Rq[0][c] * vM[0][c] + Rq[1][c] * vM[1][c] + Rq[2][c] * vM[2][c]) * p.glob;
+#pragma unroll
+                    for(int r = 0; r < 3; ++r)
+#pragma unroll
+                        for(int c = 0; c < 3; ++c)
+                            vR[r][c] = vM[r][c] * s[c];
+                    vq[0] = 2.f * (x * (vR[2][1] - vR[1][2]) + y * (vR[0][2] - vR[2][0]) + z * (vR[1][0] - vR[0][1]));
+                    vq[1] = 2.f * (-2.f * x * (vR[1][1] + vR[2][2]) + y * (vR[1][0] + vR[0][1]) +
+                                   z * (vR[2][0] + vR[0][2]) + w * (vR[2][1] - vR[1][2]));
+                    vq[2] = 2.f * (x * (vR[1][0] + vR[0][1]) - 2.f * y * (vR[0][0] + vR[2][2]) +
+                                   z * (vR[2][1] + vR[1][2]) + w * (vR[0][2] - vR[2][0]));
+                    vq[3] = 2.f * (x * (vR[2][0] + vR[0][2]) + y * (vR[2][1] + vR[1][2]) -
+                                   2.f * z * (vR[0][0] + vR[1][1]) + w * (vR[1][0] - vR[0][1]));
+                }
+            }
+            if(p.v_mean3d)
+#pragma unroll
+                for(int c = 0; c < 3; ++c)
+                    p.v_mean3d[3 * i + c] = vm[c];
+            if(p.v_scale)
+#pragma unroll
+                for(int c = 0; c < 3; ++c)
+                    p.v_scale[3 * i + c] = vs[c];
+            if(p.v_quat)
+                reinterpret_cast<float4*>(p.v_quat)[i] = make_float4(vq[0], vq[1], vq[2], vq[3]);
+            if(p.v_cov3d)
+            {
+                float2* o = reinterpret_cast<float2*>(p.v_cov3d + 6 * i);
+                o[0] = make_float2(vc3[0], vc3[1]);
+                o[1] = make_float2(vc3[2], vc3[3]);
+                o[2] = make_float2(vc3[4], vc3[5]);
+            }
+        }
+
+        // ---- v_shs[b][c] = Y_b(dir) * v_rgb[c], zero above the active degree -------------------
+        if(p.v_shs == nullptr)
+            continue;
+        if(first > 0)
+            __syncthreads(); // the rows of the last round have been read
+        if(live)
+        {
+            float Y[16];
+            const float3 d = make_float3(mean.x - p.campos[0], mean.y - p.campos[1], mean.z - p.campos[2]);
+            const int nb = min(sh_basis(p.sh_degree, d, Y), p.num_bases);
+            float* r = rows + lane * kShPitchB;
+#pragma unroll
+            for(int b = 0; b < 16; ++b)
+            {
+                if(b < p.num_bases)
+                {
+                    const float yb = b < nb ? Y[b] : 0.f;
+                    r[3 * b] = b < nb ? yb * v_rgb[0] : 0.f;
+                    r[3 * b + 1] = b < nb ? yb * v_rgb[1] : 0.f;
+                    r[3 * b + 2] = b < nb ? yb * v_rgb[2] : 0.f;
+                }
+            }
+        }
+        __syncthreads();
+        // the wavefront's rows go out 16 bytes per lane: twelve lanes per row when a row is 48 floats
+        const int wave_first = first + wave * 64;
+        const int nrows = max(0, min(64, total - wave_first));
+        if(row_floats == 48 && ((uintptr_t)p.v_shs & 15) == 0)
+        {
+            const int chunks = nrows * 12;
+#pragma unroll
+            for(int j = 0; j < 12; ++j)
+            {
+                const int e = j * 64 + lane;
+                if(e < chunks)
+                {
+                    const int row = e / 12;
+                    const int c4 = e - row * 12;
+                    const float* s = rows + row * kShPitchB + c4 * 4;
+                    float4* dst = reinterpret_cast<float4*>(p.v_shs + (chunk0 + s_list[wave_first + row]) * 48);
+                    nt_store_f4(dst + c4, make_float4(s[0], s[1], s[2], s[3]));
+                }
+            }
+        }
+        else
+        {
+            const int count = nrows * row_floats;
+            for(int e = lane; e < count; e += 64)
+            {
+                const int row = e / row_floats;
+                const int c = e - row * row_floats;
+                p.v_shs[(chunk0 + s_list[wave_first + row]) * row_floats + c] = rows[row * kShPitchB + c];
             }
         }
     }
-    else
+}
+
+// ---- the outputs' zeros: up to eight arrays in one launch --------------------------------------
+// The arrays' 16-byte-aligned middles form one range of 16-byte stores that the workgroups share
+// evenly (v_shs alone is three quarters of it); the few floats in front of and behind a middle are
+// stored one by one.  Few workgroups, one per two CUs: the kernel runs beside the blend backward, which
+// wants every wavefront slot, and 512 wavefronts still store 780 MB well within that kernel's time
+// (3 M Gaussians at 1920x1080, whole step: 0.854 ms with 96 or 128 workgroups, 0.862 with 192,
+// 0.896 with 256, 0.872 with 4096).
+constexpr int kZeroWorkgroups = 128;
+
+struct ZeroJobs
+{
+    float* ptr[8];     // null: not wanted
+    int64_t floats[8]; // length of the array
+    int64_t end[8];    // 16-byte stores of this and all earlier arrays
+};
+
+__global__ __launch_bounds__(kProjBlock) void zero_outputs_kernel(const ZeroJobs jobs)
+{
+    const int64_t total = jobs.end[7];
+    const int64_t share = (total + gridDim.x - 1) / gridDim.x;
+    const int64_t lo = (int64_t)blockIdx.x * share, hi = min(lo + share, total);
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for(int j = 0; j < 8; ++j)
     {
-        float* dst = p.v_shs + row0 * row_floats;
-        const int total = nrows * row_floats;
-        for(int e = lane; e < total; e += 64)
+        float* ptr = jobs.ptr[j];
+        if(ptr == nullptr)
+            continue;
+        const int64_t start = j ? jobs.end[j - 1] : 0;
+        const int head = (int)(((16 - ((uintptr_t)ptr & 15)) & 15) / 4);
+        float4* q = reinterpret_cast<float4*>(ptr + head) - start;
+        for(int64_t i = max(lo, start) + threadIdx.x; i < min(hi, jobs.end[j]); i += kProjBlock)
+            nt_store_f4(q + i, zero);
+        if(blockIdx.x == 0 && threadIdx.x < 4)
         {
-            const int row = e / row_floats;
-            const int c = e - row * row_floats;
-            dst[e] = rows[row * kShPitchB + c];
+            const int64_t n = jobs.floats[j];
+            if((int)threadIdx.x < head && (int64_t)threadIdx.x < n)
+                ptr[threadIdx.x] = 0.f;
+            const int64_t t = head + (jobs.end[j] - start) * 4 + threadIdx.x;
+            if(t < n)
+                ptr[t] = 0.f;
         }
     }
+}
+
+int launch_zero_outputs(int64_t n, int num_bases, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
+                        float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, hipStream_t stream)
+{
+    if(n <= 0)
+        return DSX_OK;
+    ZeroJobs jobs;
+    float* ptrs[8] = {v_mean3d, v_means2d, num_bases > 0 ? v_shs : nullptr, v_colors, v_opacity, v_scale, v_quat, v_cov3d};
+    const int64_t per[8] = {3, 3, 3 * (int64_t)num_bases, 3, 1, 3, 4, 6};
+    int64_t stores = 0;
+    bool any = false;
+    for(int j = 0; j < 8; ++j)
+    {
+        jobs.ptr[j] = ptrs[j];
+        jobs.floats[j] = ptrs[j] ? n * per[j] : 0;
+        if(ptrs[j])
+        {
+            any = true;
+            const int64_t head = (int64_t)(((16 - ((uintptr_t)ptrs[j] & 15)) & 15) / 4);
+            stores += jobs.floats[j] > head ? (jobs.floats[j] - head) / 4 : 0;
+        }
+        jobs.end[j] = stores;
+    }
+    if(!any)
+        return DSX_OK;
+    // at least 16 stores per thread, at most kZeroWorkgroups workgroups
+    const int64_t want = (stores + (int64_t)kProjBlock * 16 - 1) / ((int64_t)kProjBlock * 16);
+    const unsigned blocks = (unsigned)max((int64_t)1, min(want, (int64_t)kZeroWorkgroups));
+    {
+        DSX_TIMED("zero_outputs_kernel", stream);
+        hipLaunchKernelGGL(zero_outputs_kernel, dim3(blocks), dim3(kProjBlock), 0, stream, jobs);
+    }
+    DSX_LAUNCH_CHECK();
+    return DSX_OK;
 }
 
 int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d, const float* scales,
                         const float* quats, const float* splats, const float* cov3d, const int32_t* radii,
                         const float* grads, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
                         float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, hipStream_t stream,
-                        bool conic_in_grads)
+                        bool conic_in_grads, bool outputs_cleared)
 {
     if(n == 0)
         return DSX_OK;
+    if(!outputs_cleared)
+        if(int rc = launch_zero_outputs(n, num_bases, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat,
+                                        v_cov3d, stream))
+            return rc;
     GaussianBwdParams p;
     p.n = n;
     p.means3d = means3d;
@@ -390,7 +530,7 @@ int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const f
     p.sh_degree = cam.sh_degree;
     p.num_bases = num_bases;
     p.conic_in_grads = conic_in_grads ? 1 : 0;
-    const int64_t blocks = (n + kProjBlock - 1) / kProjBlock;
+    const int64_t blocks = (n + kBwdChunk - 1) / kBwdChunk;
     {
         DSX_TIMED("gaussian_bwd_kernel", stream);
         hipLaunchKernelGGL(gaussian_bwd_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, p);

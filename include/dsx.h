@@ -211,7 +211,12 @@ int dsx_blend_bwd(const dsx_camera* cam, int64_t n, const int32_t* ranges,
  * (may be NULL), v_colors[n*3], v_opacity[n], v_scale[n*3], v_quat[n*4], v_cov3d[n*6].
  * Any output may be NULL: that gradient is then not written (the reference computes all of them
  * and lets autograd drop those of inputs that were not given, cpp/rasterizer_torch.cu:315;
- * here an unwanted one costs no store).
+ * here an unwanted one costs no store).  v_quat must be 16-byte aligned and v_cov3d 8-byte aligned;
+ * the others need only the alignment of a float.
+ * Every output is linear in the nine sums of the Gaussian's accumulator record, so the call first
+ * clears the outputs with a fill and then works on the Gaussians that have a non-zero sum only
+ * (a NaN counts as one); a Gaussian without one gets +0 everywhere, where the reference would
+ * compute a signed zero, or NaN for a non-finite input of that Gaussian.
  * scales/quats may be NULL when the forward used cov3d_precomp (v_scale, v_quat zeroed).
  * cov3d is what the forward stored, or cov3d_precomp itself, or NULL when scales/quats are
  * given: the kernel then rebuilds it with the forward's own routine (bit-identical). */

@@ -497,3 +497,77 @@ def test_gaussian_bwd_vs_oracle(oracle, sh_degree, num_bases, n, camera):
     torch.cuda.synchronize()
     for key in o:
         assert torch.equal(o[key], o2[key]), key
+
+
+@pytest.mark.parametrize("touched_share,n", [(0.03, 20000), (0.0, 3000), (0.5, 5000)])
+def test_gaussian_bwd_sparse_sums_and_unaligned_outputs(oracle, touched_share, n):
+    """The kernel works only on Gaussians with a non-zero sum and a fill writes the zeros of all the
+    others: rows with a single non-zero sum (each of the nine places in turn) and a NaN row must be
+    found, the untouched rows must read exactly zero, and outputs that start at any float (the fill
+    stores 16 bytes at a time behind a scalar head) must be written to their last element and not
+    beyond."""
+    st_ = _stages()
+    lib = st_.N.load()
+    num_bases = 16
+    sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=256, H=256, sh_degree=3, seed=77 + n, scale_mul=2.0,
+                                               camera="rotated")
+    oracle.free(st)
+    rng = np.random.default_rng(n + 1)
+    grads = np.zeros((n, 12), np.float32)
+    rows = np.flatnonzero(rng.random(n) < touched_share)
+    grads[rows, :9] = rng.normal(size=(len(rows), 9)).astype(np.float32)
+    single = rng.choice(n, size=90, replace=False)   # one sum each, every place ten times over
+    if touched_share == 0.0:
+        single = single[:0]
+    grads[single, :9] = 0
+    grads[single, np.arange(len(single)) % 9] = rng.normal(size=len(single)).astype(np.float32) + 3.0
+    grads[:, 9:] = S["conic"]  # what the forward leaves there; must not count as a sum
+    v_xy, v_conic = np.ascontiguousarray(grads[:, 0:2]), np.ascontiguousarray(grads[:, 2:5])
+    v_op, v_rgb = np.ascontiguousarray(grads[:, 5:6]), np.ascontiguousarray(grads[:, 6:9])
+    want = oracle.project_bwd(s, A["means_3d"], A["scales"], A["rotations"], S["conic"], S["cov3d"], radii, v_xy,
+                              v_conic)
+    want["v_shs"] = oracle.sh_bwd(s, num_bases, A["means_3d"], v_rgb)
+    want["v_colors"], want["v_opacity"] = v_rgb, v_op
+    want["v_means2d"] = np.concatenate([v_xy, np.zeros((n, 1), np.float32)], axis=1)
+    bounds = oracle.gradient_bounds(s, num_bases, A["means_3d"], A["scales"], A["rotations"], S["conic"], S["cov3d"],
+                                    radii, np.abs(grads[:, :9]), rel=1e-4, floor=0.0)
+    cam = st_.camera_from_scene(sc, DEV)
+    shapes = {"v_mean3d": (n, 3), "v_means2d": (n, 3), "v_shs": (n, num_bases, 3), "v_colors": (n, 3),
+              "v_opacity": (n, 1), "v_scale": (n, 3), "v_quat": (n, 4), "v_cov3d": (n, 6)}
+    order = ("v_mean3d", "v_means2d", "v_shs", "v_colors", "v_opacity", "v_scale", "v_quat", "v_cov3d")
+    poison = 12345.0
+    idle = np.ones(n, bool)
+    idle[rows] = False
+    idle[single] = False
+    for shift in (0, 1, 3):   # floats between a 16-byte boundary and the array's first element
+        bufs, outs, lead = {}, {}, {}
+        for key, shape in shapes.items():
+            count = int(np.prod(shape))
+            bufs[key] = torch.full((count + 16,), poison, dtype=torch.float32, device=DEV)
+            # (the kernel stores quaternion gradients as 16 bytes and covariance gradients as 8)
+            lead[key] = 4 + {"v_quat": 0, "v_cov3d": 2 if shift else 0}.get(key, shift)
+            outs[key] = bufs[key][lead[key]:lead[key] + count]
+        args = [dev(A["means_3d"]), dev(A["scales"]), dev(A["rotations"]), dev(pack_splats(S, radii, A["opacities"])),
+                None, dev(radii), dev(grads)]
+        st_.N.check(lib.dsx_gaussian_bwd(cam.ref, n, num_bases, *[st_._ptr(a) for a in args],
+                                         *[st_._ptr(outs[k]) for k in order], st_._stream()))
+        torch.cuda.synchronize()
+        for key, shape in shapes.items():
+            count = int(np.prod(shape))
+            whole = bufs[key].cpu().numpy()
+            assert (whole[:lead[key]] == poison).all() and (whole[lead[key] + count:] == poison).all(), key
+            got = outs[key].cpu().numpy().reshape(shape)
+            assert (got[idle] == 0).all(), key
+            if key in ("v_colors", "v_opacity", "v_means2d"):
+                np.testing.assert_array_equal(got, want[key])
+            else:
+                err = np.abs(got.astype(np.float64) - want[key])
+                assert (err <= bounds[key]).all(), "%s (shift %d): %.3e" % (key, shift, (err - bounds[key]).max())
+    # a NaN among the sums is a sum like any other: the row is worked on and the NaN comes through
+    if len(rows):
+        g2 = grads.copy()
+        g2[rows[0], 6] = np.nan
+        o = st_.gaussian_bwd(cam, num_bases, dev(A["means_3d"]), dev(A["scales"]), dev(A["rotations"]),
+                             dev(pack_splats(S, radii, A["opacities"])), None, dev(radii), dev(g2))
+        torch.cuda.synchronize()
+        assert torch.isnan(o["v_colors"][rows[0], 0]) and torch.isnan(o["v_shs"][rows[0], 0, 0])
