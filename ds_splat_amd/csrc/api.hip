@@ -158,6 +158,11 @@ extern "C" int dsx_set_list_bin(int tiles_per_side)
     return set_list_bin(tiles_per_side);
 }
 
+extern "C" size_t dsx_grads_bytes(int64_t n)
+{
+    return grads_bytes(n < 0 ? 0 : n);
+}
+
 extern "C" int64_t dsx_ranges_count(int32_t width, int32_t height)
 {
     return ranges_layout(list_grid(width < 0 ? 0 : width, height < 0 ? 0 : height)).count;
@@ -446,7 +451,8 @@ static int gaussian_bwd_checked(const dsx_camera* cam, int64_t n, int32_t num_ba
                                 const float* scales, const float* quats, const float* splats, const float* cov3d,
                                 const int32_t* radii, const float* grads, float* v_mean3d, float* v_means2d,
                                 float* v_shs, float* v_colors, float* v_opacity, float* v_scale, float* v_quat,
-                                float* v_cov3d, void* stream, bool conic_in_grads, bool outputs_cleared = false)
+                                float* v_cov3d, void* stream, bool conic_in_grads, bool outputs_cleared = false,
+                                bool with_marks = false)
 {
     if(int rc = check_camera(cam))
         return rc;
@@ -462,7 +468,7 @@ static int gaussian_bwd_checked(const dsx_camera* cam, int64_t n, int32_t num_ba
         return DSX_ERR_BAD_ARG; // without the stored covariance the kernel rebuilds it from scale and rotation
     return launch_gaussian_bwd(*cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
                                v_means2d, num_bases > 0 ? v_shs : nullptr, v_colors, v_opacity, v_scale, v_quat,
-                               v_cov3d, as_stream(stream), conic_in_grads, outputs_cleared);
+                               v_cov3d, as_stream(stream), conic_in_grads, outputs_cleared, with_marks);
 }
 
 extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
@@ -523,21 +529,15 @@ extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, c
         return rc;
     return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream), depth_flag,
                             partition_flag, n > 0 ? grads_to_prepare : nullptr, n,
-                            list_grid(cam->image_width, cam->image_height).shift ? ranges : nullptr);
+                            list_grid(cam->image_width, cam->image_height).shift ? ranges : nullptr, true);
 }
 
-// From this many Gaussians on, the backward clears its outputs on the helper stream beside the blend
-// kernel (below, one more launch in line costs less than the fork and join)
-constexpr int64_t kClearOutputsAsideFrom = 200000;
-
-// may_fork: the outputs' zeros may be written on the device's helper stream, beside the blend kernel
-// (two events are made and destroyed for that); otherwise they are written in line on the caller's stream
 static int backward_impl(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                          const float* scales, const float* quats, const float* splats, const float* cov3d,
                          const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
                          const float* final_T, const int32_t* final_idx, const float* v_image, float* grads,
                          int32_t grads_prepared, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
-                         float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, void* stream, bool may_fork)
+                         float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, void* stream)
 {
     if(int rc = check_camera(cam))
         return rc;
@@ -547,46 +547,19 @@ static int backward_impl(const dsx_camera* cam, int64_t n, int32_t num_bases, co
         return DSX_OK;
     if(!ranges || !final_T || !final_idx || !v_image || !grads || !splats)
         return DSX_ERR_BAD_ARG;
-    hipStream_t s = as_stream(stream);
     // The per-Gaussian kernel writes only the Gaussians that received a gradient term; everything
-    // else in its outputs is zero, written here: 260 bytes per Gaussian of plain stores that the
-    // blend kernel, which is bound by its arithmetic, has the memory system free for.
-    hipStream_t side = may_fork && n >= kClearOutputsAsideFrom ? helper_stream() : nullptr;
-    hipEvent_t fork = nullptr, join = nullptr;
-    if(side)
-    {
-        const bool ok = hipEventCreateWithFlags(&fork, hipEventDisableTiming) == hipSuccess &&
-                        hipEventCreateWithFlags(&join, hipEventDisableTiming) == hipSuccess &&
-                        hipEventRecord(fork, s) == hipSuccess && hipStreamWaitEvent(side, fork, 0) == hipSuccess;
-        if(!ok)
-        {
-            (void)hipGetLastError();
-            side = nullptr;
-        }
-    }
-    int rc = launch_zero_outputs(n, num_bases, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat,
-                                 v_cov3d, side ? side : s);
-    bool joined = true;
-    if(side)
-        joined = hipEventRecord(join, side) == hipSuccess;
-    if(!rc)
-        rc = launch_blend_bwd(*cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads, s,
-                              grads_prepared != 0,
-                              list_grid(cam->image_width, cam->image_height).shift ? ranges : nullptr);
-    // the caller's stream takes the helper's work back in, whatever happened in between
-    if(side && joined)
-        joined = hipStreamWaitEvent(s, join, 0) == hipSuccess;
-    if(fork)
-        (void)hipEventDestroy(fork);
-    if(join)
-        (void)hipEventDestroy(join);
+    // else in its outputs is zero: 260 bytes per Gaussian of plain stores, which the wavefronts of the
+    // blend kernel (bound by its arithmetic, the memory system idle) issue on their way out.
+    const ZeroJobs zeros = make_zero_jobs(n, num_bases, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale,
+                                          v_quat, v_cov3d);
+    int rc = launch_blend_bwd(*cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
+                              as_stream(stream), grads_prepared != 0,
+                              list_grid(cam->image_width, cam->image_height).shift ? ranges : nullptr, true, &zeros);
     if(rc)
         return rc;
-    if(!joined)
-        return DSX_ERR_RUNTIME;
     return gaussian_bwd_checked(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
                                 v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, stream,
-                                grads_prepared != 0, true);
+                                grads_prepared != 0, true, true);
 }
 
 extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
@@ -598,7 +571,7 @@ extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases,
 {
     return backward_impl(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, ranges, sorted_ids, final_T,
                          final_idx, v_image, grads, grads_prepared, v_mean3d, v_means2d, v_shs, v_colors, v_opacity,
-                         v_scale, v_quat, v_cov3d, stream, true);
+                         v_scale, v_quat, v_cov3d, stream);
 }
 
 extern "C" int dsx_forward_core(const float* means3d, const float* shs, const float* opacities, const float* scales,
@@ -625,7 +598,6 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     if(n < 0 || !image)
         return DSX_ERR_BAD_ARG;
     const int64_t P = (int64_t)image_width * image_height;
-    const int num_tiles = dsx_num_tiles(image_width, image_height);
     const int64_t nb = dsx_num_blocks(n);
 
     auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
@@ -674,7 +646,9 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
 namespace
 {
 constexpr int64_t kStaticMaxGaussians = DSX_STATIC_MAX_GAUSSIANS;
-static __device__ __align__(256) float scratch[kStaticMaxGaussians * DSX_GRAD_FLOATS];
+// (the accumulator records and, behind them, the byte per Gaussian: grads_bytes(kStaticMaxGaussians))
+static __device__ __align__(256) float scratch[kStaticMaxGaussians * DSX_GRAD_FLOATS + kStaticMaxGaussians / 4];
+static_assert(sizeof(scratch) >= grads_bytes(kStaticMaxGaussians), "records and marks of the largest call");
 
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
@@ -714,10 +688,9 @@ extern "C" int dsx_backward_static(const dsx_camera* cam, int64_t n, int32_t num
         return DSX_ERR_RUNTIME;
     // grads_prepared = 0: the array keeps the last call's sums, so this call clears its n records
     // itself (a fill kernel with plain stores, which a caller may capture in a graph)
-    // (and writes the outputs' zeros in line: no second stream, no events made)
     return backward_impl(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, ranges, sorted_ids, final_T,
                          final_idx, v_image, grads, 0, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat,
-                         v_cov3d, stream, false);
+                         v_cov3d, stream);
 }
 
 extern "C" int dsx_set_blend_pixels_per_lane(int pixels)

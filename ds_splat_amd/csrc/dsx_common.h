@@ -288,28 +288,72 @@ int launch_sort_pairs(int64_t k, int num_tiles, int64_t* keys_a, int32_t* values
 int launch_tile_ranges(int64_t k, const int64_t* sorted_keys, int num_tiles, int32_t* ranges,
                        hipStream_t stream);
 // sort_flag_*: error words of the sorts that built the lists (null: none); the image becomes NaN if one is set
+// The accumulator of the whole backward (dsx_backward and what prepares it): n records of
+// DSX_GRAD_FLOATS floats, then one byte per Gaussian that the blend backward sets when it adds a
+// term to the record (the per-Gaussian kernel then reads 1 byte instead of 48 to learn that a
+// Gaussian has nothing to propagate), padded to 16 bytes.
+constexpr size_t grads_bytes(int64_t n)
+{
+    return (size_t)n * DSX_GRAD_FLOATS * 4 + (((size_t)n + 15) & ~(size_t)15);
+}
+inline uint8_t* grad_marks(float* grads, int64_t n)
+{
+    return reinterpret_cast<uint8_t*>(grads + n * DSX_GRAD_FLOATS);
+}
+// The zeros of the per-Gaussian backward's outputs: up to eight arrays.  Their 16-byte-aligned middles
+// form one range of 16-byte stores that the parts of a launch share evenly (v_shs alone is three
+// quarters of it); the few floats in front of and behind a middle are stored one by one.
+struct ZeroJobs
+{
+    float* ptr[8];     // null: not wanted
+    int64_t floats[8]; // length of the array
+    int64_t end[8];    // 16-byte stores of this and all earlier arrays
+    int any;           // is there anything to store?
+};
+inline ZeroJobs make_zero_jobs(int64_t n, int num_bases, float* v_mean3d, float* v_means2d, float* v_shs,
+                               float* v_colors, float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d)
+{
+    ZeroJobs jobs;
+    float* ptrs[8] = {v_mean3d, v_means2d, num_bases > 0 ? v_shs : nullptr, v_colors, v_opacity, v_scale, v_quat, v_cov3d};
+    const int64_t per[8] = {3, 3, 3 * (int64_t)num_bases, 3, 1, 3, 4, 6};
+    int64_t stores = 0;
+    jobs.any = 0;
+    for(int j = 0; j < 8; ++j)
+    {
+        jobs.ptr[j] = n > 0 ? ptrs[j] : nullptr;
+        jobs.floats[j] = jobs.ptr[j] ? n * per[j] : 0;
+        if(jobs.ptr[j])
+        {
+            jobs.any = 1;
+            const int64_t head = (int64_t)(((16 - ((uintptr_t)ptrs[j] & 15)) & 15) / 4);
+            stores += jobs.floats[j] > head ? (jobs.floats[j] - head) / 4 : 0;
+        }
+        jobs.end[j] = stores;
+    }
+    return jobs;
+}
+
 int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids,
                      const float* splats, float* image, float* final_T, int32_t* final_idx,
                      hipStream_t stream,
                      const uint32_t* sort_flag_a = nullptr, const uint32_t* sort_flag_b = nullptr,
-                     float* prepare_grads = nullptr, int64_t num_gaussians = 0, int32_t* lists = nullptr);
+                     float* prepare_grads = nullptr, int64_t num_gaussians = 0, int32_t* lists = nullptr,
+                     bool prepare_marks = false);
 int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges,
                      const int32_t* sorted_ids, const float* splats, const float* final_T,
                      const int32_t* final_idx, const float* v_image, float* grads,
-                     hipStream_t stream, bool grads_prepared = false, const int32_t* lists = nullptr);
+                     hipStream_t stream, bool grads_prepared = false, const int32_t* lists = nullptr,
+                     bool with_marks = false, const ZeroJobs* zeros = nullptr);
 int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d,
                         const float* scales, const float* quats, const float* splats,
                         const float* cov3d, const int32_t* radii, const float* grads,
                         float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
                         float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d,
-                        hipStream_t stream, bool conic_in_grads = false, bool outputs_cleared = false);
+                        hipStream_t stream, bool conic_in_grads = false, bool outputs_cleared = false,
+                        bool with_marks = false);
 // zeros in every output of launch_gaussian_bwd that is not null (it writes only the Gaussians that
 // have something to propagate; outputs_cleared tells it that this has been done)
-int launch_zero_outputs(int64_t n, int num_bases, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
-                        float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, hipStream_t stream);
-// the device's helper stream (default priority, made on first use, kept until the process ends;
-// shared by every caller thread), or nullptr when none can be made
-hipStream_t helper_stream();
+int launch_zero_outputs(const ZeroJobs& jobs, hipStream_t stream);
 int launch_fill_u32(uint32_t* p, int64_t count, uint32_t value, hipStream_t stream);
 // 1 or 4: force that form of both blend kernels for the whole process; 0: choose by image size
 int set_blend_pixels_per_lane(int pixels);
@@ -438,6 +482,54 @@ __device__ __forceinline__ void nt_store_f4(float4* p, float4 v)
     t.z = v.z;
     t.w = v.w;
     __builtin_nontemporal_store(t, reinterpret_cast<dsx_v4f*>(p));
+}
+
+// the 16-byte stores [lo, hi) of the arrays' middles, by `threads` threads (this one: tid)
+__device__ __forceinline__ void zero_range(const ZeroJobs& jobs, int64_t lo, int64_t hi, int tid, int threads)
+{
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for(int j = 0; j < 8; ++j)
+    {
+        float* ptr = jobs.ptr[j];
+        if(ptr == nullptr)
+            continue;
+        const int64_t start = j ? jobs.end[j - 1] : 0;
+        const int head = (int)(((16 - ((uintptr_t)ptr & 15)) & 15) / 4);
+        float4* q = reinterpret_cast<float4*>(ptr + head) - start;
+        for(int64_t i = max(lo, start) + tid; i < min(hi, jobs.end[j]); i += threads)
+            nt_store_f4(q + i, zero);
+    }
+}
+// the floats in front of and behind the middles (threads 0..3 of one part of the launch)
+__device__ __forceinline__ void zero_edges(const ZeroJobs& jobs, int tid)
+{
+    if(tid >= 4)
+        return;
+#pragma unroll
+    for(int j = 0; j < 8; ++j)
+    {
+        float* ptr = jobs.ptr[j];
+        if(ptr == nullptr)
+            continue;
+        const int64_t start = j ? jobs.end[j - 1] : 0;
+        const int head = (int)(((16 - ((uintptr_t)ptr & 15)) & 15) / 4);
+        const int64_t n = jobs.floats[j];
+        if(tid < head && (int64_t)tid < n)
+            ptr[tid] = 0.f;
+        const int64_t t = head + (jobs.end[j] - start) * 4 + tid;
+        if(t < n)
+            ptr[t] = 0.f;
+    }
+}
+// part `part` of `parts` stores its share of the zeros
+__device__ __forceinline__ void zero_share(const ZeroJobs& jobs, int64_t part, int64_t parts, int tid, int threads)
+{
+    const int64_t total = jobs.end[7];
+    const int64_t share = (total + parts - 1) / parts;
+    zero_range(jobs, part * share, min((part + 1) * share, total), tid, threads);
+    if(part == 0)
+        zero_edges(jobs, tid);
 }
 
 struct TileRect

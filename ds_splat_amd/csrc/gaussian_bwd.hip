@@ -3,14 +3,17 @@
 // blend backward.  Every output is linear in a Gaussian's nine accumulated sums, so a Gaussian
 // whose sums are all zero (culled, hidden behind others, or outside every tile that still had
 // light to give: the large majority of a dense scene) has all-zero gradients.  The outputs are
-// therefore cleared by a plain fill (zero_outputs_kernel, which the whole backward runs on a
-// second stream beside the blend kernel, whose work leaves the memory system idle), and this
-// kernel reads the 48-byte accumulator rows of a chunk of Gaussians, packs the ones with a
+// therefore cleared by plain stores (in the whole backward by the blend kernel's wavefronts, each a
+// share at its end: that kernel's arithmetic leaves the memory system idle), and this
+// kernel reads the 48-byte accumulator rows of a run of Gaussians (or, in the whole backward, the
+// byte per Gaussian that the blend backward set when it added a term), packs the ones with a
 // non-zero sum in LDS, and works on those only: one thread per such Gaussian, the 192-byte
 // v_shs rows assembled in LDS per wavefront and written with 16-byte stores.
 // Math follows cpp/gsplat/backward.cu:216-393, cpp/gsplat/helpers.cuh:68-220 and
 // cpp/gsplat/sh.cuh:95-186 of the reference; matrices below are indexed [row][col].
 #include "dsx_common.h"
+
+#include <atomic>
 
 namespace dsx
 {
@@ -27,6 +30,7 @@ struct GaussianBwdParams
     const float* cov3d;
     const int32_t* radii;
     const float4* grads;
+    const uint8_t* marks; // per Gaussian: did the blend backward add a term? (null: look at the sums)
     const float* view;
     const float* campos;
     float* v_mean3d;
@@ -40,6 +44,7 @@ struct GaussianBwdParams
     float fx, fy, glob;
     int sh_degree, num_bases;
     int conic_in_grads; // the accumulator's places 9..11 hold the conic (the forward put it there)
+    int run;            // Gaussians per workgroup: a multiple of the wavefront, at most kBwdListMax
 };
 
 __device__ __forceinline__ void mat3_mul(const float (&A)[3][3], const float (&B)[3][3], float (&C)[3][3])
@@ -83,8 +88,14 @@ __device__ __forceinline__ int sh_basis(int deg, float3 d, float* Y)
     return 16;
 }
 
-constexpr int kBwdChunk = 1024;                       // Gaussians per workgroup
-constexpr int kBwdPerThread = kBwdChunk / kProjBlock; // accumulator rows a thread tests
+// One wavefront per workgroup, each with its own run of Gaussians.  The runs are sized so that all
+// workgroups are resident at once whenever the list below can hold a run (12 per CU: 164 VGPRs,
+// 10 KB of LDS): a scene where few Gaussians have work then costs one pass of latency (find the
+// few, do them) instead of one per wave of workgroups, and a scene where all have work gives every
+// wavefront the same share.
+constexpr int kBwdListMax = 2048;  // longest run (its list of Gaussians with work sits in LDS)
+constexpr int kBwdRunMin = 256;
+constexpr int kBwdResidentPerCu = 12;
 
 // does any of the nine sums of an accumulator row differ from zero? (a NaN does)
 __device__ __forceinline__ bool any_sum(const float4& g0, const float4& g1, const float4& g2)
@@ -93,68 +104,110 @@ __device__ __forceinline__ bool any_sum(const float4& g0, const float4& g1, cons
            g1.w != 0.f || g2.x != 0.f;
 }
 
-__global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const GaussianBwdParams p)
+// what the kernel reads of one Gaussian
+struct GaussianBwdInputs
 {
-    __shared__ float sh_lds[4][64 * kShPitchB];
-    __shared__ uint16_t s_list[kBwdChunk];                 // the chunk's Gaussians with work, in index order
-    __shared__ int s_count[kBwdPerThread * 4 + 1];         // per (row of the test, wavefront): how many
+    int64_t i; // which Gaussian
+    bool live; // (false: this lane has none in this round)
+    float4 g0, g1, g2;
+    float3 mean;
+    int radius;
+    float sc[3];
+    float4 quat;
+    float c3[6];
+    float4 conic;
+};
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int64_t chunk0 = (int64_t)blockIdx.x * kBwdChunk;
-
-    // ---- which Gaussians of the chunk have anything to propagate ------------------------------
-    uint64_t mask[kBwdPerThread];
-#pragma unroll
-    for(int j = 0; j < kBwdPerThread; ++j)
+// the inputs of entry `at + lane` of the run's list
+__device__ __forceinline__ GaussianBwdInputs load_inputs(const GaussianBwdParams& p, int64_t run0,
+                                                         const uint16_t* list, int at, int total, int lane)
+{
+    GaussianBwdInputs in = {};
+    in.live = at + lane < total;
+    if(!in.live)
+        return in;
+    const int64_t i = run0 + list[at + lane];
+    in.i = i;
+    in.g0 = p.grads[3 * i];
+    in.g1 = p.grads[3 * i + 1];
+    in.g2 = p.grads[3 * i + 2];
+    in.mean = make_float3(p.means3d[3 * i], p.means3d[3 * i + 1], p.means3d[3 * i + 2]);
+    in.radius = p.radii[i];
+    if(p.scales)
     {
-        const int64_t i = chunk0 + j * kProjBlock + tid;
-        bool work = false;
-        if(i < p.n)
-            work = any_sum(p.grads[3 * i], p.grads[3 * i + 1], p.grads[3 * i + 2]);
-        mask[j] = __ballot(work);
-        if(lane == 0)
-            s_count[j * 4 + wave] = __popcll(mask[j]);
+        in.sc[0] = p.scales[3 * i];
+        in.sc[1] = p.scales[3 * i + 1];
+        in.sc[2] = p.scales[3 * i + 2];
+        in.quat = reinterpret_cast<const float4*>(p.quats)[i];
     }
-    __syncthreads();
-    int total = 0; // Gaussians with work in the rows before row j, then in the whole chunk
-#pragma unroll
-    for(int j = 0; j < kBwdPerThread; ++j)
+    if(p.cov3d)
     {
-        int before = 0, row_total = 0; // ... in front of this wavefront's 64 of row j, and in row j
+        const float2* cs = reinterpret_cast<const float2*>(p.cov3d + 6 * i);
+        const float2 c01 = cs[0], c23 = cs[1], c45 = cs[2];
+        in.c3[0] = c01.x, in.c3[1] = c01.y, in.c3[2] = c23.x, in.c3[3] = c23.y, in.c3[4] = c45.x, in.c3[5] = c45.y;
+    }
+    // the conic: behind the sums when the forward prepared the accumulator, else from the splat record
+    in.conic = p.conic_in_grads ? make_float4(in.g2.y, in.g2.z, in.g2.w, 0.f) : p.splats[3 * i + 1];
+    return in;
+}
+
+__global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(3, 3))) void gaussian_bwd_kernel(const GaussianBwdParams p)
+{
+    __shared__ float rows[32 * kShPitchB];
+    __shared__ uint16_t s_list[kBwdListMax]; // the run's Gaussians with work, in index order
+
+    const int lane = threadIdx.x;
+    const int64_t run0 = (int64_t)blockIdx.x * p.run;
+    const int run = (int)min((int64_t)p.run, p.n - run0);
+
+    // ---- which Gaussians of the run have anything to propagate --------------------------------
+    int total = 0;
+    for(int first = 0; first < run; first += 4 * DSX_WAVE)
+    {
+        bool work[4];
 #pragma unroll
-        for(int w = 0; w < 4; ++w)
+        for(int j = 0; j < 4; ++j)
         {
-            const int c = s_count[j * 4 + w];
-            before += w < wave ? c : 0;
-            row_total += c;
+            const int local = first + j * DSX_WAVE + lane;
+            const int64_t i = run0 + local;
+            work[j] = false;
+            if(local < run)
+                work[j] = p.marks ? p.marks[i] != 0 : any_sum(p.grads[3 * i], p.grads[3 * i + 1], p.grads[3 * i + 2]);
         }
-        if((mask[j] >> lane) & 1)
-            s_list[total + before + __popcll(mask[j] & ((1ull << lane) - 1ull))] = (uint16_t)(j * kProjBlock + tid);
-        total += row_total;
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+        {
+            const uint64_t mask = __ballot(work[j]);
+            if(work[j])
+                s_list[total + __popcll(mask & ((1ull << lane) - 1ull))] = (uint16_t)(first + j * DSX_WAVE + lane);
+            total += __popcll(mask);
+        }
     }
-    __syncthreads();
+    __syncthreads(); // (one wavefront: orders the LDS writes before the reads)
 
+    // The inputs of a round are fetched while the round before is being computed: the wavefronts of
+    // a launch start together and stay in step, so without this the memory system would idle while all
+    // of them compute and the arithmetic units while all of them wait.
     const int row_floats = p.num_bases * 3;
-    float* rows = sh_lds[wave];
-    for(int first = 0; first < total; first += kProjBlock)
+    GaussianBwdInputs ahead = load_inputs(p, run0, s_list, 0, total, lane);
+    for(int first = 0; first < total; first += DSX_WAVE)
     {
-        const bool live = first + tid < total;
-        const int64_t i = live ? chunk0 + s_list[first + tid] : 0;
+        const GaussianBwdInputs in = ahead;
+        ahead = load_inputs(p, run0, s_list, first + DSX_WAVE, total, lane);
+        const bool live = in.live;
+        const int64_t i = in.i;
 
         float v_rgb[3] = {0.f, 0.f, 0.f};
-        float3 mean = make_float3(0.f, 0.f, 0.f);
+        const float3 mean = in.mean;
         if(live)
         {
-            const float4 g0 = p.grads[3 * i], g1 = p.grads[3 * i + 1], g2 = p.grads[3 * i + 2];
+            const float4 g0 = in.g0, g1 = in.g1;
             const float v_x = g0.x, v_y = g0.y;
             const float vc[3] = {g0.z, g0.w, g1.x};
             const float v_o = g1.y;
             v_rgb[0] = g1.z;
             v_rgb[1] = g1.w;
-            v_rgb[2] = g2.x;
-            mean = make_float3(p.means3d[3 * i], p.means3d[3 * i + 1], p.means3d[3 * i + 2]);
+            v_rgb[2] = in.g2.x;
 
             // straight copies: screen-space mean gradient (z column zero), colour and opacity
             // (every output is optional: a null pointer means that the caller has no use for it)
@@ -175,7 +228,7 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
 
             float vm[3] = {0.f, 0.f, 0.f}, vs[3] = {0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f};
             float vc3[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            if(p.radii[i] > 0)
+            if(in.radius > 0)
             {
                 const float* V = p.view;
                 const float R[3][3] = {{V[0], V[1], V[2]}, {V[4], V[5], V[6]}, {V[8], V[9], V[10]}};
@@ -194,12 +247,7 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
                 // conic -> cov2d:  v_Sigma = -X G X, X = conic, G = symmetrised v_conic
                 float v_cov2d[3];
                 {
-                    // the conic: behind the sums when the forward prepared the accumulator, else from the splat record
-                    float4 q1;
-                    if(p.conic_in_grads)
-                        q1 = make_float4(g2.y, g2.z, g2.w, 0.f);
-                    else
-                        q1 = p.splats[3 * i + 1];
+                    const float4 q1 = in.conic;
                     const float X[2][2] = {{q1.x, q1.y}, {q1.y, q1.z}};
                     const float G[2][2] = {{vc[0], 0.5f * vc[1]}, {0.5f * vc[1], vc[2]}};
                     float M[2][2], N[2][2];
@@ -234,15 +282,12 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
                     float c3[6];
                     if(p.cov3d)
                     {
-                        const float2* cs = reinterpret_cast<const float2*>(p.cov3d + 6 * i);
-                        const float2 c01 = cs[0], c23 = cs[1], c45 = cs[2];
-                        c3[0] = c01.x, c3[1] = c01.y, c3[2] = c23.x, c3[3] = c23.y, c3[4] = c45.x, c3[5] = c45.y;
+#pragma unroll
+                        for(int c = 0; c < 6; ++c)
+                            c3[c] = in.c3[c];
                     }
                     else
-                    {
-                        const float sc[3] = {p.scales[3 * i], p.scales[3 * i + 1], p.scales[3 * i + 2]};
-                        cov3d_from_scale_rot(sc, reinterpret_cast<const float4*>(p.quats)[i], p.glob, c3);
-                    }
+                        cov3d_from_scale_rot(in.sc, in.quat, p.glob, c3);
                     const float S[3][3] = {{c3[0], c3[1], c3[2]}, {c3[1], c3[3], c3[4]}, {c3[2], c3[4], c3[5]}};
                     const float Gc[2][2] = {{v_cov2d[0], 0.5f * v_cov2d[1]}, {0.5f * v_cov2d[1], v_cov2d[2]}};
                     // GT = Gc T (2x3)
@@ -296,14 +341,13 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
                     const float vV[3][3] = {{vc3[0], 0.5f * vc3[1], 0.5f * vc3[2]},
                                             {0.5f * vc3[1], vc3[3], 0.5f * vc3[4]},
                                             {0.5f * vc3[2], 0.5f * vc3[4], vc3[5]}};
-                    const float4 q = reinterpret_cast<const float4*>(p.quats)[i];
+                    const float4 q = in.quat;
                     const float w = q.x, x = q.y, y = q.z, z = q.w;
                     const float Rq[3][3] = {
                         {1.f - 2.f * (y * y + z * z), 2.f * (x * y - w * z), 2.f * (x * z + w * y)},
                         {2.f * (x * y + w * z), 1.f - 2.f * (x * x + z * z), 2.f * (y * z - w * x)},
                         {2.f * (x * z - w * y), 2.f * (y * z + w * x), 1.f - 2.f * (x * x + y * y)}};
-                    const float s[3] = {p.glob * p.scales[3 * i], p.glob * p.scales[3 * i + 1],
-                                        p.glob * p.scales[3 * i + 2]};
+                    const float s[3] = {p.glob * in.sc[0], p.glob * in.sc[1], p.glob * in.sc[2]};
                     float M[3][3], vM[3][3], vR[3][3];
 #pragma unroll
                     for(int r = 0; r < 3; ++r)
@@ -355,132 +399,83 @@ __global__ __launch_bounds__(kProjBlock) void gaussian_bwd_kernel(const Gaussian
         // ---- v_shs[b][c] = Y_b(dir) * v_rgb[c], zero above the active degree -------------------
         if(p.v_shs == nullptr)
             continue;
-        if(first > 0)
-            __syncthreads(); // the rows of the last round have been read
+        float Y[16];
+        int nb = 0;
         if(live)
         {
-            float Y[16];
             const float3 d = make_float3(mean.x - p.campos[0], mean.y - p.campos[1], mean.z - p.campos[2]);
-            const int nb = min(sh_basis(p.sh_degree, d, Y), p.num_bases);
-            float* r = rows + lane * kShPitchB;
+            nb = min(sh_basis(p.sh_degree, d, Y), p.num_bases);
+        }
+        // the rows pass through LDS half a wavefront at a time (32 rows: 6 KB, so that twelve
+        // workgroups fit a CU) and go out 16 bytes per lane: twelve lanes per row of 48 floats
+        const int nrows = min(DSX_WAVE, total - first);
 #pragma unroll
-            for(int b = 0; b < 16; ++b)
+        for(int half = 0; half < 2; ++half)
+        {
+            __syncthreads(); // the rows of the last half have been read
+            if(live && (lane >> 5) == half)
             {
-                if(b < p.num_bases)
+                float* r = rows + (lane & 31) * kShPitchB;
+#pragma unroll
+                for(int b = 0; b < 16; ++b)
                 {
-                    const float yb = b < nb ? Y[b] : 0.f;
-                    r[3 * b] = b < nb ? yb * v_rgb[0] : 0.f;
-                    r[3 * b + 1] = b < nb ? yb * v_rgb[1] : 0.f;
-                    r[3 * b + 2] = b < nb ? yb * v_rgb[2] : 0.f;
+                    if(b < p.num_bases)
+                    {
+                        const float yb = b < nb ? Y[b] : 0.f;
+                        r[3 * b] = b < nb ? yb * v_rgb[0] : 0.f;
+                        r[3 * b + 1] = b < nb ? yb * v_rgb[1] : 0.f;
+                        r[3 * b + 2] = b < nb ? yb * v_rgb[2] : 0.f;
+                    }
                 }
             }
-        }
-        __syncthreads();
-        // the wavefront's rows go out 16 bytes per lane: twelve lanes per row when a row is 48 floats
-        const int wave_first = first + wave * 64;
-        const int nrows = max(0, min(64, total - wave_first));
-        if(row_floats == 48 && ((uintptr_t)p.v_shs & 15) == 0)
-        {
-            const int chunks = nrows * 12;
-#pragma unroll
-            for(int j = 0; j < 12; ++j)
+            __syncthreads();
+            const int half_rows = max(0, min(32, nrows - 32 * half));
+            const uint16_t* ids = s_list + first + 32 * half;
+            if(row_floats == 48 && ((uintptr_t)p.v_shs & 15) == 0)
             {
-                const int e = j * 64 + lane;
-                if(e < chunks)
+                const int chunks = half_rows * 12;
+#pragma unroll
+                for(int j = 0; j < 6; ++j)
                 {
-                    const int row = e / 12;
-                    const int c4 = e - row * 12;
-                    const float* s = rows + row * kShPitchB + c4 * 4;
-                    float4* dst = reinterpret_cast<float4*>(p.v_shs + (chunk0 + s_list[wave_first + row]) * 48);
-                    nt_store_f4(dst + c4, make_float4(s[0], s[1], s[2], s[3]));
+                    const int e = j * 64 + lane;
+                    if(e < chunks)
+                    {
+                        const int row = e / 12;
+                        const int c4 = e - row * 12;
+                        const float* s = rows + row * kShPitchB + c4 * 4;
+                        float4* dst = reinterpret_cast<float4*>(p.v_shs + (run0 + ids[row]) * 48);
+                        nt_store_f4(dst + c4, make_float4(s[0], s[1], s[2], s[3]));
+                    }
                 }
             }
-        }
-        else
-        {
-            const int count = nrows * row_floats;
-            for(int e = lane; e < count; e += 64)
+            else
             {
-                const int row = e / row_floats;
-                const int c = e - row * row_floats;
-                p.v_shs[(chunk0 + s_list[wave_first + row]) * row_floats + c] = rows[row * kShPitchB + c];
+                const int count = half_rows * row_floats;
+                for(int e = lane; e < count; e += 64)
+                {
+                    const int row = e / row_floats;
+                    const int c = e - row * row_floats;
+                    p.v_shs[(run0 + ids[row]) * row_floats + c] = rows[row * kShPitchB + c];
+                }
             }
         }
     }
 }
 
-// ---- the outputs' zeros: up to eight arrays in one launch --------------------------------------
-// The arrays' 16-byte-aligned middles form one range of 16-byte stores that the workgroups share
-// evenly (v_shs alone is three quarters of it); the few floats in front of and behind a middle are
-// stored one by one.  Few workgroups, one per two CUs: the kernel runs beside the blend backward, which
-// wants every wavefront slot, and 512 wavefronts still store 780 MB well within that kernel's time
-// (3 M Gaussians at 1920x1080, whole step: 0.854 ms with 96 or 128 workgroups, 0.862 with 192,
-// 0.896 with 256, 0.872 with 4096).
-constexpr int kZeroWorkgroups = 128;
-
-struct ZeroJobs
-{
-    float* ptr[8];     // null: not wanted
-    int64_t floats[8]; // length of the array
-    int64_t end[8];    // 16-byte stores of this and all earlier arrays
-};
-
+// ---- the outputs' zeros as a launch of their own (the stage entry point; the whole backward has
+// them written by the blend kernel's wavefronts instead, see zero_share) ---------------------------
 __global__ __launch_bounds__(kProjBlock) void zero_outputs_kernel(const ZeroJobs jobs)
 {
-    const int64_t total = jobs.end[7];
-    const int64_t share = (total + gridDim.x - 1) / gridDim.x;
-    const int64_t lo = (int64_t)blockIdx.x * share, hi = min(lo + share, total);
-    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-    for(int j = 0; j < 8; ++j)
-    {
-        float* ptr = jobs.ptr[j];
-        if(ptr == nullptr)
-            continue;
-        const int64_t start = j ? jobs.end[j - 1] : 0;
-        const int head = (int)(((16 - ((uintptr_t)ptr & 15)) & 15) / 4);
-        float4* q = reinterpret_cast<float4*>(ptr + head) - start;
-        for(int64_t i = max(lo, start) + threadIdx.x; i < min(hi, jobs.end[j]); i += kProjBlock)
-            nt_store_f4(q + i, zero);
-        if(blockIdx.x == 0 && threadIdx.x < 4)
-        {
-            const int64_t n = jobs.floats[j];
-            if((int)threadIdx.x < head && (int64_t)threadIdx.x < n)
-                ptr[threadIdx.x] = 0.f;
-            const int64_t t = head + (jobs.end[j] - start) * 4 + threadIdx.x;
-            if(t < n)
-                ptr[t] = 0.f;
-        }
-    }
+    zero_share(jobs, blockIdx.x, gridDim.x, threadIdx.x, kProjBlock);
 }
 
-int launch_zero_outputs(int64_t n, int num_bases, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
-                        float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, hipStream_t stream)
+int launch_zero_outputs(const ZeroJobs& jobs, hipStream_t stream)
 {
-    if(n <= 0)
+    if(!jobs.any)
         return DSX_OK;
-    ZeroJobs jobs;
-    float* ptrs[8] = {v_mean3d, v_means2d, num_bases > 0 ? v_shs : nullptr, v_colors, v_opacity, v_scale, v_quat, v_cov3d};
-    const int64_t per[8] = {3, 3, 3 * (int64_t)num_bases, 3, 1, 3, 4, 6};
-    int64_t stores = 0;
-    bool any = false;
-    for(int j = 0; j < 8; ++j)
-    {
-        jobs.ptr[j] = ptrs[j];
-        jobs.floats[j] = ptrs[j] ? n * per[j] : 0;
-        if(ptrs[j])
-        {
-            any = true;
-            const int64_t head = (int64_t)(((16 - ((uintptr_t)ptrs[j] & 15)) & 15) / 4);
-            stores += jobs.floats[j] > head ? (jobs.floats[j] - head) / 4 : 0;
-        }
-        jobs.end[j] = stores;
-    }
-    if(!any)
-        return DSX_OK;
-    // at least 16 stores per thread, at most kZeroWorkgroups workgroups
-    const int64_t want = (stores + (int64_t)kProjBlock * 16 - 1) / ((int64_t)kProjBlock * 16);
-    const unsigned blocks = (unsigned)max((int64_t)1, min(want, (int64_t)kZeroWorkgroups));
+    // at least 16 stores per thread, at most eight workgroups per CU
+    const int64_t want = (jobs.end[7] + (int64_t)kProjBlock * 16 - 1) / ((int64_t)kProjBlock * 16);
+    const unsigned blocks = (unsigned)max((int64_t)1, min(want, (int64_t)2048));
     {
         DSX_TIMED("zero_outputs_kernel", stream);
         hipLaunchKernelGGL(zero_outputs_kernel, dim3(blocks), dim3(kProjBlock), 0, stream, jobs);
@@ -489,17 +484,39 @@ int launch_zero_outputs(int64_t n, int num_bases, float* v_mean3d, float* v_mean
     return DSX_OK;
 }
 
+// CUs of the current device (asked once per device; 256 if the question fails)
+static int compute_units()
+{
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> known[kMaxDevices] = {};
+    int device = 0;
+    if(hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+        return 256;
+    int cus = known[device].load(std::memory_order_relaxed);
+    if(cus == 0)
+    {
+        if(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
+        {
+            (void)hipGetLastError();
+            cus = 256;
+        }
+        known[device].store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+
 int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d, const float* scales,
                         const float* quats, const float* splats, const float* cov3d, const int32_t* radii,
                         const float* grads, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
                         float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, hipStream_t stream,
-                        bool conic_in_grads, bool outputs_cleared)
+                        bool conic_in_grads, bool outputs_cleared, bool with_marks)
 {
     if(n == 0)
         return DSX_OK;
     if(!outputs_cleared)
-        if(int rc = launch_zero_outputs(n, num_bases, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat,
-                                        v_cov3d, stream))
+        if(int rc = launch_zero_outputs(make_zero_jobs(n, num_bases, v_mean3d, v_means2d, v_shs, v_colors, v_opacity,
+                                                       v_scale, v_quat, v_cov3d),
+                                        stream))
             return rc;
     GaussianBwdParams p;
     p.n = n;
@@ -510,6 +527,7 @@ int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const f
     p.cov3d = cov3d;
     p.radii = radii;
     p.grads = reinterpret_cast<const float4*>(grads);
+    p.marks = with_marks ? grad_marks(const_cast<float*>(grads), n) : nullptr;
     p.view = cam.view;
     p.campos = cam.campos;
     p.v_mean3d = v_mean3d;
@@ -530,10 +548,14 @@ int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const f
     p.sh_degree = cam.sh_degree;
     p.num_bases = num_bases;
     p.conic_in_grads = conic_in_grads ? 1 : 0;
-    const int64_t blocks = (n + kBwdChunk - 1) / kBwdChunk;
+    // runs that make all workgroups resident at once, if the list can hold such a run
+    const int64_t resident = (int64_t)compute_units() * kBwdResidentPerCu;
+    const int64_t even = ((n + resident - 1) / resident + DSX_WAVE - 1) / DSX_WAVE * DSX_WAVE;
+    p.run = (int)max((int64_t)kBwdRunMin, min(even, (int64_t)kBwdListMax));
+    const int64_t blocks = (n + p.run - 1) / p.run;
     {
         DSX_TIMED("gaussian_bwd_kernel", stream);
-        hipLaunchKernelGGL(gaussian_bwd_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream, p);
+        hipLaunchKernelGGL(gaussian_bwd_kernel, dim3((unsigned)blocks), dim3(DSX_WAVE), 0, stream, p);
     }
     DSX_LAUNCH_CHECK();
     return DSX_OK;

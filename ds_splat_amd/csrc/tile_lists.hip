@@ -22,7 +22,7 @@ namespace dsx
 // ends): work that does not depend on the depth sort runs there, beside the sort's
 // latency-bound passes.  Returns nullptr when no stream can be made (the caller then stays on
 // its own stream).
-hipStream_t helper_stream()
+static hipStream_t helper_stream()
 {
     constexpr int kMaxDevices = 64;
     static std::mutex mutex;

@@ -72,8 +72,8 @@ at::Tensor& pinned_key_count()
 // image[H,W,3], radii[N], splats[N,12], sorted_ids[K], ranges[dsx_ranges_count], final_T[H,W], final_idx[H,W]
 // (the 3-D covariances are not kept: the backward rebuilds them from scales and rotations, or
 // reads cov3d_precomp) and, when prepare_backward is set, the backward's gradient accumulator
-// [N,12], which the blend kernel prepares on the side: sums zeroed, conics in the spare places
-// (undefined otherwise)
+// (dsx_grads_bytes(N) bytes as float32), which the blend kernel prepares on the side: sums zeroed,
+// conics in the spare places, the byte per Gaussian behind the records cleared (undefined otherwise)
 std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
                                 int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view,
                                 const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
@@ -112,7 +112,7 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
     at::Tensor final_idx = at::empty({height, width}, i32);
     const size_t ws_bytes = dsx_workspace_bytes(n, k, (int32_t)width, (int32_t)height);
     at::Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 1)}, u8);
-    at::Tensor grads = prepare_backward && n > 0 ? at::empty({n, DSX_GRAD_FLOATS}, f32) : at::Tensor();
+    at::Tensor grads = prepare_backward && n > 0 ? at::empty({(int64_t)(dsx_grads_bytes(n) / 4)}, f32) : at::Tensor();
     check(dsx_forward_finish(&cam.c, n, k, splats.data_ptr<float>(), order.data_ptr(), sorted_ids.data_ptr<int32_t>(),
                              ranges.data_ptr<int32_t>(), image.data_ptr<float>(), final_T.data_ptr<float>(),
                              final_idx.data_ptr<int32_t>(), ws.data_ptr(), ws_bytes,
@@ -157,9 +157,9 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
     const bool prepared = prepared_grads.has_value() && prepared_grads->defined();
     if(prepared)
         TORCH_CHECK(prepared_grads->is_contiguous() && prepared_grads->scalar_type() == at::kFloat &&
-                        prepared_grads->numel() == n * DSX_GRAD_FLOATS && prepared_grads->device() == dev,
-                    "prepared_grads must be the float32 [N, 12] accumulator of this forward");
-    at::Tensor grads = prepared ? *prepared_grads : at::empty({n, DSX_GRAD_FLOATS}, f32);
+                        prepared_grads->numel() == (int64_t)(dsx_grads_bytes(n) / 4) && prepared_grads->device() == dev,
+                    "prepared_grads must be the float32 accumulator of this forward (dsx_grads_bytes(N) bytes)");
+    at::Tensor grads = prepared ? *prepared_grads : at::empty({(int64_t)(dsx_grads_bytes(n) / 4)}, f32);
     check(dsx_backward(&cam.c, n, (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
                        splats.data_ptr<float>(), fptr(cov3d_precomp), radii.data_ptr<int32_t>(),
                        ranges.data_ptr<int32_t>(), sorted_ids.numel() ? sorted_ids.data_ptr<int32_t>() : nullptr,

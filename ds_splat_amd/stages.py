@@ -221,6 +221,19 @@ def blend_bwd(cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image):
     return grads
 
 
+def new_accumulator(n, dev):
+    """The whole backward's accumulator as flat float32: dsx_grads_bytes(n) bytes, the n records of 12
+    floats and, behind them, the byte per Gaussian (see accumulator_views)."""
+    return torch.empty((int(N.load().dsx_grads_bytes(n)) // 4,), dtype=torch.float32, device=dev)
+
+
+def accumulator_views(grads, n):
+    """(records[n, 12] float32, marks[n] uint8) of a buffer of new_accumulator."""
+    records = grads[:n * N.GRAD_FLOATS].view(n, N.GRAD_FLOATS)
+    marks = grads[n * N.GRAD_FLOATS:].view(torch.uint8)[:n]
+    return records, marks
+
+
 def _bwd_outputs(n, num_bases, dev):
     e = lambda *s: torch.empty(s, dtype=torch.float32, device=dev)
     return dict(v_mean3d=e(n, 3), v_means2d=e(n, 3), v_shs=e(n, num_bases, 3) if num_bases > 0 else None,
@@ -303,7 +316,7 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     st.final_idx = torch.empty((cam.height, cam.width), dtype=torch.int32, device=dev)
     nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
-    st.grads = torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=dev) if prepare_grads else None
+    st.grads = new_accumulator(n, dev) if prepare_grads else None
     N.check(lib.dsx_forward_finish(cam.ref, n, k, _ptr(st.splats), _ptr(order), _ptr(st.sorted_ids),
                                    _ptr(st.lists), _ptr(image), _ptr(st.final_T), _ptr(st.final_idx), _ptr(ws),
                                    nbytes, _ptr(st.grads), stream))
@@ -317,12 +330,12 @@ def backward(cam, st, num_bases, means3d, scales, quats, v_image):
     o = _bwd_outputs(n, num_bases, dev)
     # an accumulator that the forward prepared serves one backward; after that it holds sums
     prepared = getattr(st, "grads", None) is not None
-    grads = st.grads if prepared else torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=dev)
+    grads = st.grads if prepared else new_accumulator(n, dev)
     st.grads = None
     N.check(lib.dsx_backward(cam.ref, n, num_bases, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(st.splats),
                              _ptr(st.cov3d), _ptr(st.radii), _ptr(st.lists), _ptr(st.sorted_ids), _ptr(st.final_T),
                              _ptr(st.final_idx), _ptr(v_image), _ptr(grads), int(prepared), _ptr(o["v_mean3d"]),
                              _ptr(o["v_means2d"]), _ptr(o["v_shs"]), _ptr(o["v_colors"]), _ptr(o["v_opacity"]),
                              _ptr(o["v_scale"]), _ptr(o["v_quat"]), _ptr(o["v_cov3d"]), _stream()))
-    o["grads"] = grads
+    o["grads"], o["marks"] = accumulator_views(grads, n)
     return o

@@ -73,11 +73,18 @@ typedef struct dsx_camera
  *
  * Gradient accumulator record, DSX_GRAD_FLOATS floats:
  *   [0] v_x [1] v_y [2] v_conic_a [3] v_conic_b [4] v_conic_c [5] v_opacity
- *   [6] v_red [7] v_green [8] v_blue [9..11] unused
+ *   [6] v_red [7] v_green [8] v_blue [9..11] unused (the conic, once dsx_forward_finish has prepared it)
+ * The accumulator of the whole backward (dsx_forward_finish's grads_to_prepare, dsx_backward's
+ * grads) is a buffer of dsx_grads_bytes(n) bytes, 16-byte aligned: the n records and, behind
+ * them, one byte per Gaussian that the blend backward sets when it adds a term to the record.
+ * The stage entry points dsx_blend_bwd / dsx_gaussian_bwd take the n records alone.
  */
 
 const char* dsx_error_string(int status);
 int dsx_version(void);
+/* bytes of the accumulator that dsx_forward_finish prepares and dsx_backward uses:
+ * n * DSX_GRAD_FLOATS * 4 for the records + n bytes rounded up to 16 */
+size_t dsx_grads_bytes(int64_t n);
 
 /* number of workgroups of the per-Gaussian kernels = entries of `block_sums` */
 int64_t dsx_num_blocks(int64_t n);
@@ -248,9 +255,10 @@ int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
  * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H).  If one of the two
  * sorts gave up a bounded wait (see dsx_sort_flags) the image is written as NaN: a failure
  * shows without a read-back of the flags.
- * grads_to_prepare (may be NULL; 16-byte aligned): the [n*12] accumulator that a dsx_backward of
- * this forward will use.  The blend kernel, which leaves the memory system idle, prepares it on
- * the side (the nine sums zeroed, each Gaussian's conic in the three spare places), and that
+ * grads_to_prepare (may be NULL; 16-byte aligned, dsx_grads_bytes(n) bytes): the accumulator that
+ * a dsx_backward of this forward will use.  The blend kernel, which leaves the memory system idle,
+ * prepares it on the side (the nine sums zeroed, each Gaussian's conic in the three spare places,
+ * the byte per Gaussian behind the records cleared), and that
  * dsx_backward is then called with grads_prepared = 1: it needs no fill of its own and its
  * per-Gaussian kernel does not fetch the splat records for the conic. */
 int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
@@ -258,9 +266,12 @@ int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float*
                        float* final_T, int32_t* final_idx, void* workspace,
                        size_t workspace_bytes, float* grads_to_prepare, void* stream);
 
-/* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316. grads is scratch [n*12];
- * grads_prepared != 0 says that dsx_forward_finish has prepared it (true for one call: this
- * one leaves sums in it). */
+/* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316. grads is scratch of
+ * dsx_grads_bytes(n) bytes, 16-byte aligned; grads_prepared != 0 says that dsx_forward_finish has
+ * prepared it (true for one call: this one leaves sums in it).  The outputs are as for
+ * dsx_gaussian_bwd: zero wherever the blend backward added no term to a Gaussian's record (most
+ * of a dense scene), written by the blend kernel's wavefronts on their way out; the per-Gaussian
+ * kernel then works on the marked Gaussians only. */
 int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
                  const float* scales, const float* quats, const float* splats, const float* cov3d,
                  const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
@@ -272,9 +283,9 @@ int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const floa
 /* dsx_backward for callers that cannot allocate or bring device scratch: code under HIP graph
  * capture, tight serving or training loops, harnesses that forbid hipMalloc.  No counterpart in
  * the reference (its backward allocates every temporary through torch).  The same computation and
- * the same arguments as dsx_backward, except that the [n * 12] gradient accumulator is not an
- * argument: it is a device array built into the library, DSX_STATIC_MAX_GAUSSIANS records =
- * 24 MiB, which every GPU the library runs on holds until the process ends.  The call allocates
+ * the same arguments as dsx_backward, except that the gradient accumulator is not an
+ * argument: it is a device array built into the library, dsx_grads_bytes(DSX_STATIC_MAX_GAUSSIANS) =
+ * 24.5 MiB, which every GPU the library runs on holds until the process ends.  The call allocates
  * and frees nothing, on the device or through any library; it returns DSX_ERR_STATIC_LIMIT for
  * n > DSX_STATIC_MAX_GAUSSIANS.  The array keeps the previous call's sums; each call clears the
  * n records it uses with a fill kernel (plain stores) before accumulating.  All calls on one GPU

@@ -211,8 +211,9 @@ def test_forward_prepares_the_accumulator_for_one_backward(blend_form, pixels_pe
     image1, st1 = stages.forward(cam, *args, prepare_grads=True)
     torch.cuda.synchronize()
     # nine sums zeroed, the conic (floats 4..6 of the splat record) in the three spare places
-    assert st0.grads is None and st1.grads.shape == (n, 12) and bool((st1.grads[:, :9] == 0).all())
-    assert torch.equal(st1.grads[:, 9:12], st1.splats[:, 4:7])
+    records, marks = stages.accumulator_views(st1.grads, n)
+    assert st0.grads is None and bool((records[:, :9] == 0).all()) and bool((marks == 0).all())
+    assert torch.equal(records[:, 9:12], st1.splats[:, 4:7])
     assert torch.equal(image0, image1)
     bwd = lambda st: stages.backward(cam, st, 16, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["v_image"])
     o0, o1 = bwd(st0), bwd(st1)
@@ -220,10 +221,19 @@ def test_forward_prepares_the_accumulator_for_one_backward(blend_form, pixels_pe
     o2 = bwd(st1)
     torch.cuda.synchronize()
     for k in o0:
+        if k == "marks":
+            continue
         cols = slice(0, 9) if k == "grads" else slice(None)   # the accumulator's spare places are not sums
         scale = max(1.0, float(o0[k].abs().max()))
         for other in (o1, o2):
             assert torch.allclose(o0[k][:, cols], other[k][:, cols], rtol=1e-3, atol=1e-4 * scale), k
+    # the byte per Gaussian: set wherever a sum is, the same set every time, and some but not all
+    for o in (o0, o1, o2):
+        unmarked = o["marks"] == 0
+        assert bool((o["grads"][unmarked][:, :9] == 0).all()) and torch.equal(o["marks"], o0["marks"])
+        assert 0 < int(unmarked.sum()) < n
+        for k in ("v_mean3d", "v_shs", "v_scale", "v_quat", "v_opacity"):
+            assert bool((o[k][unmarked] == 0).all()), k
 
 
 def test_backward_twice_through_the_api_gives_the_same_gradients():
