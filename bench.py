@@ -45,18 +45,21 @@ def measured_traffic(workload, num_keys):
                                     "scale_fetch": rec.get("scale_fetch"), "scale_write": rec.get("scale_write")}
 
 
-def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters):
+def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters, marked):
     """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch.
-    k: pairs of the tile lists as built (per bin of tiles); lists: how many lists they are partitioned into."""
+    k: pairs of the tile lists as built (per bin of tiles); lists: how many lists they are partitioned into;
+    marked: Gaussians whose accumulator record received a term in the blend backward."""
     slot_bytes = 2 if lists + 1 <= 65535 else 4
     if kernel == "project_fwd_kernel":
         # inputs 44 + 12c bytes, outputs radii + splat record + depth key + tile rectangle (the 3-D
         # covariance is not stored on this path: the backward rebuilds it)
         return "hbm", n * (44 + 12 * coeffs + 4 + 48 + 4 + 8), "B"
     if kernel == "gaussian_bwd_kernel":
-        # reads 88 (no stored covariance); writes v_mean3d 12 + v_means2d 12 + v_scale 12 + v_quat 16 + v_shs 12c
-        # (v_colors and v_cov3d are not written: the step gives neither colours nor covariances, so nothing takes them)
-        return "hbm", n * (88 + 52 + 12 * coeffs), "B"
+        # one byte per Gaussian (did its record receive a term?), then for the marked ones only: reads 88 (no
+        # stored covariance), writes v_mean3d 12 + v_means2d 12 + v_scale 12 + v_quat 16 + v_shs 12c (v_colors and
+        # v_cov3d are not written: the step gives neither colours nor covariances, so nothing takes them).  The
+        # zeros of everybody else's outputs are stored by the blend backward's wavefronts (n * (52 + 12c) bytes).
+        return "hbm", n + marked * (88 + 52 + 12 * coeffs), "B"
     if kernel == "hist32_kernel":
         return "hbm", 4 * n, "B"
     if kernel == "onesweep32_kernel<sort>":                  # depth sort of the Gaussians: key + id, in and out
@@ -232,6 +235,9 @@ def main():
     from ds_splat_amd import stages
     cam = stages.camera_from_scene(sc, dev)
     _, st = stages.forward(cam, t["means_3d"], t["scales"], t["rotations"], t["opacities"], t["shs"])
+    marked = 0
+    if do_backward:
+        marked = int(stages.backward(cam, st, 16, t["means_3d"], t["scales"], t["rotations"], v_image)["marks"].sum())
     torch.cuda.synchronize()
     k = st.num_keys
     tiles = cam.num_tiles
@@ -286,7 +292,7 @@ def main():
     for name, (tot, cnt) in per_kernel.items():
         launches_per_step = cnt / args.steps
         avg = tot / cnt
-        bound, work, unit = algorithmic_work(name, n, k, W * H, lists, coeffs, counters)
+        bound, work, unit = algorithmic_work(name, n, k, W * H, lists, coeffs, counters, marked)
         table.append((tot / args.steps, name, avg, launches_per_step, bound, work, unit))
     table.sort(reverse=True)
     measured, traffic_source = measured_traffic(spec.name, k) if args.n is None else ({}, None)
@@ -325,7 +331,7 @@ def main():
         "config": {"workload": "%s: %d Gaussians, %dx%d, SH degree %d, %s" %
                                (spec.name, n, W, H, sc["sh_degree"], "forward+backward" if do_backward else "forward"),
                    "num_keys": int(k), "num_keys_per_tile_lists": k_per_tile, "tiles": int(tiles),
-                   "list_bin_tiles": list_bin, "lists": int(lists)},
+                   "list_bin_tiles": list_bin, "lists": int(lists), "gaussians_with_gradient": marked},
         "mpix_per_s": round(W * H / (ms_per_step * 1e-3) / 1e6, 1),
         "ms_per_step_with_kernel_events": round(ms_per_step_traced, 4),
         # the host's share of a step (enqueue + the wait for the pair count) and the device's (sum of the
