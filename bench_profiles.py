@@ -76,8 +76,10 @@ def git_commit():
     try:
         head = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True,
                               check=True).stdout.strip()
-        dirty = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--untracked-files=no"],
-                               capture_output=True, text=True, check=True).stdout.strip()
+        status = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--untracked-files=no"],
+                                capture_output=True, text=True, check=True).stdout.splitlines()
+        # (the summaries under profiles/ are this tool's own output, not code that was measured)
+        dirty = [line for line in status if not line[3:].startswith("profiles/")]
         return head + ("+uncommitted changes" if dirty else "")
     except Exception:
         return "unknown"
@@ -143,7 +145,8 @@ def algorithmic_bytes(bench):
     out = {}
     for k in ("project_fwd_kernel", "gaussian_bwd_kernel", "hist32_kernel", "onesweep32_kernel<sort>",
               "ordered_block_sums_kernel", "emit_ordered_kernel", "onesweep32_kernel<tile partition>"):
-        bound, work, _ = bench_module.algorithmic_work(k, n, cfg["num_keys"], w * h, cfg["lists"], (deg + 1) ** 2, None)
+        bound, work, _ = bench_module.algorithmic_work(k, n, cfg["num_keys"], w * h, cfg["lists"], (deg + 1) ** 2, None,
+                                                       cfg.get("gaussians_with_gradient", 0))
         if bound == "hbm":
             out[k] = work
     return out, n
