@@ -73,8 +73,11 @@ def gpu_forward_state(sc, scale_mul=1.0):
 def check_grads(leaves, B, ok, what=""):
     got = {key: leaves[leaf].grad.cpu().numpy() for leaf, key in GRAD_KEYS}
     worst = check_grads_against_bounds(got, B, B["bounds"], ok, what)
-    print("%s: gradients of %d of %d Gaussians compared (%.1f %%), largest error / bound = %.3f" % (
-        what, int(ok.sum()), ok.size, 100.0 * ok.mean(), worst))
+    moved = B["abs_sums"].sum(axis=1) > 0      # Gaussians that receive any gradient term
+    print("%s: gradients of %d of %d Gaussians compared (%.1f %%), of the %d that receive a term %d (%.1f %%); "
+          "largest error / bound = %.3f" % (what, int(ok.sum()), ok.size, 100.0 * ok.mean(), int(moved.sum()),
+                                            int((ok & moved).sum()), 100.0 * (ok & moved).sum() / max(1, moved.sum()),
+                                            worst))
     return worst
 
 
