@@ -106,7 +106,7 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--list-bin", type=int, default=0, choices=(0, 1, 2, 4),
+    ap.add_argument("--list-bin", type=int, default=0, choices=(0, 1, 2, 4, 8),
                     help="tiles per side of the bins the tile lists are built for (0: the library's choice)")
     ap.add_argument("--verbose", action="store_true", help="per-kernel table on stderr")
     ap.add_argument("--copy-probe", action="store_true",

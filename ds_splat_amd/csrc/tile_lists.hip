@@ -44,16 +44,21 @@ static hipStream_t helper_stream()
     return streams[device];
 }
 
-// Bin size of the tile lists: 4 x 4 tiles from 2048 tiles on (a Gaussian's rectangle then touches a
-// few bins instead of a dozen tiles, and emission and partition shrink accordingly), one list per
-// tile below: a 256 x 256 image has 16 bins, and its 1024 blend wavefronts (four per tile there)
-// would each filter a list sixteen times the tile's own (measured: forward 0.175 ms with lists per
-// tile, 0.186 with bins of 2 x 2, 0.208 with 4 x 4).  set_list_bin overrides it for the process.
+// Bin size of the tile lists: one list per tile below 2048 tiles (a 256 x 256 image has 16 bins of
+// 4 x 4, and its 1024 blend wavefronts, four per tile there, would each filter a list sixteen times
+// the tile's own: forward 0.175 ms with lists per tile, 0.186 with bins of 2 x 2, 0.208 with 4 x 4);
+// from 2048 tiles on, bins of 4 x 4 tiles (a Gaussian's rectangle then touches a few bins instead of
+// a dozen tiles, and emission and partition shrink accordingly), or of 8 x 8 where that brings the
+// lists, slot 0 included, down to the 256 that ONE partition pass handles (1920 x 1080: 135 lists
+// instead of 510; 3 M small Gaussians 0.840 -> 0.827 ms per step, 1 M large ones 1.04 -> 0.68; a
+// 3840 x 2160 image needs two passes either way and its forward is slower with the larger bins,
+// 1.24 -> 1.32 ms, because every tile filters four times as many entries).  set_list_bin overrides
+// the choice for the process.
 static std::atomic<int> g_list_bin{0};
 
 int set_list_bin(int tiles_per_side)
 {
-    if(tiles_per_side != 0 && tiles_per_side != 1 && tiles_per_side != 2 && tiles_per_side != 4)
+    if(tiles_per_side != 0 && tiles_per_side != 1 && tiles_per_side != 2 && tiles_per_side != 4 && tiles_per_side != 8)
         return DSX_ERR_BAD_ARG;
     g_list_bin.store(tiles_per_side, std::memory_order_relaxed);
     return DSX_OK;
@@ -65,8 +70,13 @@ ListGrid list_grid(int image_width, int image_height)
     g.ntx = tiles_x(image_width);
     g.nty = tiles_y(image_height);
     const int forced = g_list_bin.load(std::memory_order_relaxed);
-    const int side = forced ? forced : (g.ntx * g.nty >= 2048 ? 4 : 1);
-    g.shift = side == 4 ? 2 : (side == 2 ? 1 : 0);
+    int side = forced ? forced : 1;
+    if(!forced && g.ntx * g.nty >= 2048)
+    {
+        auto lists = [&](int b) { return ((g.ntx + b - 1) / b) * ((g.nty + b - 1) / b); };
+        side = (slot_bits(lists(4)) > 8 && slot_bits(lists(8)) <= 8) ? 8 : 4;
+    }
+    g.shift = side == 8 ? 3 : (side == 4 ? 2 : (side == 2 ? 1 : 0));
     g.nbx = (g.ntx + side - 1) / side;
     g.nby = (g.nty + side - 1) / side;
     return g;

@@ -92,13 +92,14 @@ int64_t dsx_num_blocks(int64_t n);
 int32_t dsx_num_tiles(int32_t width, int32_t height);
 int32_t dsx_sort_passes(int32_t num_tiles);
 /* The tile lists of the whole forward (dsx_forward_project / dsx_forward_finish / dsx_backward,
- * dsx_depth_order / dsx_tile_lists) are built per BIN of b x b tiles, b = 1, 2 or 4: a Gaussian
+ * dsx_depth_order / dsx_tile_lists) are built per BIN of b x b tiles, b = 1, 2, 4 or 8: a Gaussian
  * enters the list of every bin that its tile rectangle touches, and a blend tile walks its bin's
  * list and keeps the entries whose rectangle contains the tile.  With b = 1 the lists are the
  * reference's own (sorted_ids is the value array of its sorted keys, bit for bit); with b > 1 the
  * same entries reach every pixel in the same order, final_idx holds the same indices, and emission
  * and partition handle a fraction of the pairs.  dsx_list_bin says which b the library uses for an
- * image size (4 from 2048 tiles on, else 1); dsx_set_list_bin forces one for the whole process
+ * image size (1 below 2048 tiles; above, 8 where that brings the lists down to the 256 slots of a
+ * single partition pass and 4 does not, else 4); dsx_set_list_bin forces one for the whole process
  * (0: back to the library's choice) — not between the two halves of a forward or between a
  * forward and its backward.  dsx_ranges_count: int32 words of the `ranges` buffer of those entry
  * points: tiles + 1 words of per-tile ranges as the reference defines them and, for b > 1, the

@@ -63,8 +63,12 @@ def test_host_helpers():
     # bins of the tile lists: 4 x 4 tiles from 2048 tiles on, unless forced; the `ranges` buffer grows with them
     assert lib.dsx_list_bin(1920, 1080) == 1 and lib.dsx_ranges_count(1920, 1080) == 8160 + 1
     assert lib.dsx_set_list_bin(0) == 0 and lib.dsx_set_list_bin(3) == -1
-    assert lib.dsx_list_bin(1920, 1080) == 4 and lib.dsx_list_bin(1024, 512) == 4 and lib.dsx_list_bin(1024, 496) == 1
-    assert lib.dsx_ranges_count(1920, 1080) == (8160 + 1) + 1 + (30 * 17 + 1) + 8 * 8160
+    # per tile below 2048 tiles; 8 x 8 where that needs one partition pass and 4 x 4 two (1080p: 135 against
+    # 510 lists); 4 x 4 where it fits one pass itself (128 lists) or where both need two (4K: 510 against 2040)
+    assert lib.dsx_list_bin(1920, 1080) == 8 and lib.dsx_list_bin(1024, 512) == 4 and lib.dsx_list_bin(1024, 496) == 1
+    assert lib.dsx_list_bin(3840, 2160) == 4 and lib.dsx_set_list_bin(8) == 0 and lib.dsx_list_bin(640, 480) == 8
+    assert lib.dsx_set_list_bin(0) == 0
+    assert lib.dsx_ranges_count(1920, 1080) == (8160 + 1) + 1 + (15 * 9 + 1) + 8 * 8160
     assert lib.dsx_ranges_count(240, 240) == 225 + 1
     assert lib.dsx_sort_workspace_bytes(1 << 20, 8160) > (1 << 20) * 12
     assert lib.dsx_sort_u32_workspace_bytes(1 << 20, 32) > (1 << 20) * 8

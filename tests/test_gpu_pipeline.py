@@ -93,7 +93,8 @@ def check_grads(leaves, B, ok, what=""):
     ("cfg0", 16384, 256, 256, 3, 2.0, (0.2, 0.4, 0.9), "rotated", 2),
     ("cfg0", 20000, 320, 200, 3, 2.0, None, "inside", 4),
     ("cfg1", 40000, 480, 270, 3, 1.5, (0.5, 0.1, 0.3), "anisotropic", 1),
-    ("cfg4", 3000, 320, 180, 2, 0.5, None, "rotated", 4),
+    ("cfg4", 3000, 320, 180, 2, 0.5, None, "rotated", 8),
+    ("cfg1", 40000, 640, 360, 3, 2.0, (0.3, 0.3, 0.3), "inside", 8),
     ("cfg1", 40000, 1000, 520, 3, 2.0, (0.1, 0.2, 0.3), "rotated", 0),  # 63 x 33 tiles: ragged against the bins
 ])
 @pytest.mark.parametrize("pixels_per_lane", ["1", "4"])
@@ -123,7 +124,7 @@ def test_api_forward_backward_vs_oracle(oracle, name, n, W, H, deg, scale_mul, b
     assert (leaves["means2d"].grad[:, 2] == 0).all()
 
 
-@pytest.mark.parametrize("bins", [1, 2, 4])
+@pytest.mark.parametrize("bins", [1, 2, 4, 8])
 def test_api_internal_integers_bit_exact(oracle, list_bin, bins):
     """Tile ranges, tile counts, radii and last blended index of the whole forward, bit for bit,
     whatever the bin size of the lists; with one list per tile also the sorted order itself

@@ -21,7 +21,7 @@ def draw(rng):
     c["pick"] = rng.integers(0, n, c["giants"])
     # half of the scenes through a camera drawn at random: anywhere around (or inside) the cloud,
     # rolled, non-square pixels, a scale modifier
-    c["bins"] = int(rng.choice([1, 2, 4]))      # tiles per side of the bins the lists are built for
+    c["bins"] = int(rng.choice([1, 2, 4, 8]))      # tiles per side of the bins the lists are built for
     c["camera"] = None
     if rng.random() < 0.5:
         eye = rng.uniform([-4.0, -3.0, -3.0], [4.0, 3.0, 8.0])

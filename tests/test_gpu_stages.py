@@ -325,17 +325,17 @@ def test_tile_lists_with_general_cameras(oracle, list_bin, camera):
     test_tile_lists_bit_exact(oracle, list_bin, 30000, 640, 360, 3.0, 0, camera=camera)
 
 
-@pytest.mark.parametrize("bin_side", [2, 4])
+@pytest.mark.parametrize("bin_side", [2, 4, 8])
 @pytest.mark.parametrize("n,W,H,scale_mul,flip,giants,camera", [
     (20000, 256, 256, 2.0, 0, 0, "identity"), (3000, 200, 120, 12.0, 0, 0, "identity"),
     (500, 64, 48, 3.0, 120, 0, "identity"), (1, 32, 32, 1.0, 0, 0, "identity"), (2, 32, 32, 1.0, 0, 0, "identity"),
     (30000, 1280, 720, 0.5, 40, 25, "identity"), (30000, 640, 360, 3.0, 0, 0, "inside"),
-    (20000, 1000, 520, 4.0, 100, 0, "anisotropic"),      # 63 x 33 tiles: ragged against bins of 2 and of 4
+    (20000, 1000, 520, 4.0, 100, 0, "anisotropic"),      # 63 x 33 tiles: ragged against every bin size
     (60, 1920, 1080, 2.0, 30, 0, "identity"),             # most bins empty
     (300, 500, 300, 2.0, 300, 0, "identity"),             # every Gaussian behind the camera: slot 0 only
 ])
 def test_binned_tile_lists_vs_oracle(oracle, list_bin, bin_side, n, W, H, scale_mul, flip, giants, camera):
-    """Lists per bin of 2 x 2 or 4 x 4 tiles: every bin's list holds the Gaussians whose tile
+    """Lists per bin of 2 x 2, 4 x 4 or 8 x 8 tiles: every bin's list holds the Gaussians whose tile
     rectangle touches the bin, by (depth bits, index); slot 0 is the oracle's own run of negative-depth
     pairs; the per-tile ranges (with the reference's rules about the last run) and the highest occupied
     tile are those of the oracle's fully sorted keys.  Bit for bit."""
