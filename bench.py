@@ -303,6 +303,13 @@ def main():
             continue
         traffic = measured.get(name)
         entry = roofline_entry(name, avg, lps, bound, work, int(traffic) if traffic else None)
+        # the blend kernels carry stores for their neighbours (the launch time and the traffic include them,
+        # the algorithmic work does not): the forward prepares the backward's accumulator, the backward
+        # writes the zeros of the per-Gaussian backward's outputs
+        if name == "blend_bwd_kernel":
+            entry["side_job_bytes"] = int(n * (52 + 12 * coeffs))
+        elif name == "blend_fwd_kernel" and do_backward:
+            entry["side_job_bytes"] = int(n * (48 + 16 + 48 + 1))
         if roofline is None:
             roofline = entry
         if roofline_hbm is None and bound == "hbm":
