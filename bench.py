@@ -309,7 +309,7 @@ def main():
         if name == "blend_bwd_kernel":
             entry["side_job_bytes"] = int(n * (52 + 12 * coeffs))
         elif name == "blend_fwd_kernel" and do_backward:
-            entry["side_job_bytes"] = int(n * (48 + 16 + 48 + 1))
+            entry["side_job_bytes"] = int(n * (48 + 16 + 1))   # record written, conic read, mark cleared
         if roofline is None:
             roofline = entry
         if roofline_hbm is None and bound == "hbm":
