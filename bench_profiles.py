@@ -8,21 +8,21 @@ bench.py quotes as `roofline.traffic` (with the commit the counters were taken a
 
     # on the MI355X box, repository root (each counter set in a run of its own):
     export TMPDIR=/tmp
-    rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof -o bench -- \\
+    rocprofv3 --kernel-trace --stats --output-format csv -d out/prof -o bench -- \\
         python3 bench.py --steps 20 --warmup 5 --no-cpu-baseline
-    rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/pmc_fetch -o f -- \\
-        python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe > gpurun_out/pmc_fetch.json
-    rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -o w -- \\
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out/pmc_fetch -o f -- \\
+        python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe > out/pmc_fetch.json
+    rocprofv3 --pmc WRITE_SIZE --output-format csv -d out/pmc_write -o w -- \\
         python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe
     rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_INSTS_SALU \\
-        SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT --output-format csv -d gpurun_out/pmc_sq -o s -- \\
+        SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT --output-format csv -d out/pmc_sq -o s -- \\
         python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline
 
     # anywhere the CSV files are (the commit is read from git when --commit is not given):
-    python3 bench_profiles.py stats   gpurun_out/prof --name bench_cfg2_fwd_bwd_kernel_stats
-    python3 bench_profiles.py traffic gpurun_out/pmc_fetch gpurun_out/pmc_write --bench-json gpurun_out/pmc_fetch.json \\
+    python3 bench_profiles.py stats   out/prof --name bench_cfg2_fwd_bwd_kernel_stats
+    python3 bench_profiles.py traffic out/pmc_fetch out/pmc_write --bench-json out/pmc_fetch.json \\
         --name cfg2_hbm_traffic_per_kernel
-    python3 bench_profiles.py sq      gpurun_out/pmc_sq gpurun_out/prof --name cfg2_sq_counters_per_kernel
+    python3 bench_profiles.py sq      out/pmc_sq out/prof --name cfg2_sq_counters_per_kernel
 """
 import argparse
 import collections
@@ -38,15 +38,20 @@ import sys
 ROOT = os.path.dirname(os.path.abspath(__file__))
 PROFILES = os.path.join(ROOT, "profiles")
 
-STATS_CMD = ("rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof -o bench -- "
+# the commands whose output this tool reads; {dir} is the directory that the tool was given
+STATS_CMD = ("rocprofv3 --kernel-trace --stats --output-format csv -d {dir} -o bench -- "
              "python3 bench.py --steps 20 --warmup 5 --no-cpu-baseline")
-FETCH_CMD = ("rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/pmc_fetch -o f -- "
+FETCH_CMD = ("rocprofv3 --pmc FETCH_SIZE --output-format csv -d {dir} -o f -- "
              "python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe")
-WRITE_CMD = ("rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -o w -- "
+WRITE_CMD = ("rocprofv3 --pmc WRITE_SIZE --output-format csv -d {dir} -o w -- "
              "python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe")
 SQ_CMD = ("rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_INSTS_SALU "
-          "SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT --output-format csv -d gpurun_out/pmc_sq -o s -- "
+          "SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT --output-format csv -d {dir} -o s -- "
           "python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline")
+
+
+def command(template, directory):
+    return template.format(dir=os.path.normpath(directory))
 
 
 def short_name(kernel):
@@ -123,7 +128,7 @@ def cmd_stats(args):
         for r in csv.DictReader(open(sorted(trace)[-1])):
             med[r["Kernel_Name"]].append(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]))
     lines = ["# %s" % args.title, "", "Commit: %s" % (args.commit or git_commit()), "",
-             "Command (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "", "    " + STATS_CMD, "",
+             "Command (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "", "    " + command(STATS_CMD, args.dir), "",
              "rocprofv3 kernel statistics (all launches of the run, warm-up included; the median is taken from the",
              "kernel trace of the same run):", "",
              "| kernel | calls | total ms | avg us | median us | % |", "|---|---|---|---|---|---|"]
@@ -165,8 +170,9 @@ def cmd_traffic(args):
     lines = ["# HBM traffic per launch (FETCH_SIZE / WRITE_SIZE), %s" % cfg["workload"], "",
              "Commit: %s" % commit, "",
              "Commands (on the MI355X box, repository root, after `export TMPDIR=/tmp`; one counter per run):", "",
-             "    " + FETCH_CMD, "    " + WRITE_CMD,
-             "    python3 bench_profiles.py traffic gpurun_out/pmc_fetch gpurun_out/pmc_write --bench-json <the first run's JSON line> --name %s" % args.name,
+             "    " + command(FETCH_CMD, args.fetch_dir), "    " + command(WRITE_CMD, args.write_dir),
+             "    python3 bench_profiles.py traffic %s %s --bench-json <the first run's JSON line> --name %s" % (
+                 os.path.normpath(args.fetch_dir), os.path.normpath(args.write_dir), args.name),
              "",
              "Calibration: `--copy-probe` runs one 1 GiB device-to-device copy (`%s`, reads 1048576 KiB, writes 1048576 KiB)." % copy,
              "The counters read FETCH_SIZE = %.1f KiB and WRITE_SIZE = %.1f KiB for it, so the scale factors are %.4f (fetch) and %.4f (write)." % (
@@ -206,8 +212,8 @@ def cmd_sq(args):
     times = kernel_times_ms(args.stats_dir)
     avg = lambda x: sum(x) / len(x)
     lines = ["# SQ counters per kernel (VALU issue, LDS bank conflicts)", "", "Commit: %s" % (args.commit or git_commit()), "",
-             "Commands (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "", "    " + SQ_CMD,
-             "    " + STATS_CMD + "    # the `kernel ms` column", "",
+             "Commands (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "", "    " + command(SQ_CMD, args.sq_dir),
+             "    " + command(STATS_CMD, args.stats_dir) + "    # the `kernel ms` column", "",
              "Averages per launch. A wave64 VALU instruction occupies its SIMD for 4 clocks, so the chip (256 CU x 4 SIMD at 2.4 GHz)",
              "issues at most 614 G wave-instructions/s: `VALU floor` = SQ_INSTS_VALU / 614e9 is the time the kernel's VALU",
              "instructions alone need (quarter-rate instructions such as exp and rcp count once here, so the true floor is higher);",
