@@ -35,7 +35,7 @@ def blend_form():
 
 @pytest.fixture
 def list_bin():
-    """Returns a function that forces the bin size of the tile lists (1, 2 or 4 tiles a side; 0: the
+    """Returns a function that forces the bin size of the tile lists (1, 2, 4 or 8 tiles a side; 0: the
     library's choice) for the rest of the test; the library's own choice is restored afterwards."""
     from ds_splat_amd import _native
     lib = _native.load()
