@@ -124,7 +124,7 @@ extern "C" const char* dsx_error_string(int status)
 
 extern "C" int dsx_version(void)
 {
-    return 100;
+    return 200;
 }
 
 extern "C" int64_t dsx_num_blocks(int64_t n)

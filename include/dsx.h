@@ -81,6 +81,8 @@ typedef struct dsx_camera
  */
 
 const char* dsx_error_string(int status);
+/* 100 * major + minor.  200: the `ranges` buffer has dsx_ranges_count words and the accumulator
+ * dsx_grads_bytes bytes (100 had tiles + 1 words and n * 12 floats). */
 int dsx_version(void);
 /* bytes of the accumulator that dsx_forward_finish prepares and dsx_backward uses:
  * n * DSX_GRAD_FLOATS * 4 for the records + n bytes rounded up to 16 */
