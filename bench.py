@@ -45,7 +45,7 @@ def measured_traffic(workload, num_keys):
                                     "scale_fetch": rec.get("scale_fetch"), "scale_write": rec.get("scale_write")}
 
 
-def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters, marked):
+def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters, marked, carries_rects=True):
     """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch.
     k: pairs of the tile lists as built (per bin of tiles); lists: how many lists they are partitioned into;
     marked: Gaussians whose accumulator record received a term in the blend backward."""
@@ -62,8 +62,10 @@ def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters, marked):
         return "hbm", n + marked * (88 + 52 + 12 * coeffs), "B"
     if kernel == "hist32_kernel":
         return "hbm", 4 * n, "B"
-    if kernel == "onesweep32_kernel<sort>":                  # depth sort of the Gaussians: key + id, in and out
-        return "hbm", 16 * n, "B"
+    if kernel == "onesweep32_kernel<sort>":
+        # depth sort of the Gaussians: key + id, in and out; images of at most 127 x 127 tiles also carry each
+        # Gaussian's packed tile rectangle through the passes (4 bytes in and out) instead of gathering them
+        return "hbm", (24 if carries_rects else 16) * n, "B"
     if kernel == "ordered_block_sums_kernel":
         return "hbm", 8 * n, "B"
     if kernel == "emit_ordered_kernel":
@@ -292,7 +294,8 @@ def main():
     for name, (tot, cnt) in per_kernel.items():
         launches_per_step = cnt / args.steps
         avg = tot / cnt
-        bound, work, unit = algorithmic_work(name, n, k, W * H, lists, coeffs, counters, marked)
+        bound, work, unit = algorithmic_work(name, n, k, W * H, lists, coeffs, counters, marked,
+                                             (W + 15) // 16 <= 127 and (H + 15) // 16 <= 127)
         table.append((tot / args.steps, name, avg, launches_per_step, bound, work, unit))
     table.sort(reverse=True)
     measured, traffic_source = measured_traffic(spec.name, k) if args.n is None else ({}, None)

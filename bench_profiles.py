@@ -151,7 +151,8 @@ def algorithmic_bytes(bench):
     for k in ("project_fwd_kernel", "gaussian_bwd_kernel", "hist32_kernel", "onesweep32_kernel<sort>",
               "ordered_block_sums_kernel", "emit_ordered_kernel", "onesweep32_kernel<tile partition>"):
         bound, work, _ = bench_module.algorithmic_work(k, n, cfg["num_keys"], w * h, cfg["lists"], (deg + 1) ** 2, None,
-                                                       cfg.get("gaussians_with_gradient", 0))
+                                                       cfg.get("gaussians_with_gradient", 0),
+                                                       (w + 15) // 16 <= 127 and (h + 15) // 16 <= 127)
         if bound == "hbm":
             out[k] = work
     return out, n

@@ -235,6 +235,7 @@ struct OrderLayout
     size_t ids_b;      // uint32[n]
     size_t rects;      // uint2[n]   packed tile rectangle (written by the projection)
     size_t rects_sorted; // uint2[n] the same in depth order
+    size_t rects32;    // uint32[n]  packed rectangles on their way through the depth sort
     size_t block_sums; // uint32[blocks + 1] tile counts of 256 consecutive Gaussians IN DEPTH ORDER, scanned
     size_t slot_hist;  // uint32[kMaxPasses32 * 256] digit histograms of the tile slots of all pairs
     size_t cover;      // int32[(ntx + 1) * (nty + 1) + 1] pairs per tile (corner grid, then its 2-D prefix sum)
@@ -263,7 +264,8 @@ ListsWorkspace lists_workspace(int64_t k, int num_tiles);
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
                   uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src = nullptr,
-                  uint2* gather_dst = nullptr, bool already_cleared = false);
+                  uint2* gather_dst = nullptr, bool already_cleared = false, uint32_t* carry_a = nullptr,
+                  uint32_t* carry_b = nullptr);
 // already_cleared: the words of depth_order_clear_region are zero already (the projection did it)
 int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream,
                        bool already_cleared = false, void* k_host = nullptr, hipEvent_t k_copied = nullptr);

@@ -229,17 +229,46 @@ constexpr int kLookBatch32 = DSX_LOOK32;
 static_assert(kDepthSortThreads >= kBins32 && kListSortThreads >= kBins32, "one thread per digit");
 static_assert(kDepthSortTile <= 65535 && kListSortTile <= 65535, "u16 ranks");
 
+// A tile rectangle as the projection packs it (16-bit fields) in 29 bits: 7 bits each for first
+// column, first row, width and height, then the depth's sign.  For images of at most 127 x 127 tiles.
+constexpr int kRect32MaxTiles = 127;
+__device__ __forceinline__ uint32_t rect_to_32(uint2 r)
+{
+    return (r.x & 0x7fu) | (((r.x >> 16) & 0x7fu) << 7) | ((r.y & 0x7fu) << 14) | (((r.y >> 16) & 0x7fu) << 21) |
+           ((r.y >> 31) << 28);
+}
+__device__ __forceinline__ uint2 rect_from_32(uint32_t v)
+{
+    return make_uint2((v & 0x7fu) | (((v >> 7) & 0x7fu) << 16),
+                      ((v >> 14) & 0x7fu) | (((v >> 21) & 0x7fu) << 16) | ((v >> 28) << 31));
+}
+
+// What a pass does about the Gaussians' tile rectangles, which the emission wants in depth order.
+// Either the last pass gathers them (gather_dst[position] = gather_src[value]; a pair whose key is
+// kNoPairsKey gets a zero record without the read): 1.9 M random 8-byte reads that pull 128-byte
+// lines.  Or every pass carries the rectangle as a second 32-bit value (kCarry): the first pass
+// reads the rectangles in index order, packs them (pack_src), the passes in between move them like
+// the values (carry_in -> carry_out), and the last pass unpacks into unpack_dst.
+struct RectJob
+{
+    const uint2* gather_src;
+    uint2* gather_dst;
+    const uint2* pack_src;
+    const uint32_t* carry_in;
+    uint32_t* carry_out;
+    uint2* unpack_dst;
+};
+
 // vals_in == nullptr: the values are the input positions (iota).  keys_out == nullptr: the
-// keys are not needed after this pass.  gather_src != nullptr: gather_dst[position] =
-// gather_src[value] for every pair, except that a pair whose key is kNoPairsKey gets a zero
-// record without the read.  KeyT: uint32_t, or uint16_t for tile slots that fit.
-template <typename KeyT, int kSort32Threads, int kSort32Items>
+// keys are not needed after this pass.  KeyT: uint32_t, or uint16_t for tile slots that fit.
+template <typename KeyT, int kSort32Threads, int kSort32Items, bool kCarry>
 __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
     const KeyT* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, KeyT* __restrict__ keys_out,
     uint32_t* __restrict__ vals_out, int64_t count, int shift, uint32_t mask, const uint32_t* __restrict__ hist_counts,
-    uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag, const uint2* __restrict__ gather_src,
-    uint2* __restrict__ gather_dst)
+    uint32_t* status, uint32_t* tile_counter, uint32_t* error_flag, const RectJob rects)
 {
+    const uint2* __restrict__ gather_src = rects.gather_src;
+    uint2* __restrict__ gather_dst = rects.gather_dst;
     constexpr int kSort32Tile = kSort32Threads * kSort32Items;
     constexpr int kSort32Waves = kSort32Threads / DSX_WAVE;
     __shared__ uint32_t s_keys[kSort32Tile]; // reused for the values in the second round
@@ -369,6 +398,19 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
         if(local < tile_n)
             val[it] = vals_in ? __builtin_nontemporal_load(vals_in + tile_base + local) : (uint32_t)(tile_base + local);
     }
+    uint32_t carried[kCarry ? kSort32Items : 1];
+    if(kCarry)
+    {
+#pragma unroll
+        for(int it = 0; it < kSort32Items; ++it)
+        {
+            const int local = wave * (kSort32Items * 64) + it * 64 + lane;
+            carried[it] = 0;
+            if(local < tile_n)
+                carried[it] = rects.pack_src ? rect_to_32(rects.pack_src[tile_base + local])
+                                             : __builtin_nontemporal_load(rects.carry_in + tile_base + local);
+        }
+    }
 
     // ---- chained scan over earlier tiles (decoupled look-back), one thread per digit -------
     if(digit_thread)
@@ -467,6 +509,31 @@ __global__ __launch_bounds__(kSort32Threads) void onesweep32_kernel(
                 gather_dst[out] = ((no_record >> it) & 1u) ? make_uint2(0u, 0u) : gather_src[v];
         }
     }
+    if(kCarry)
+    {
+        // ---- the carried rectangles through the same buffer, same positions ------------------
+        __syncthreads();
+#pragma unroll
+        for(int it = 0; it < kSort32Items; ++it)
+            s_keys[(pos2[it >> 1] >> (16 * (it & 1))) & 0xffffu] = carried[it];
+        __syncthreads();
+#pragma unroll
+        for(int it = 0; it < kSort32Items; ++it)
+        {
+            const int j = it * kSort32Threads + tid;
+            if((it & 3) == 0)
+                __builtin_amdgcn_sched_barrier(0);
+            if(j < tile_n)
+            {
+                const uint32_t v = s_keys[j];
+                const uint32_t out = s_gbase[(dig4[it >> 2] >> (8 * (it & 3))) & 0xffu] + (uint32_t)j;
+                if(rects.unpack_dst)
+                    rects.unpack_dst[out] = rect_from_32(v);
+                else
+                    rects.carry_out[out] = v;
+            }
+        }
+    }
 }
 
 Sort32Workspace sort32_workspace(int64_t count, int key_bits, int tile_keys)
@@ -500,11 +567,16 @@ static int sort32_clear(int64_t count, int key_bits, int tile_keys, void* sort_w
 // histogram area when counts is null).
 // Ping-pong between (keys_a, vals_a) and (keys_b, vals_b); *keys_out / *vals_out say where the
 // result is (keys only when keep_keys).
-template <typename KeyT, int kThreads, int kItems>
+// gather_src / gather_dst: records that the last pass brings to the values' sorted positions by a
+// gather.  carry_a / carry_b (with gather_src and gather_dst): the records travel through the passes
+// as packed 32-bit values instead, in ping-pong buffers of their own (the first pass packs them from
+// gather_src, the last one unpacks them into gather_dst).
+template <typename KeyT, int kThreads, int kItems, bool kCarry = false>
 static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* vals_a, KeyT* keys_b, uint32_t* vals_b,
                          bool iota_values, bool keep_keys, void* sort_ws, const char* label, hipStream_t stream,
                          KeyT** keys_out, uint32_t** vals_out, const uint2* gather_src = nullptr,
-                         uint2* gather_dst = nullptr, const uint32_t* counts = nullptr)
+                         uint2* gather_dst = nullptr, const uint32_t* counts = nullptr, uint32_t* carry_a = nullptr,
+                         uint32_t* carry_b = nullptr)
 {
     const Sort32Workspace w = sort32_workspace(count, key_bits, kThreads * kItems);
     const Digits32 plan = digits32(key_bits);
@@ -517,17 +589,31 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
     uint32_t* vin = vals_a;
     KeyT* kout = keys_b;
     uint32_t* vout = vals_b;
+    uint32_t* cin = carry_a;
+    uint32_t* cout = carry_b;
     for(int p = 0; p < w.passes; ++p)
     {
         const bool last = p == w.passes - 1;
+        RectJob job = {};
+        if(kCarry)
+        {
+            job.pack_src = p == 0 ? gather_src : nullptr;
+            job.carry_in = cin;
+            job.carry_out = cout;
+            job.unpack_dst = last ? gather_dst : nullptr;
+        }
+        else if(last)
+        {
+            job.gather_src = gather_src;
+            job.gather_dst = gather_dst;
+        }
         {
             DSX_TIMED(label, stream);
-            hipLaunchKernelGGL((onesweep32_kernel<KeyT, kThreads, kItems>), dim3((unsigned)w.tiles), dim3(kThreads), 0, stream,
-                               (const KeyT*)kin, (const uint32_t*)((p == 0 && iota_values) ? nullptr : vin),
+            hipLaunchKernelGGL((onesweep32_kernel<KeyT, kThreads, kItems, kCarry>), dim3((unsigned)w.tiles), dim3(kThreads), 0,
+                               stream, (const KeyT*)kin, (const uint32_t*)((p == 0 && iota_values) ? nullptr : vin),
                                (last && !keep_keys) ? (KeyT*)nullptr : kout, vout, count, plan.shift[p], plan.mask[p],
                                raw + p * kBins32, status + (size_t)p * w.tiles * kBins32,
-                               counters + p, counters + w.passes, last ? gather_src : (const uint2*)nullptr,
-                               last ? gather_dst : (uint2*)nullptr);
+                               counters + p, counters + w.passes, job);
         }
         DSX_LAUNCH_CHECK();
         KeyT* tk = kin;
@@ -536,6 +622,9 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
         uint32_t* tv = vin;
         vin = vout;
         vout = tv;
+        uint32_t* tc = cin;
+        cin = cout;
+        cout = tc;
     }
     *keys_out = kin;
     *vals_out = vin;
@@ -546,7 +635,7 @@ static int sort32_passes(int64_t count, int key_bits, KeyT* keys_a, uint32_t* va
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,
                   uint32_t* vals_b, bool iota_values, bool keep_keys, void* sort_ws, hipStream_t stream,
                   uint32_t** keys_out, uint32_t** vals_out, const uint2* gather_src, uint2* gather_dst,
-                  bool already_cleared)
+                  bool already_cleared, uint32_t* carry_a, uint32_t* carry_b)
 {
     *keys_out = keys_a;
     *vals_out = vals_a;
@@ -566,7 +655,18 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
                            reinterpret_cast<uint32_t*>(static_cast<char*>(sort_ws) + w.hist));
     }
     DSX_LAUNCH_CHECK();
-    if(sort32_tile_keys(count) == kListSortTile)
+    const bool large = sort32_tile_keys(count) == kListSortTile;
+    if(carry_a && carry_b && gather_src && gather_dst)
+    {
+        if(large)
+            return sort32_passes<uint32_t, kListSortThreads, kListSortItems, true>(
+                count, key_bits, keys_a, vals_a, keys_b, vals_b, iota_values, keep_keys, sort_ws,
+                "onesweep32_kernel<sort>", stream, keys_out, vals_out, gather_src, gather_dst, nullptr, carry_a, carry_b);
+        return sort32_passes<uint32_t, kDepthSortThreads, kDepthSortItems, true>(
+            count, key_bits, keys_a, vals_a, keys_b, vals_b, iota_values, keep_keys, sort_ws, "onesweep32_kernel<sort>",
+            stream, keys_out, vals_out, gather_src, gather_dst, nullptr, carry_a, carry_b);
+    }
+    if(large)
         return sort32_passes<uint32_t, kListSortThreads, kListSortItems>(count, key_bits, keys_a, vals_a, keys_b, vals_b,
                                                                          iota_values, keep_keys, sort_ws,
                                                                          "onesweep32_kernel<sort>", stream, keys_out,
@@ -598,6 +698,8 @@ OrderLayout order_layout(int64_t n, int image_width, int image_height)
     off = align(off + (size_t)n * 8);
     o.rects_sorted = off;
     off = align(off + (size_t)n * 8);
+    o.rects32 = off;
+    off = align(off + (size_t)n * 4);
     o.block_sums = off;
     off = align(off + (size_t)((n + kProjBlock - 1) / kProjBlock + 1) * 4);
     o.slot_hist = off;
@@ -1077,9 +1179,14 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
 
     uint32_t *ko, *vo;
     // 32 key bits = 4 passes: the values (iota in pass 0) go b, a, b, a and end in ids_a
+    // the rectangles travel through the passes when they pack into 32 bits (the passes end in
+    // rects_sorted, whose first half holds the packed ones of the passes in between), else the last
+    // pass gathers them
+    const bool carry = tiles_x(cam.image_width) <= kRect32MaxTiles && tiles_y(cam.image_height) <= kRect32MaxTiles;
     rc = launch_sort32(n, 32, keys_a, ids_a, keys_b, ids_b, true, false, base + o.sort, stream, &ko, &vo,
                        reinterpret_cast<const uint2*>(base + o.rects), reinterpret_cast<uint2*>(base + o.rects_sorted),
-                       true);
+                       true, carry ? reinterpret_cast<uint32_t*>(base + o.rects_sorted) : nullptr,
+                       carry ? reinterpret_cast<uint32_t*>(base + o.rects32) : nullptr);
     if(rc)
         return finish(rc);
     if(vo != ids_a)
