@@ -202,6 +202,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                                                              const float4* __restrict__ splats,
                                                              float* __restrict__ image, float* __restrict__ final_T,
                                                              int32_t* __restrict__ final_idx, int W, int H, int ntx,
+                                                             uint32_t last_id,
                                                              const uint32_t* __restrict__ sort_flag_a,
                                                              const uint32_t* __restrict__ sort_flag_b,
                                                              float4* __restrict__ prep, int64_t prep_count,
@@ -285,7 +286,9 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             const int e = b + slot;
             bool useful = false;
             bool member = false;
-            const int g = g_ahead[h];
+            // (an id is taken for what it is only up to the last Gaussian: lists that a failed sort or a
+            // caller's mix-up left in disorder then give a wrong image, not a fetch outside the records)
+            const int g = (int)min((uint32_t)g_ahead[h], last_id);
             g_ahead[h] = e + kFwdBatch < end ? ids[e + kFwdBatch] : 0;
             if(e < end)
             {
@@ -459,6 +462,8 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
         L.nbx = lg.nbx;
         L.nty = nty;
     }
+    // the largest id that the kernel takes from the lists (all of them when the caller did not say how many Gaussians there are)
+    const uint32_t last_id = num_gaussians > 0 ? (uint32_t)(num_gaussians - 1) : 0xffffffffu;
     {
         DSX_TIMED("blend_fwd_kernel", stream);
         const bool four = blend_pixels_per_lane(ntx * nty, kFwdFourPixelsFrom) == 4;
@@ -466,7 +471,7 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
         const float4* sp = reinterpret_cast<const float4*>(splats);
 #define DSX_LAUNCH_FWD(PIX, BINNED)                                                                              \
     hipLaunchKernelGGL((blend_fwd_kernel<PIX, BINNED>), grid, dim3(DSX_WAVE), 0, stream, ranges, sorted_ids, sp,   \
-                       image, final_T, final_idx, cam.image_width, cam.image_height, ntx, sort_flag_a,            \
+                       image, final_T, final_idx, cam.image_width, cam.image_height, ntx, last_id, sort_flag_a,   \
                        sort_flag_b, prep, prep_count, prep_marks, L)
         if(four && lists)
             DSX_LAUNCH_FWD(4, true);
@@ -569,8 +574,8 @@ template <int kBwdPix, bool kBinned>
 __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const int32_t* __restrict__ ranges, const int32_t* __restrict__ ids, const float4* __restrict__ splats,
     const float* __restrict__ final_T, const int32_t* __restrict__ final_idx, const float* __restrict__ v_image,
-    const float* __restrict__ bg, float* grads, uint8_t* marks, int W, int H, int ntx, const BinLists lists,
-    const ZeroJobs zeros)
+    const float* __restrict__ bg, float* grads, uint8_t* marks, int W, int H, int ntx, uint32_t last_id,
+    const BinLists lists, const ZeroJobs zeros)
 {
     __shared__ float4 s_a[kBwdBatch]; // pixel x, pixel y, conic a, conic b
     __shared__ float4 s_b[kBwdBatch]; // conic c, opacity, red, green
@@ -663,7 +668,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             const int e = top - slot;
             bool useful = false;
             bool member = false;
-            const int g = g_ahead[h];
+            const int g = (int)min((uint32_t)g_ahead[h], last_id); // (as in the forward)
             g_ahead[h] = e - kBwdBatch >= start ? ids[e - kBwdBatch] : 0;
             if(e >= start)
             {
@@ -814,6 +819,7 @@ int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, co
         L.nbx = lg.nbx;
         L.nty = nty;
     }
+    const uint32_t last_id = (uint32_t)(n - 1);
     {
         DSX_TIMED("blend_bwd_kernel", stream);
         const bool four = blend_pixels_per_lane(ntx * nty, kBwdFourPixelsFrom) == 4;
@@ -822,7 +828,7 @@ int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, co
 #define DSX_LAUNCH_BWD(PIX, BINNED)                                                                              \
     hipLaunchKernelGGL((blend_bwd_kernel<PIX, BINNED>), grid, dim3(DSX_WAVE), 0, stream, ranges, sorted_ids, sp,   \
                        final_T, final_idx, v_image, cam.bg, grads, with_marks ? grad_marks(grads, n) : nullptr,       \
-                       cam.image_width, cam.image_height, ntx, L, Z)
+                       cam.image_width, cam.image_height, ntx, last_id, L, Z)
         if(four && lists)
             DSX_LAUNCH_BWD(4, true);
         else if(four)

@@ -258,6 +258,9 @@ int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
  * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H).  If one of the two
  * sorts gave up a bounded wait (see dsx_sort_flags) the image is written as NaN: a failure
  * shows without a read-back of the flags.
+ * The blend kernels of dsx_forward_finish and dsx_backward take an id from the lists only up to
+ * n - 1 (larger or negative ones read as n - 1): lists in disorder give a wrong image or gradient,
+ * not a fetch outside the splat records.  (dsx_blend_fwd is not told n and trusts its lists.)
  * grads_to_prepare (may be NULL; 16-byte aligned, dsx_grads_bytes(n) bytes): the accumulator that
  * a dsx_backward of this forward will use.  The blend kernel, which leaves the memory system idle,
  * prepares it on the side (the nine sums zeroed, each Gaussian's conic in the three spare places,

@@ -240,6 +240,26 @@ def test_forward_prepares_the_accumulator_for_one_backward(blend_form, pixels_pe
             assert bool((o[k][unmarked] == 0).all()), k
 
 
+def test_backward_takes_ids_only_up_to_the_last_gaussian():
+    """The blend kernels gather splat records at the ids they find in the lists.  Lists in disorder
+    (a sort that gave up its bounded wait, a caller that handed the backward another forward's ids)
+    must give wrong numbers, not a fetch outside the records: every id is clamped to n - 1.  Here a
+    backward runs on lists in which every fifth id has been replaced by a value far outside."""
+    from ds_splat_amd import stages
+    n = 20000
+    sc = make_scene("cfg1", n=n, width=320, height=200, sh_degree=3)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    cam = stages.camera_from_scene(sc, DEV)
+    args = (t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
+    _, st = stages.forward(cam, *args)
+    bad = torch.tensor([0x7fffffff, -1, n, 1 << 30, -(1 << 31)], dtype=torch.int32, device=DEV)
+    st.sorted_ids[::5] = bad[torch.arange(st.sorted_ids[::5].numel(), device=DEV) % 5]
+    o = stages.backward(cam, st, 16, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["v_image"])
+    torch.cuda.synchronize()
+    # the replaced entries all read as Gaussian n - 1: it is marked, and nothing outside the arrays was touched
+    assert int(o["marks"][n - 1]) == 1 and bool(torch.isfinite(o["v_opacity"]).all())
+
+
 def test_backward_twice_through_the_api_gives_the_same_gradients():
     """retain_graph: the second backward finds the accumulator used and clears it for itself."""
     from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
