@@ -63,7 +63,7 @@ def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters, marked, carr
     if kernel == "hist32_kernel":
         return "hbm", 4 * n, "B"
     if kernel == "onesweep32_kernel<sort>":
-        # depth sort of the Gaussians: key + id, in and out; images of at most 127 x 127 tiles also carry each
+        # depth sort of the Gaussians: key + id, in and out; images of at most 255 x 255 tiles also carry each
         # Gaussian's packed tile rectangle through the passes (4 bytes in and out) instead of gathering them
         return "hbm", (24 if carries_rects else 16) * n, "B"
     if kernel == "ordered_block_sums_kernel":
@@ -295,7 +295,7 @@ def main():
         launches_per_step = cnt / args.steps
         avg = tot / cnt
         bound, work, unit = algorithmic_work(name, n, k, W * H, lists, coeffs, counters, marked,
-                                             (W + 15) // 16 <= 127 and (H + 15) // 16 <= 127)
+                                             (W + 15) // 16 <= 255 and (H + 15) // 16 <= 255)
         table.append((tot / args.steps, name, avg, launches_per_step, bound, work, unit))
     table.sort(reverse=True)
     measured, traffic_source = measured_traffic(spec.name, k) if args.n is None else ({}, None)

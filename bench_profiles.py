@@ -152,7 +152,7 @@ def algorithmic_bytes(bench):
               "ordered_block_sums_kernel", "emit_ordered_kernel", "onesweep32_kernel<tile partition>"):
         bound, work, _ = bench_module.algorithmic_work(k, n, cfg["num_keys"], w * h, cfg["lists"], (deg + 1) ** 2, None,
                                                        cfg.get("gaussians_with_gradient", 0),
-                                                       (w + 15) // 16 <= 127 and (h + 15) // 16 <= 127)
+                                                       (w + 15) // 16 <= 255 and (h + 15) // 16 <= 255)
         if bound == "hbm":
             out[k] = work
     return out, n

@@ -229,18 +229,22 @@ constexpr int kLookBatch32 = DSX_LOOK32;
 static_assert(kDepthSortThreads >= kBins32 && kListSortThreads >= kBins32, "one thread per digit");
 static_assert(kDepthSortTile <= 65535 && kListSortTile <= 65535, "u16 ranks");
 
-// A tile rectangle as the projection packs it (16-bit fields) in 29 bits: 7 bits each for first
-// column, first row, width and height, then the depth's sign.  For images of at most 127 x 127 tiles.
-constexpr int kRect32MaxTiles = 127;
+// A tile rectangle as the projection packs it (16-bit fields) in 32 bits: 8 bits each for first
+// column, first row, width and height, for images of at most 255 x 255 tiles.  The depth's sign
+// takes the first column's place: column 255 does not exist, and what reads the sorted rectangles
+// wants only the pair count of a Gaussian behind the camera (all its pairs go to slot 0), so its
+// first column and row are not carried.
+constexpr int kRect32MaxTiles = 255;
 __device__ __forceinline__ uint32_t rect_to_32(uint2 r)
 {
-    return (r.x & 0x7fu) | (((r.x >> 16) & 0x7fu) << 7) | ((r.y & 0x7fu) << 14) | (((r.y >> 16) & 0x7fu) << 21) |
-           ((r.y >> 31) << 28);
+    const uint32_t size = ((r.y & 0xffu) << 16) | (((r.y >> 16) & 0xffu) << 24);
+    return (r.y >> 31) ? (0xffu | size) : ((r.x & 0xffu) | (((r.x >> 16) & 0xffu) << 8) | size);
 }
 __device__ __forceinline__ uint2 rect_from_32(uint32_t v)
 {
-    return make_uint2((v & 0x7fu) | (((v >> 7) & 0x7fu) << 16),
-                      ((v >> 14) & 0x7fu) | (((v >> 21) & 0x7fu) << 16) | ((v >> 28) << 31));
+    const bool behind = (v & 0xffu) == 0xffu;
+    const uint32_t size = ((v >> 16) & 0xffu) | ((v >> 24) << 16);
+    return behind ? make_uint2(0u, size | 0x80000000u) : make_uint2((v & 0xffu) | (((v >> 8) & 0xffu) << 16), size);
 }
 
 // What a pass does about the Gaussians' tile rectangles, which the emission wants in depth order.

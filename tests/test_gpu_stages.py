@@ -317,11 +317,12 @@ def test_tile_lists_with_a_few_screen_filling_gaussians(oracle, list_bin):
     test_tile_lists_bit_exact(oracle, list_bin, 30000, 1280, 720, 0.5, 40, giants=25)
 
 
-@pytest.mark.parametrize("W,H", [(2032, 2032), (2033, 2000), (2000, 2048)])
+@pytest.mark.parametrize("W,H", [(4080, 1000), (1000, 4080), (4081, 1000), (1000, 4096)])
 def test_tile_lists_at_the_limit_of_packed_rectangles(oracle, list_bin, W, H):
-    """Images of at most 127 x 127 tiles carry each Gaussian's tile rectangle through the depth sort
-    packed into 32 bits (7 bits a field); beyond, the last pass gathers them.  At the limit and just past
-    it in either direction, with Gaussians whose rectangle is the whole image (width and height 127)."""
+    """Images of at most 255 x 255 tiles carry each Gaussian's tile rectangle through the depth sort
+    packed into 32 bits (8 bits a field, column 255 standing for "behind the camera"); beyond, the last
+    pass gathers them.  At the limit and just past it in either direction, with Gaussians whose
+    rectangle spans the whole image (width or height 255) and Gaussians behind the camera."""
     test_tile_lists_bit_exact(oracle, list_bin, 3000, W, H, 4.0, 20, giants=6)
 
 
