@@ -142,6 +142,13 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
     const auto f32 = at::TensorOptions().dtype(at::kFloat).device(dev);
     TORCH_CHECK(v_image.is_contiguous() && v_image.scalar_type() == at::kFloat && v_image.numel() == height * width * 3,
                 "v_image must be a contiguous float32 [H, W, 3] tensor");
+    // The lists that `ranges` and `sorted_ids` describe are per tile or per bin of tiles, as the library
+    // chose (or was told) when the forward ran; the size of `ranges` says which.  A backward that read
+    // them the other way would walk off the end of sorted_ids.
+    TORCH_CHECK(ranges.is_contiguous() && ranges.scalar_type() == at::kInt &&
+                    ranges.numel() == dsx_ranges_count((int32_t)width, (int32_t)height),
+                "ranges does not have the layout of this image size and of the tile lists' current bin size "
+                "(dsx_set_list_bin must not change between a forward and its backward)");
     auto out = [&](int bit, std::initializer_list<int64_t> shape) {
         return (wanted >> bit) & 1 ? at::empty(shape, f32) : at::Tensor();
     };

@@ -654,6 +654,29 @@ def test_a_sort_that_gave_up_poisons_the_image():
     assert torch.isnan(image).all()
 
 
+def test_backward_refuses_lists_of_another_bin_size(list_bin):
+    """The bin size of the tile lists is process-wide state for tests; if it changes between a forward
+    and its backward, the saved lists no longer mean what the backward's kernels would take them for
+    (per-tile ranges run far past the end of per-bin ids).  The binding sees it from the size of
+    `ranges` and raises before anything is launched."""
+    from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
+    sc = make_scene("cfg1", n=20000, width=640, height=360, sh_degree=3)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    settings = GaussianRasterizationSettings(
+        image_height=sc["height"], image_width=sc["width"], tanfovx=sc["tanfovx"], tanfovy=sc["tanfovy"], bg=t["bg"],
+        scale_modifier=1.0, viewmatrix=t["viewmatrix"], projmatrix=t["projmatrix"], sh_degree=sc["sh_degree"],
+        max_sh_degree=3, campos=t["campos"], prefiltered=False, debug=False)
+    for before, after in ((4, 1), (1, 4), (4, 8)):
+        list_bin(before)
+        means = t["means_3d"].clone().requires_grad_(True)
+        image, _ = GaussianRasterizer(settings)(means, torch.zeros_like(means), t["shs"], None, t["opacities"],
+                                                t["scales"], t["rotations"], None)
+        list_bin(after)
+        with pytest.raises(RuntimeError, match="dsx_set_list_bin must not change"):
+            image.backward(t["v_image"])
+        torch.cuda.synchronize()
+
+
 def test_api_rejects_bad_inputs_with_the_reference_messages():
     """cpp/rasterizer_torch.cu:176-190 and :124-129: every check fires before anything is launched."""
     from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
