@@ -328,6 +328,9 @@ def backward(cam, st, num_bases, means3d, scales, quats, v_image):
     n = means3d.shape[0]
     dev = means3d.device
     o = _bwd_outputs(n, num_bases, dev)
+    if st.lists.numel() != int(lib.dsx_ranges_count(cam.width, cam.height)):
+        raise RuntimeError("the forward built its tile lists for another bin size (dsx_set_list_bin must not change "
+                           "between a forward and its backward)")
     # an accumulator that the forward prepared serves one backward; after that it holds sums
     prepared = getattr(st, "grads", None) is not None
     grads = st.grads if prepared else new_accumulator(n, dev)
