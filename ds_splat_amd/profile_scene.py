@@ -27,6 +27,7 @@ def _scene(args):
 
 
 def main(argv=None):
+    """Runs the harness; returns the image of the last iteration (callers that check what was timed)."""
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     src = ap.add_mutually_exclusive_group(required=True)
     src.add_argument("--scene", help="TorchScript scene dump (see ds_splat_amd.scene_io)")
@@ -56,6 +57,7 @@ def main(argv=None):
             _native.check(lib.dsx_forward_core(*[p(t) for t in tensors], n, p(view), p(proj), p(sc["campos"]), W, H,
                                                sc["tanfovx"], sc["tanfovy"], sc["scale_modifier"], 3, sc["sh_degree"],
                                                p(image), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)))
+            return image
         name = "rasterizer_core"
     else:
         settings = GaussianRasterizationSettings(
@@ -75,8 +77,10 @@ def main(argv=None):
                 for t in leaves.values():
                     t.grad = None
                 image.backward(v_image)
+            return image.detach()
         name = "rasterizer_forward_backward" if args.backward else "rasterizer_forward"
 
+    rendered = None
     with torch.cuda.device(dev):
         for i in range(args.iters):
             last = i == args.iters - 1
@@ -85,13 +89,14 @@ def main(argv=None):
                 _native.trace_read()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            step()
+            rendered = step()
             torch.cuda.synchronize()
             print("Timing step:%s took: %.3fms" % (name, (time.perf_counter() - t0) * 1e3))
             if args.kernels and last:
                 for kernel, ms in _native.trace_read():
                     print("    %-36s %.4f ms" % (kernel, ms))
                 _native.trace_enable(False)
+    return rendered      # the last iteration's image [H, W, 3] (None without an iteration)
 
 
 if __name__ == "__main__":

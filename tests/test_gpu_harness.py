@@ -5,11 +5,13 @@ and through the raw-pointer forward; the "Timing step" lines, the kernel names a
 result are checked."""
 import re
 
+import numpy as np
 import pytest
 import torch
 
 from ds_splat_amd.synthetic import make_scene
 from helpers import set_camera
+from oracle.binding import make_settings
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -89,3 +91,33 @@ def test_the_loaded_dump_renders_like_the_scene_it_was_made_from(dump):
                    d["projmatrix"], d["campos"], d["tanfovx"], d["tanfovy"], d["scale_modifier"], d["image_height"],
                    d["image_width"], d["sh_degree"])
     assert torch.equal(a, b) and torch.equal(ra, rb) and float(a.max()) > 0
+
+
+def _oracle_render_of_the_dump(oracle, path):
+    """The CPU oracle's forward on the tensors of the dump itself (read back from the file, so the
+    comparison covers the save / load round trip and the matrix conventions of the dump)."""
+    from ds_splat_amd import scene_io
+    d = scene_io.load_scene(path)
+    s = make_settings(d["image_height"], d["image_width"], d["tanfovx"], d["tanfovy"], np.zeros(3, np.float32),
+                      d["scale_modifier"], d["viewmatrix"].t().contiguous().numpy(),
+                      d["projmatrix"].t().contiguous().numpy(), d["sh_degree"], d["campos"].numpy())
+    img, radii, st = oracle.forward(s, d["means_3d"].numpy(), d["scales"].numpy(), d["rotations"].numpy(),
+                                    d["opacities"].numpy(), d["shs"].numpy())
+    S = oracle.state(s, st, d["means_3d"].shape[0])
+    oracle.free(st)
+    return img, S
+
+
+@pytest.mark.parametrize("mode", [[], ["--backward"], ["--core"]], ids=["api", "api_backward", "core"])
+def test_what_the_harness_renders_is_the_oracles_image(dump, oracle, capsys, mode):
+    """The image the harness's timed call produces (through the API, and through the raw-pointer forward)
+    against the CPU oracle's render of the dump (the reference's harness renders the dumped scene the same
+    way, tests/rasterizer_test.cpp:145-212): rtol 1e-4 / atol 1e-5 wherever no blend decision is borderline."""
+    from ds_splat_amd import profile_scene
+    path, sc = dump
+    got = profile_scene.main(["--scene", path, "--iters", "2", "--device", DEV] + mode)
+    capsys.readouterr()
+    img_o, S = _oracle_render_of_the_dump(oracle, path)
+    ok = S["margin"] > 1e-4
+    assert ok.mean() > 0.98 and float(img_o.max()) > 0.1
+    np.testing.assert_allclose(got.cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
