@@ -25,9 +25,10 @@ class SceneSpec:
     z_range: tuple          # ... x [z0, z1]
     scale_mu: float         # per-axis scale = exp(N(mu, sigma))
     scale_sigma: float
-    opacity_mu: float       # opacity = sigmoid(N(mu, 1))
+    opacity_mu: float       # opacity = sigmoid(N(mu, opacity_sigma))
     backward: bool
     seed: int
+    opacity_sigma: float = 1.0
 
 
 WORKLOADS = {
@@ -36,6 +37,12 @@ WORKLOADS = {
     "cfg2": SceneSpec("cfg2", 3_000_000, 1920, 1080, 3, 5.0, (2.0, 20.0), -3.5, 0.6, 0.0, True, 1236),
     "cfg3": SceneSpec("cfg3", 6_000_000, 3840, 2160, 3, 8.0, (1.0, 30.0), -4.0, 0.5, 0.0, False, 1237),
     "cfg4": SceneSpec("cfg4", 1_000_000, 1920, 1080, 3, 3.0, (2.0, 12.0), -1.5, 0.7, -1.0, True, 1238),
+    # The regime of a scene in training, which the five above do not reach (their opaque Gaussians
+    # saturate a pixel after a few percent of its tile's list, and almost no Gaussian behind the first
+    # layer receives a gradient): faint Gaussians, opacity about 0.02 to 0.08, so that no pixel's
+    # transmittance falls to 1e-4.  Every pixel walks its whole list (about 300 blended Gaussians per
+    # pixel) and every visible Gaussian receives a gradient.
+    "dense": SceneSpec("dense", 2_000_000, 1920, 1080, 3, 5.0, (2.0, 20.0), -3.5, 0.6, -3.3, True, 1239, 0.4),
 }
 
 
@@ -76,7 +83,7 @@ def make_scene(spec, n=None, width=None, height=None, sh_degree=None, seed=None)
     scales = torch.exp(torch.randn(n, 3, generator=g, dtype=torch.float32) * spec.scale_sigma + spec.scale_mu)
     quats = torch.randn(n, 4, generator=g, dtype=torch.float32)
     quats = (quats / quats.norm(dim=1, keepdim=True)).contiguous()
-    opacities = torch.sigmoid(torch.randn(n, 1, generator=g, dtype=torch.float32) + spec.opacity_mu)
+    opacities = torch.sigmoid(torch.randn(n, 1, generator=g, dtype=torch.float32) * spec.opacity_sigma + spec.opacity_mu)
     shs = torch.zeros(n, 16, 3, dtype=torch.float32)
     shs[:, 0, :] = torch.randn(n, 3, generator=g, dtype=torch.float32) * 0.5
     if sh_degree > 0:
