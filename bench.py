@@ -112,8 +112,7 @@ def main():
                     help="tiles per side of the bins the tile lists are built for (0: the library's choice)")
     ap.add_argument("--verbose", action="store_true", help="per-kernel table on stderr")
     ap.add_argument("--copy-probe", action="store_true",
-                    help="also run one 1 GiB device copy (a kernel of known traffic that scales HBM byte counters) and "
-                         "the streaming probe (read / write / copy rates that plain kernels reach here)")
+                    help="also run one 1 GiB device copy: a kernel of known traffic that scales the HBM byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding "
@@ -127,7 +126,7 @@ def main():
     from ds_splat_amd import _native
     from ds_splat_amd.synthetic import WORKLOADS, make_scene
 
-    _native.check(_native.load().dsx_set_list_bin(args.list_bin))
+    _native.set_default_list_bin(args.list_bin)
     spec = WORKLOADS[args.workload]
     dev = torch.device("cuda:0")
     sc = make_scene(spec, n=args.n)
@@ -157,38 +156,11 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    stream_ceiling = None
     if args.copy_probe:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
-        # what plain streaming kernels of this library's access shape reach on this device (1 GiB each):
-        # the probe library is measurement tooling, separate from libdsx.so
-        import ctypes as C
-        probe = C.CDLL(os.path.join(ROOT, "ds_splat_amd", "lib", "libdsx_probe.so"))
-        probe.dsxp_stream_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p,
-                                            C.POINTER(C.c_float)]
-        stream = torch.cuda.current_stream().cuda_stream
-        nbytes = src.numel() * 4
-        mixed_bytes = 28 * 16 * 3_000_000   # 10 + 18 arrays of 3 M 16-byte elements: the backward's volume
-        sizes = (nbytes, nbytes, nbytes, mixed_bytes, mixed_bytes // 2)
-        reps = 5
-        times = []
-        for mode in (0, 1, 2, 3, 4):
-            for rep in range(2 + reps):
-                ms = C.c_float(0.0)
-                rc = probe.dsxp_stream_probe(src.data_ptr(), dst.data_ptr(), sizes[mode], mode, stream, C.byref(ms))
-                if rc != 0:
-                    raise RuntimeError("dsxp_stream_probe failed with %d" % rc)
-                if rep >= 2:
-                    times.append(float(ms.value))
-        per_mode = [min(times[m * reps:(m + 1) * reps]) for m in range(5)]
-        stream_ceiling = {"unit": "GB/s", "bytes": nbytes,
-                          "read": round(nbytes / per_mode[0] / 1e6, 1), "write": round(nbytes / per_mode[1] / 1e6, 1),
-                          "copy": round(2 * nbytes / per_mode[2] / 1e6, 1),
-                          "mixed_10_reads_18_writes": round(mixed_bytes / per_mode[3] / 1e6, 1),
-                          "mixed_5_reads_9_writes": round(mixed_bytes // 2 / per_mode[4] / 1e6, 1)}
         del src, dst
 
     # timed region: K steps, nothing but the public API between the two synchronisations
@@ -355,8 +327,6 @@ def main():
         "roofline_hbm": roofline_hbm,
         "cpu_baseline": cpu_baseline,
     }
-    if stream_ceiling is not None:
-        out["stream_ceiling"] = stream_ceiling
     print(json.dumps(out))
 
 

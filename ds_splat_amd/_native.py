@@ -30,6 +30,7 @@ class Camera(C.Structure):
         ("proj", C.c_void_p),
         ("campos", C.c_void_p),
         ("bg", C.c_void_p),
+        ("list_bin", C.c_int32),
     ]
 
 
@@ -45,10 +46,10 @@ SIGNATURES = {
     "dsx_num_blocks": (_I64, [_I64]),
     "dsx_num_tiles": (_I32, [_I32, _I32]),
     "dsx_sort_passes": (_I32, [_I32]),
-    "dsx_workspace_bytes": (C.c_size_t, [_I64, _I64, _I32, _I32]),
+    "dsx_workspace_bytes": (C.c_size_t, [_I64, _I64, _I32, _I32, _I32]),
     "dsx_sort_workspace_bytes": (C.c_size_t, [_I64, _I32]),
     "dsx_sort_u32_workspace_bytes": (C.c_size_t, [_I64, _I32]),
-    "dsx_order_bytes": (C.c_size_t, [_I64, _I32, _I32]),
+    "dsx_order_bytes": (C.c_size_t, [_I64, _I32, _I32, _I32]),
     "dsx_project_fwd": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P] * 4 + [_P, C.c_size_t, _P]),
     "dsx_scan_u32": (C.c_int, [_I64, _P, _P, _P]),
     "dsx_emit_keys": (C.c_int, [_CAM, _I64, _I64, _P, _P, _P, _P, _P]),
@@ -57,15 +58,15 @@ SIGNATURES = {
     "dsx_sort_pairs_u32": (C.c_int, [_I64, _I32, _P, _P, _P, C.c_size_t, _P]),
     "dsx_depth_order": (C.c_int, [_CAM, _I64, _P, C.c_size_t, _P]),
     "dsx_order_view": (C.c_int, [_I64, _P, C.POINTER(_P), C.POINTER(_P)]),
-    "dsx_sort_flags": (C.c_int, [_I64, _I64, _I32, _I32, _P, _P, C.POINTER(_P), C.POINTER(_P)]),
+    "dsx_sort_flags": (C.c_int, [_I64, _I64, _I32, _I32, _I32, _P, _P, C.POINTER(_P), C.POINTER(_P)]),
     "dsx_tile_lists": (C.c_int, [_CAM, _I64, _I64, _P, _P, _P, _P, C.c_size_t, _P]),
-    "dsx_blend_fwd": (C.c_int, [_CAM] + [_P] * 6 + [_P]),
-    "dsx_blend_bwd": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P]),
+    "dsx_blend_fwd": (C.c_int, [_CAM, _I64, _I64] + [_P] * 6 + [_P]),
+    "dsx_blend_bwd": (C.c_int, [_CAM, _I64, _I64] + [_P] * 7 + [_P]),
     "dsx_gaussian_bwd": (C.c_int, [_CAM, _I64, _I32] + [_P] * 7 + [_P] * 8 + [_P]),
     "dsx_forward_project": (C.c_int, [_CAM, _I64] + [_P] * 7 + [_P] * 4 + [_P, C.c_size_t, _P, _P]),
     "dsx_forward_finish": (C.c_int, [_CAM, _I64, _I64] + [_P] * 7 + [_P, C.c_size_t, _P, _P]),
-    "dsx_backward": (C.c_int, [_CAM, _I64, _I32] + [_P] * 11 + [_P, _I32] + [_P] * 8 + [_P]),
-    "dsx_backward_static": (C.c_int, [_CAM, _I64, _I32] + [_P] * 11 + [_P] * 8 + [_P]),
+    "dsx_backward": (C.c_int, [_CAM, _I64, _I64, _I32] + [_P] * 11 + [_P, _I32] + [_P] * 8 + [_P]),
+    "dsx_backward_static": (C.c_int, [_CAM, _I64, _I64, _I32] + [_P] * 11 + [_P] * 8 + [_P]),
     "dsx_forward_core": (C.c_int, [_P] * 5 + [_I64] + [_P] * 3 + [_I32, _I32, C.c_float, C.c_float, C.c_float,
                                                                     _I32, _I32, _P, _P]),
 }
@@ -80,12 +81,29 @@ class TraceEntry(C.Structure):
 SIGNATURES["dsx_trace_enable"] = (C.c_int, [C.c_int])
 SIGNATURES["dsx_trace_read"] = (C.c_int, [C.POINTER(TraceEntry), C.c_int])
 SIGNATURES["dsx_set_blend_pixels_per_lane"] = (C.c_int, [C.c_int])
-SIGNATURES["dsx_list_bin"] = (_I32, [_I32, _I32])
-SIGNATURES["dsx_set_list_bin"] = (C.c_int, [C.c_int])
-SIGNATURES["dsx_ranges_count"] = (_I64, [_I32, _I32])
+SIGNATURES["dsx_list_bin"] = (_I32, [_I32, _I32, _I32])
+SIGNATURES["dsx_ranges_count"] = (_I64, [_I32, _I32, _I32])
 SIGNATURES["dsx_grads_bytes"] = (C.c_size_t, [_I64])
 
 _lib = None
+
+# Tiles per side of the bins that the tile lists are built for when a caller does not say: 0 leaves the
+# choice to the library (by image size).  A Python-side default for the callers in this package
+# (rasterizer, stages, benchmark); the native library keeps no such setting: every call is told.
+_default_list_bin = 0
+
+
+def default_list_bin():
+    return _default_list_bin
+
+
+def set_default_list_bin(tiles_per_side):
+    """0 (the library's choice by image size), 1, 2, 4 or 8.  Takes effect for forwards that start
+    afterwards; a backward always uses the bin size of its own forward."""
+    global _default_list_bin
+    if int(tiles_per_side) not in (0, 1, 2, 4, 8):
+        raise ValueError("list_bin must be 0, 1, 2, 4 or 8")
+    _default_list_bin = int(tiles_per_side)
 
 
 def load():

@@ -100,6 +100,8 @@ int check_camera(const dsx_camera* cam)
     // (cpp/rasterizer_torch.cu:124-129); degree 4 has no forward there, so 0..3 it is
     if(cam->sh_degree < 0 || cam->sh_degree > 3 || cam->max_sh_degree < cam->sh_degree || cam->max_sh_degree > 3)
         return DSX_ERR_BAD_ARG;
+    if(!valid_list_bin(cam->list_bin))
+        return DSX_ERR_BAD_ARG;
     return DSX_OK;
 }
 
@@ -113,7 +115,9 @@ extern "C" const char* dsx_error_string(int status)
         case DSX_ERR_BAD_ARG: return "dsx: bad argument (null pointer, negative size or unsupported SH degree)";
         case DSX_ERR_LAUNCH: return "dsx: kernel launch failed";
         case DSX_ERR_RUNTIME: return "dsx: HIP runtime call failed";
-        case DSX_ERR_TOO_LARGE: return "dsx: too many tile keys for 32-bit key indexing (K >= 2^30)";
+        case DSX_ERR_TOO_LARGE:
+            return "dsx: too many (tile, Gaussian) pairs for 32-bit indexing (2^30 pairs of the lists that are built, "
+                   "or 2^31 pairs of the per-tile lists that the ranges and final_idx index)";
         case DSX_ERR_WORKSPACE: return "dsx: workspace too small (see dsx_workspace_bytes)";
         case DSX_ERR_STATIC_LIMIT:
             return "dsx: more Gaussians than the built-in scratch of dsx_backward_static holds "
@@ -124,7 +128,7 @@ extern "C" const char* dsx_error_string(int status)
 
 extern "C" int dsx_version(void)
 {
-    return 200;
+    return 300;
 }
 
 extern "C" int64_t dsx_num_blocks(int64_t n)
@@ -142,20 +146,19 @@ extern "C" int32_t dsx_sort_passes(int32_t num_tiles)
     return sort_passes(num_tiles);
 }
 
-extern "C" size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height)
+extern "C" size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height, int32_t list_bin)
 {
     (void)n;
-    return lists_workspace(k < 0 ? 0 : k, list_grid(width, height).lists()).bytes;
+    if(!valid_list_bin(list_bin))
+        return 0;
+    return lists_workspace(k < 0 ? 0 : k, list_grid(width, height, list_bin).lists()).bytes;
 }
 
-extern "C" int32_t dsx_list_bin(int32_t width, int32_t height)
+extern "C" int32_t dsx_list_bin(int32_t width, int32_t height, int32_t list_bin)
 {
-    return 1 << list_grid(width, height).shift;
-}
-
-extern "C" int dsx_set_list_bin(int tiles_per_side)
-{
-    return set_list_bin(tiles_per_side);
+    if(!valid_list_bin(list_bin))
+        return 0;
+    return 1 << list_grid(width < 0 ? 0 : width, height < 0 ? 0 : height, list_bin).shift;
 }
 
 extern "C" size_t dsx_grads_bytes(int64_t n)
@@ -163,9 +166,11 @@ extern "C" size_t dsx_grads_bytes(int64_t n)
     return grads_bytes(n < 0 ? 0 : n);
 }
 
-extern "C" int64_t dsx_ranges_count(int32_t width, int32_t height)
+extern "C" int64_t dsx_ranges_count(int32_t width, int32_t height, int32_t list_bin)
 {
-    return ranges_layout(list_grid(width < 0 ? 0 : width, height < 0 ? 0 : height)).count;
+    if(!valid_list_bin(list_bin))
+        return 0;
+    return ranges_layout(list_grid(width < 0 ? 0 : width, height < 0 ? 0 : height, list_bin)).count;
 }
 
 extern "C" size_t dsx_sort_workspace_bytes(int64_t k, int32_t num_tiles)
@@ -173,9 +178,11 @@ extern "C" size_t dsx_sort_workspace_bytes(int64_t k, int32_t num_tiles)
     return sort_workspace(k < 0 ? 0 : k, num_tiles < 0 ? 0 : num_tiles).bytes;
 }
 
-extern "C" size_t dsx_order_bytes(int64_t n, int32_t width, int32_t height)
+extern "C" size_t dsx_order_bytes(int64_t n, int32_t width, int32_t height, int32_t list_bin)
 {
-    return order_layout(n < 0 ? 0 : n, width < 0 ? 0 : width, height < 0 ? 0 : height).bytes;
+    if(!valid_list_bin(list_bin))
+        return 0;
+    return order_layout(n < 0 ? 0 : n, width < 0 ? 0 : width, height < 0 ? 0 : height, list_bin).bytes;
 }
 
 namespace
@@ -221,7 +228,7 @@ static int project_fwd_checked(const dsx_camera* cam, int64_t n, const float* me
     uint2* rects = nullptr;
     if(order)
     {
-        const OrderLayout o = order_layout(n, cam->image_width, cam->image_height);
+        const OrderLayout o = order_layout(n, cam->image_width, cam->image_height, cam->list_bin);
         if(order_bytes < o.bytes)
             return DSX_ERR_WORKSPACE;
         depth_keys = reinterpret_cast<uint32_t*>(static_cast<char*>(order) + o.depth_keys);
@@ -351,7 +358,7 @@ extern "C" int dsx_depth_order(const dsx_camera* cam, int64_t n, void* order, si
         return DSX_OK;
     if(!order)
         return DSX_ERR_BAD_ARG;
-    if(order_bytes < order_layout(n, cam->image_width, cam->image_height).bytes)
+    if(order_bytes < order_layout(n, cam->image_width, cam->image_height, cam->list_bin).bytes)
         return DSX_ERR_WORKSPACE;
     return launch_depth_order(*cam, n, order, as_stream(stream));
 }
@@ -369,11 +376,11 @@ extern "C" int dsx_order_view(int64_t n, const void* order, const uint32_t** dep
     return DSX_OK;
 }
 
-extern "C" int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t height, const void* order,
-                              const void* workspace, const uint32_t** depth_sort_flag,
+extern "C" int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t height, int32_t list_bin,
+                              const void* order, const void* workspace, const uint32_t** depth_sort_flag,
                               const uint32_t** partition_flag)
 {
-    if(n < 0 || k < 0 || width <= 0 || height <= 0)
+    if(n < 0 || k < 0 || width <= 0 || height <= 0 || !valid_list_bin(list_bin))
         return DSX_ERR_BAD_ARG;
     if(depth_sort_flag)
     {
@@ -391,7 +398,7 @@ extern "C" int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t heigh
         *partition_flag = nullptr;
         if(workspace && k > 0)
         {
-            const int tiles = list_grid(width, height).lists();
+            const int tiles = list_grid(width, height, list_bin).lists();
             const ListsWorkspace lw = lists_workspace(k, tiles);
             const Sort32Workspace w = sort32_workspace(k, slot_bits(tiles), kListSortTile);
             *partition_flag =
@@ -414,36 +421,42 @@ extern "C" int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const
     {
         if(!order || !sorted_ids || !workspace)
             return DSX_ERR_BAD_ARG;
-        if(workspace_bytes < lists_workspace(k, list_grid(cam->image_width, cam->image_height).lists()).bytes)
+        if(workspace_bytes < lists_workspace(k, list_grid(*cam).lists()).bytes)
             return DSX_ERR_WORKSPACE;
     }
     return launch_tile_lists(*cam, n, k, order, sorted_ids, ranges, workspace, as_stream(stream));
 }
 
-extern "C" int dsx_blend_fwd(const dsx_camera* cam, const int32_t* ranges, const int32_t* sorted_ids,
-                             const float* splats, float* image, float* final_T, int32_t* final_idx, void* stream)
+extern "C" int dsx_blend_fwd(const dsx_camera* cam, int64_t n, int64_t k, int32_t* ranges,
+                             const int32_t* sorted_ids, const float* splats, float* image, float* final_T,
+                             int32_t* final_idx, void* stream)
 {
     if(int rc = check_camera(cam))
         return rc;
-    if(!ranges || !image || !final_T || !final_idx)
+    if(n < 0 || k < 0 || !ranges || !image || !final_T || !final_idx)
         return DSX_ERR_BAD_ARG;
-    return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream));
+    if(k >= (1ll << 31))
+        return DSX_ERR_TOO_LARGE;
+    return launch_blend_fwd(*cam, n, k, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream),
+                            false);
 }
 
-extern "C" int dsx_blend_bwd(const dsx_camera* cam, int64_t n, const int32_t* ranges, const int32_t* sorted_ids,
-                             const float* splats, const float* final_T, const int32_t* final_idx,
-                             const float* v_image, float* grads, void* stream)
+extern "C" int dsx_blend_bwd(const dsx_camera* cam, int64_t n, int64_t k, const int32_t* ranges,
+                             const int32_t* sorted_ids, const float* splats, const float* final_T,
+                             const int32_t* final_idx, const float* v_image, float* grads, void* stream)
 {
     if(int rc = check_camera(cam))
         return rc;
-    if(n < 0)
+    if(n < 0 || k < 0)
         return DSX_ERR_BAD_ARG;
+    if(k >= (1ll << 31))
+        return DSX_ERR_TOO_LARGE;
     if(n == 0)
         return DSX_OK;
     if(!ranges || !final_T || !final_idx || !v_image || !grads || !splats)
         return DSX_ERR_BAD_ARG;
-    return launch_blend_bwd(*cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
-                            as_stream(stream));
+    return launch_blend_bwd(*cam, n, k, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
+                            as_stream(stream), false);
 }
 
 // conic_in_grads: places 9..11 of every accumulator record hold the conic (dsx_forward_finish put it there)
@@ -481,6 +494,16 @@ extern "C" int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_ba
                                 v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat, v_cov3d, stream, false);
 }
 
+// The pair counts a forward can index: the lists that are built are sorted with 30-bit counters, and
+// the per-tile pairs (the reference's K) are what the fine ranges, final_idx and the walk records
+// index as int32.  With binned lists the first is a fraction of the second, so both are checked.
+static int check_pair_counts(int64_t list_pairs, int64_t tile_pairs)
+{
+    if(list_pairs < 0 || tile_pairs < 0 || list_pairs >= (1ll << 30) || tile_pairs >= (1ll << 31))
+        return DSX_ERR_TOO_LARGE;
+    return DSX_OK;
+}
+
 extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
                                    const float* quats, const float* opacities, const float* shs,
                                    const float* cov3d_precomp, const float* colors_precomp, float* splats,
@@ -489,15 +512,15 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
 {
     if(!num_keys || (n > 0 && !order))
         return DSX_ERR_BAD_ARG;
-    *num_keys = 0;
+    num_keys[0] = num_keys[1] = 0;
     hipStream_t s = as_stream(stream);
     int rc = project_fwd_checked(cam, n, means3d, scales, quats, opacities, shs, cov3d_precomp, colors_precomp,
                                  splats, radii, cov3d, block_sums, order, order_bytes, stream, true);
     if(rc || n == 0)
         return rc;
-    // K is the sum of the rectangles' tile counts: the corner-grid kernel, first thing beside the
-    // depth sort, adds them up, and K travels to the host while the depth order is computed.  The
-    // wait below is for that copy only (it overlaps when *num_keys is pinned host memory; with
+    // The pair counts are sums over the rectangles: the corner-grid kernel, first thing beside the
+    // depth sort, adds them up, and they travel to the host while the depth order is computed.  The
+    // wait below is for that copy only (it overlaps when num_keys is pinned host memory; with
     // pageable memory the copy is synchronous and nothing is lost).
     hipEvent_t copied;
     if(hipEventCreateWithFlags(&copied, hipEventDisableTiming) != hipSuccess)
@@ -510,7 +533,11 @@ extern "C" int dsx_forward_project(const dsx_camera* cam, int64_t n, const float
         return rc;
     if(!ok)
         return DSX_ERR_RUNTIME;
-    return *num_keys >= (1ll << 30) || *num_keys < 0 ? DSX_ERR_TOO_LARGE : DSX_OK;
+    // the device wrote (per-tile pairs, bin pairs); the caller gets (pairs of the lists, per-tile pairs)
+    const int64_t tile_pairs = num_keys[0], bin_pairs = num_keys[1];
+    num_keys[0] = list_grid(*cam).shift ? bin_pairs : tile_pairs;
+    num_keys[1] = tile_pairs;
+    return check_pair_counts(num_keys[0], num_keys[1]);
 }
 
 extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float* splats,
@@ -524,15 +551,16 @@ extern "C" int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, c
     if(rc)
         return rc;
     const uint32_t *depth_flag = nullptr, *partition_flag = nullptr;
-    rc = dsx_sort_flags(n, k, cam->image_width, cam->image_height, order, workspace, &depth_flag, &partition_flag);
+    rc = dsx_sort_flags(n, k, cam->image_width, cam->image_height, cam->list_bin, order, workspace, &depth_flag,
+                        &partition_flag);
     if(rc)
         return rc;
-    return launch_blend_fwd(*cam, ranges, sorted_ids, splats, image, final_T, final_idx, as_stream(stream), depth_flag,
-                            partition_flag, n > 0 ? grads_to_prepare : nullptr, n,
-                            list_grid(cam->image_width, cam->image_height).shift ? ranges : nullptr, true);
+    return launch_blend_fwd(*cam, n, n > 0 ? k : 0, ranges, sorted_ids, splats, image, final_T, final_idx,
+                            as_stream(stream), true, depth_flag, partition_flag, n > 0 ? grads_to_prepare : nullptr,
+                            true);
 }
 
-static int backward_impl(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+static int backward_impl(const dsx_camera* cam, int64_t n, int64_t k, int32_t num_bases, const float* means3d,
                          const float* scales, const float* quats, const float* splats, const float* cov3d,
                          const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
                          const float* final_T, const int32_t* final_idx, const float* v_image, float* grads,
@@ -541,20 +569,21 @@ static int backward_impl(const dsx_camera* cam, int64_t n, int32_t num_bases, co
 {
     if(int rc = check_camera(cam))
         return rc;
-    if(n < 0 || num_bases < 0 || num_bases > 16)
+    if(n < 0 || k < 0 || num_bases < 0 || num_bases > 16)
         return DSX_ERR_BAD_ARG;
+    if(k >= (1ll << 30))
+        return DSX_ERR_TOO_LARGE;
     if(n == 0)
         return DSX_OK;
-    if(!ranges || !final_T || !final_idx || !v_image || !grads || !splats)
+    if(!ranges || !final_T || !final_idx || !v_image || !grads || !splats || (k > 0 && !sorted_ids))
         return DSX_ERR_BAD_ARG;
     // The per-Gaussian kernel writes only the Gaussians that received a gradient term; everything
     // else in its outputs is zero: 260 bytes per Gaussian of plain stores, which the wavefronts of the
     // blend kernel (bound by its arithmetic, the memory system idle) issue on their way out.
     const ZeroJobs zeros = make_zero_jobs(n, num_bases, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale,
                                           v_quat, v_cov3d);
-    int rc = launch_blend_bwd(*cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
-                              as_stream(stream), grads_prepared != 0,
-                              list_grid(cam->image_width, cam->image_height).shift ? ranges : nullptr, true, &zeros);
+    int rc = launch_blend_bwd(*cam, n, k, ranges, sorted_ids, splats, final_T, final_idx, v_image, grads,
+                              as_stream(stream), true, grads_prepared != 0, true, &zeros);
     if(rc)
         return rc;
     return gaussian_bwd_checked(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, grads, v_mean3d,
@@ -562,16 +591,16 @@ static int backward_impl(const dsx_camera* cam, int64_t n, int32_t num_bases, co
                                 grads_prepared != 0, true, true);
 }
 
-extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+extern "C" int dsx_backward(const dsx_camera* cam, int64_t n, int64_t k, int32_t num_bases, const float* means3d,
                             const float* scales, const float* quats, const float* splats, const float* cov3d,
                             const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
                             const float* final_T, const int32_t* final_idx, const float* v_image, float* grads,
                             int32_t grads_prepared, float* v_mean3d, float* v_means2d, float* v_shs, float* v_colors,
                             float* v_opacity, float* v_scale, float* v_quat, float* v_cov3d, void* stream)
 {
-    return backward_impl(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, ranges, sorted_ids, final_T,
-                         final_idx, v_image, grads, grads_prepared, v_mean3d, v_means2d, v_shs, v_colors, v_opacity,
-                         v_scale, v_quat, v_cov3d, stream);
+    return backward_impl(cam, n, k, num_bases, means3d, scales, quats, splats, cov3d, radii, ranges, sorted_ids,
+                         final_T, final_idx, v_image, grads, grads_prepared, v_mean3d, v_means2d, v_shs, v_colors,
+                         v_opacity, v_scale, v_quat, v_cov3d, stream);
 }
 
 extern "C" int dsx_forward_core(const float* means3d, const float* shs, const float* opacities, const float* scales,
@@ -593,6 +622,7 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     cam.proj = proj;
     cam.campos = campos;
     cam.bg = campos; // unused by the forward
+    cam.list_bin = 0;
     if(int rc = check_camera(&cam))
         return rc;
     if(n < 0 || !image)
@@ -606,23 +636,24 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     o_cov3d = align(o_radii + (size_t)n * 4);
     o_bs = align(o_cov3d + (size_t)n * 24);
     o_ranges = align(o_bs + (size_t)nb * 4);
-    o_T = align(o_ranges + (size_t)dsx_ranges_count(image_width, image_height) * 4);
+    o_T = align(o_ranges + (size_t)dsx_ranges_count(image_width, image_height, 0) * 4);
     o_idx = align(o_T + (size_t)P * 4);
     o_order = align(o_idx + (size_t)P * 4);
-    const size_t order_bytes = order_layout(n, image_width, image_height).bytes;
+    const size_t order_bytes = order_layout(n, image_width, image_height, 0).bytes;
     stage1 = align(o_order + order_bytes);
     char* buf = nullptr;
     if(hipMallocAsync(reinterpret_cast<void**>(&buf), stage1 + 256, s) != hipSuccess)
         return DSX_ERR_RUNTIME;
-    int64_t k = 0;
+    int64_t counts[2] = {0, 0};
     int rc = dsx_forward_project(&cam, n, means3d, scales, quats, opacities, shs, nullptr, nullptr,
                                  reinterpret_cast<float*>(buf + o_splats), reinterpret_cast<int32_t*>(buf + o_radii),
                                  reinterpret_cast<float*>(buf + o_cov3d), reinterpret_cast<uint32_t*>(buf + o_bs),
-                                 buf + o_order, order_bytes, &k, stream);
+                                 buf + o_order, order_bytes, counts, stream);
+    const int64_t k = counts[0];
     char* buf2 = nullptr;
     if(rc == DSX_OK)
     {
-        const size_t ws = lists_workspace(k, list_grid(image_width, image_height).lists()).bytes;
+        const size_t ws = lists_workspace(k, list_grid(cam).lists()).bytes;
         const size_t o_ids = align(ws);
         if(hipMallocAsync(reinterpret_cast<void**>(&buf2), o_ids + (size_t)k * 4 + 256, s) != hipSuccess)
             rc = DSX_ERR_RUNTIME;
@@ -672,7 +703,8 @@ float* static_scratch()
 }
 } // namespace
 
-extern "C" int dsx_backward_static(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+extern "C" int dsx_backward_static(const dsx_camera* cam, int64_t n, int64_t k, int32_t num_bases,
+                                   const float* means3d,
                                    const float* scales, const float* quats, const float* splats,
                                    const float* cov3d, const int32_t* radii, const int32_t* ranges,
                                    const int32_t* sorted_ids, const float* final_T, const int32_t* final_idx,
@@ -688,9 +720,9 @@ extern "C" int dsx_backward_static(const dsx_camera* cam, int64_t n, int32_t num
         return DSX_ERR_RUNTIME;
     // grads_prepared = 0: the array keeps the last call's sums, so this call clears its n records
     // itself (a fill kernel with plain stores, which a caller may capture in a graph)
-    return backward_impl(cam, n, num_bases, means3d, scales, quats, splats, cov3d, radii, ranges, sorted_ids, final_T,
-                         final_idx, v_image, grads, 0, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale, v_quat,
-                         v_cov3d, stream);
+    return backward_impl(cam, n, k, num_bases, means3d, scales, quats, splats, cov3d, radii, ranges, sorted_ids,
+                         final_T, final_idx, v_image, grads, 0, v_mean3d, v_means2d, v_shs, v_colors, v_opacity, v_scale,
+                         v_quat, v_cov3d, stream);
 }
 
 extern "C" int dsx_set_blend_pixels_per_lane(int pixels)

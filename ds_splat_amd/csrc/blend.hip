@@ -202,7 +202,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                                                              const float4* __restrict__ splats,
                                                              float* __restrict__ image, float* __restrict__ final_T,
                                                              int32_t* __restrict__ final_idx, int W, int H, int ntx,
-                                                             uint32_t last_id,
+                                                             uint32_t last_id, int k,
+                                                             const int32_t* __restrict__ header, int header_shift,
                                                              const uint32_t* __restrict__ sort_flag_a,
                                                              const uint32_t* __restrict__ sort_flag_b,
                                                              float4* __restrict__ prep, int64_t prep_count,
@@ -225,19 +226,27 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     const float box_x0 = (float)(tx * kTile) + 0.5f, box_y0 = (float)(ty * kTile + 4 * band) + 0.5f;
     const float span_y = kFwdPix == 4 ? 15.0f : 3.0f;
 
-    int start, end;
-    TileSource src;
+    // The lists are data from the device: positions are taken for what they are only inside
+    // sorted_ids[0, k), and a `ranges` buffer that was built for another bin size (its header word,
+    // which every layout has in the same place, says which) is not read any further; the image is
+    // then NaN, like after a sort that gave up.
+    const bool layout_ok = header == nullptr || *header == header_shift;
+    int start = 0, end = 0;
+    TileSource src = {};
     if(kBinned)
     {
-        src = tile_source(lists, tile, ntx);
+        if(layout_ok)
+            src = tile_source(lists, tile, ntx);
         start = src.start;
         end = src.end;
     }
-    else
+    else if(layout_ok)
     {
         start = ranges[tile];
         end = ranges[tile + 1];
     }
+    start = min(max(start, 0), k);
+    end = min(max(end, 0), k);
     int seen = 0;     // entries of the tile's own list met so far (binned lists)
     int pos_hi = -1;  // position of the last entry that any pixel blended (binned lists)
 
@@ -364,7 +373,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
 
     // A sort pass that gave up waiting on its predecessor (bounded wait, never seen to happen)
     // leaves its flag set and the tile lists wrong: make that loud instead of plausible.
-    if((sort_flag_a && *sort_flag_a) || (sort_flag_b && *sort_flag_b))
+    if(!layout_ok || (sort_flag_a && *sort_flag_a) || (sort_flag_b && *sort_flag_b))
     {
 #pragma unroll
         for(int p = 0; p < kFwdPix; ++p)
@@ -384,7 +393,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             final_idx[pix] = last[p];
         }
     }
-    if(kBinned)
+    if(kBinned && layout_ok)
     {
         // for the backward: where this wavefront's walk ended, as a position in the bin's list and
         // as an index in the sorted key array (-1, -1 if it blended nothing).  The four-pixel form
@@ -432,38 +441,49 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     }
 }
 
-// lists: null when ranges / sorted_ids are the per-tile lists (the stage entry point), else the
-// `ranges` buffer of binned lists in ranges_layout() (the kernel also writes its `walk` part)
-int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids, const float* splats,
-                     float* image, float* final_T, int32_t* final_idx, hipStream_t stream,
-                     const uint32_t* sort_flag_a, const uint32_t* sort_flag_b, float* prepare_grads,
-                     int64_t num_gaussians, int32_t* lists, bool prepare_marks)
+// The BinLists view of a `ranges` buffer in ranges_layout(lg) (lists per bin: lg.shift > 0)
+static BinLists bin_lists(const ListGrid& lg, int32_t* ranges)
 {
-    const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
+    BinLists L = {};
+    if(lg.shift)
+    {
+        const RangesLayout rl = ranges_layout(lg);
+        L.fine = ranges + rl.fine;
+        L.last_tile = ranges + rl.last_tile;
+        L.bins = ranges + rl.bins;
+        L.walk = ranges + rl.walk;
+        L.shift = lg.shift;
+        L.nbx = lg.nbx;
+        L.nty = lg.nty;
+    }
+    return L;
+}
+
+// ranges: the `ranges` buffer in ranges_layout(list_grid(cam)) (the kernel also writes its `walk` part
+// when the lists are per bin).  check_header: the buffer has its header word, which must name the
+// bin size of this call (always so for binned lists; per-tile lists may come as the tiles + 1 words
+// of launch_tile_ranges, which have none).  n, k: Gaussians and entries of sorted_ids; ids and list
+// positions beyond them are not followed.
+int launch_blend_fwd(const dsx_camera& cam, int64_t n, int64_t k, int32_t* ranges, const int32_t* sorted_ids,
+                     const float* splats, float* image, float* final_T, int32_t* final_idx, hipStream_t stream,
+                     bool check_header, const uint32_t* sort_flag_a, const uint32_t* sort_flag_b,
+                     float* prepare_grads, bool prepare_marks)
+{
+    const ListGrid lg = list_grid(cam);
+    const int ntx = lg.ntx, nty = lg.nty;
     if(ntx * nty == 0)
         return prepare_grads ? DSX_ERR_BAD_ARG : DSX_OK; // (no image, no kernel, nothing prepared)
     if(prepare_grads && (((uintptr_t)prepare_grads & 15) != 0 || splats == nullptr))
         return DSX_ERR_BAD_ARG;
+    if(n < 0 || k < 0 || k > 0x7fffffffll || (k > 0 && (sorted_ids == nullptr || splats == nullptr || n == 0)))
+        return DSX_ERR_BAD_ARG;
     float4* prep = reinterpret_cast<float4*>(prepare_grads);
-    const int64_t prep_count = prepare_grads ? num_gaussians : 0;
-    uint8_t* prep_marks = prepare_grads && prepare_marks ? grad_marks(prepare_grads, num_gaussians) : nullptr;
-    BinLists L = {};
-    if(lists)
-    {
-        const ListGrid lg = list_grid(cam.image_width, cam.image_height);
-        if(lg.shift == 0)
-            return DSX_ERR_BAD_ARG;
-        const RangesLayout rl = ranges_layout(lg);
-        L.fine = lists + rl.fine;
-        L.last_tile = lists + rl.last_tile;
-        L.bins = lists + rl.bins;
-        L.walk = lists + rl.walk;
-        L.shift = lg.shift;
-        L.nbx = lg.nbx;
-        L.nty = nty;
-    }
-    // the largest id that the kernel takes from the lists (all of them when the caller did not say how many Gaussians there are)
-    const uint32_t last_id = num_gaussians > 0 ? (uint32_t)(num_gaussians - 1) : 0xffffffffu;
+    const int64_t prep_count = prepare_grads ? n : 0;
+    uint8_t* prep_marks = prepare_grads && prepare_marks ? grad_marks(prepare_grads, n) : nullptr;
+    const BinLists L = bin_lists(lg, ranges);
+    const int32_t* header = (lg.shift || check_header) ? ranges + ranges_layout(lg).header : nullptr;
+    // the largest id that the kernel takes from the lists
+    const uint32_t last_id = n > 0 ? (uint32_t)(n - 1) : 0u;
     {
         DSX_TIMED("blend_fwd_kernel", stream);
         const bool four = blend_pixels_per_lane(ntx * nty, kFwdFourPixelsFrom) == 4;
@@ -471,13 +491,13 @@ int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t
         const float4* sp = reinterpret_cast<const float4*>(splats);
 #define DSX_LAUNCH_FWD(PIX, BINNED)                                                                              \
     hipLaunchKernelGGL((blend_fwd_kernel<PIX, BINNED>), grid, dim3(DSX_WAVE), 0, stream, ranges, sorted_ids, sp,   \
-                       image, final_T, final_idx, cam.image_width, cam.image_height, ntx, last_id, sort_flag_a,   \
-                       sort_flag_b, prep, prep_count, prep_marks, L)
-        if(four && lists)
+                       image, final_T, final_idx, cam.image_width, cam.image_height, ntx, last_id, (int)k, header,  \
+                       lg.shift, sort_flag_a, sort_flag_b, prep, prep_count, prep_marks, L)
+        if(four && lg.shift)
             DSX_LAUNCH_FWD(4, true);
         else if(four)
             DSX_LAUNCH_FWD(4, false);
-        else if(lists)
+        else if(lg.shift)
             DSX_LAUNCH_FWD(1, true);
         else
             DSX_LAUNCH_FWD(1, false);
@@ -574,8 +594,8 @@ template <int kBwdPix, bool kBinned>
 __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const int32_t* __restrict__ ranges, const int32_t* __restrict__ ids, const float4* __restrict__ splats,
     const float* __restrict__ final_T, const int32_t* __restrict__ final_idx, const float* __restrict__ v_image,
-    const float* __restrict__ bg, float* grads, uint8_t* marks, int W, int H, int ntx, uint32_t last_id,
-    const BinLists lists, const ZeroJobs zeros)
+    const float* __restrict__ bg, float* grads, uint8_t* marks, int W, int H, int ntx, uint32_t last_id, int k,
+    const int32_t* __restrict__ header, int header_shift, const BinLists lists, const ZeroJobs zeros)
 {
     __shared__ float4 s_a[kBwdBatch]; // pixel x, pixel y, conic a, conic b
     __shared__ float4 s_b[kBwdBatch]; // conic c, opacity, red, green
@@ -618,11 +638,13 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
         m = max(m, bin_final[p]);
     }
 
-    int start, hi;
-    TileSource src;
+    // lists that were built for another bin size than this launch assumes are not read (see the forward)
+    const bool layout_ok = header == nullptr || *header == header_shift;
+    int start = 0, hi = -1;
+    TileSource src = {};
     int index_hi = 0; // index (in the sorted key array) of the entry at position hi (binned lists)
     int above = 0;    // entries of the tile's own list met so far, from the top (binned lists)
-    if(kBinned)
+    if(kBinned && layout_ok)
     {
         // the forward's walk of this tile ended at position hi of the bin's list, on the entry
         // with index index_hi (the larger of the four bands' figures: both grow together)
@@ -633,11 +655,13 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
         index_hi = max(max(w[1], w[3]), max(w[5], w[7]));
         if(src.count <= 0)
             hi = -1;
+        hi = min(hi, k - 1); // (positions outside sorted_ids are not followed, as in the forward)
+        start = max(start, 0);
     }
-    else
+    else if(layout_ok)
     {
-        start = ranges[tile];
-        const int end = ranges[tile + 1];
+        start = max(ranges[tile], 0);
+        const int end = min(ranges[tile + 1], k);
         // last entry any pixel of this tile blended
 #pragma unroll
         for(int o = 32; o > 0; o >>= 1)
@@ -787,38 +811,28 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
         zero_share(zeros, blockIdx.x, gridDim.x, lane, DSX_WAVE);
 }
 
-// lists: as for launch_blend_fwd (null: ranges / sorted_ids are per-tile lists)
-int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, const int32_t* sorted_ids,
+// ranges, check_header, n, k: as for launch_blend_fwd (the kernel reads the `walk` part that the forward wrote)
+int launch_blend_bwd(const dsx_camera& cam, int64_t n, int64_t k, const int32_t* ranges, const int32_t* sorted_ids,
                      const float* splats, const float* final_T, const int32_t* final_idx, const float* v_image,
-                     float* grads, hipStream_t stream, bool grads_prepared, const int32_t* lists, bool with_marks,
+                     float* grads, hipStream_t stream, bool check_header, bool grads_prepared, bool with_marks,
                      const ZeroJobs* zeros)
 {
+    if(k < 0 || k > 0x7fffffffll || (k > 0 && sorted_ids == nullptr))
+        return DSX_ERR_BAD_ARG;
     // (the marks lie right behind the records, padded to whole words: one fill covers both)
     if(!grads_prepared)
         if(int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(grads),
                                     with_marks ? (int64_t)(grads_bytes(n) / 4) : n * DSX_GRAD_FLOATS, 0u, stream))
             return rc;
-    const int ntx = tiles_x(cam.image_width), nty = tiles_y(cam.image_height);
+    const ListGrid lg = list_grid(cam);
+    const int ntx = lg.ntx, nty = lg.nty;
     if(ntx * nty == 0 || n == 0)
         return zeros ? launch_zero_outputs(*zeros, stream) : DSX_OK; // (no tile, no wavefront to store them)
     ZeroJobs Z = {};
     if(zeros)
         Z = *zeros;
-    BinLists L = {};
-    if(lists)
-    {
-        const ListGrid lg = list_grid(cam.image_width, cam.image_height);
-        if(lg.shift == 0)
-            return DSX_ERR_BAD_ARG;
-        const RangesLayout rl = ranges_layout(lg);
-        L.fine = lists + rl.fine;
-        L.last_tile = lists + rl.last_tile;
-        L.bins = lists + rl.bins;
-        L.walk = const_cast<int32_t*>(lists) + rl.walk;
-        L.shift = lg.shift;
-        L.nbx = lg.nbx;
-        L.nty = nty;
-    }
+    const BinLists L = bin_lists(lg, const_cast<int32_t*>(ranges));
+    const int32_t* header = (lg.shift || check_header) ? ranges + ranges_layout(lg).header : nullptr;
     const uint32_t last_id = (uint32_t)(n - 1);
     {
         DSX_TIMED("blend_bwd_kernel", stream);
@@ -828,12 +842,12 @@ int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges, co
 #define DSX_LAUNCH_BWD(PIX, BINNED)                                                                              \
     hipLaunchKernelGGL((blend_bwd_kernel<PIX, BINNED>), grid, dim3(DSX_WAVE), 0, stream, ranges, sorted_ids, sp,   \
                        final_T, final_idx, v_image, cam.bg, grads, with_marks ? grad_marks(grads, n) : nullptr,       \
-                       cam.image_width, cam.image_height, ntx, last_id, L, Z)
-        if(four && lists)
+                       cam.image_width, cam.image_height, ntx, last_id, (int)k, header, lg.shift, L, Z)
+        if(four && lg.shift)
             DSX_LAUNCH_BWD(4, true);
         else if(four)
             DSX_LAUNCH_BWD(4, false);
-        else if(lists)
+        else if(lg.shift)
             DSX_LAUNCH_BWD(1, true);
         else
             DSX_LAUNCH_BWD(1, false);

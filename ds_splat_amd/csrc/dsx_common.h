@@ -185,14 +185,24 @@ struct ListGrid
     // what the partition sorts by: bins when the lists are binned, tiles when they are not
     int lists() const { return shift ? bins() : tiles(); }
 };
-ListGrid list_grid(int image_width, int image_height);
-// 0: choose by image size; 1, 2, 4: bins of that many tiles a side, for the whole process
-int set_list_bin(int tiles_per_side);
+// list_bin: 0: choose by image size; 1, 2, 4, 8: bins of that many tiles a side (dsx_camera::list_bin)
+ListGrid list_grid(int image_width, int image_height, int list_bin);
+inline ListGrid list_grid(const dsx_camera& cam)
+{
+    return list_grid(cam.image_width, cam.image_height, cam.list_bin);
+}
+inline bool valid_list_bin(int b)
+{
+    return b == 0 || b == 1 || b == 2 || b == 4 || b == 8;
+}
 
 // Layout of the `ranges` buffer of the forward (int32 words):
 //   fine[tiles + 1]   ranges of the per-tile lists as the reference defines them (the index of a
 //                     tile's first pair in the fully sorted key array; the last word is the
 //                     number of pairs)
+//   shift[1]          log2 of the bin side that the lists were built for (0: one list per tile): the
+//                     blend kernels compare it with the bin size they are launched for and walk
+//                     nothing when the two differ
 // and, when the lists are binned,
 //   last_tile[1]      highest tile that holds a pair of non-negative depth, -1 if none
 //   bins[bins + 1]    ranges of the bin lists inside sorted_ids
@@ -201,16 +211,19 @@ int set_list_bin(int tiles_per_side);
 //                     blended, and that entry's index in the per-tile list
 struct RangesLayout
 {
-    int fine, last_tile, bins, walk, count;
+    int fine, header, last_tile, bins, walk, count;
+    int ready; // words that exist before the blend forward runs (everything but `walk`)
 };
 inline RangesLayout ranges_layout(const ListGrid& g)
 {
     RangesLayout r;
     r.fine = 0;
-    r.last_tile = g.tiles() + 1;
+    r.header = g.tiles() + 1;
+    r.last_tile = r.header + 1;
     r.bins = r.last_tile + 1;
     r.walk = r.bins + g.bins() + 1;
-    r.count = g.shift ? r.walk + g.tiles() * 8 : g.tiles() + 1;
+    r.count = g.shift ? r.walk + g.tiles() * 8 : r.header + 1;
+    r.ready = g.shift ? r.walk : r.count;
     return r;
 }
 
@@ -246,7 +259,7 @@ struct OrderLayout
     size_t bytes;
 };
 // the grid is the last member, so every other offset depends on n alone
-OrderLayout order_layout(int64_t n, int image_width = 0, int image_height = 0);
+OrderLayout order_layout(int64_t n, int image_width = 0, int image_height = 0, int list_bin = 0);
 
 // Workspace of the tile lists for k keys.
 struct ListsWorkspace
@@ -335,16 +348,13 @@ inline ZeroJobs make_zero_jobs(int64_t n, int num_bases, float* v_mean3d, float*
     return jobs;
 }
 
-int launch_blend_fwd(const dsx_camera& cam, const int32_t* ranges, const int32_t* sorted_ids,
-                     const float* splats, float* image, float* final_T, int32_t* final_idx,
-                     hipStream_t stream,
-                     const uint32_t* sort_flag_a = nullptr, const uint32_t* sort_flag_b = nullptr,
-                     float* prepare_grads = nullptr, int64_t num_gaussians = 0, int32_t* lists = nullptr,
-                     bool prepare_marks = false);
-int launch_blend_bwd(const dsx_camera& cam, int64_t n, const int32_t* ranges,
-                     const int32_t* sorted_ids, const float* splats, const float* final_T,
-                     const int32_t* final_idx, const float* v_image, float* grads,
-                     hipStream_t stream, bool grads_prepared = false, const int32_t* lists = nullptr,
+int launch_blend_fwd(const dsx_camera& cam, int64_t n, int64_t k, int32_t* ranges, const int32_t* sorted_ids,
+                     const float* splats, float* image, float* final_T, int32_t* final_idx, hipStream_t stream,
+                     bool check_header, const uint32_t* sort_flag_a = nullptr, const uint32_t* sort_flag_b = nullptr,
+                     float* prepare_grads = nullptr, bool prepare_marks = false);
+int launch_blend_bwd(const dsx_camera& cam, int64_t n, int64_t k, const int32_t* ranges, const int32_t* sorted_ids,
+                     const float* splats, const float* final_T, const int32_t* final_idx, const float* v_image,
+                     float* grads, hipStream_t stream, bool check_header, bool grads_prepared = false,
                      bool with_marks = false, const ZeroJobs* zeros = nullptr);
 int launch_gaussian_bwd(const dsx_camera& cam, int64_t n, int num_bases, const float* means3d,
                         const float* scales, const float* quats, const float* splats,

@@ -12,7 +12,6 @@
 // once and moved twice, instead of 12 bytes moved five times.
 #include "dsx_common.h"
 
-#include <atomic>
 #include <mutex>
 
 namespace dsx
@@ -46,32 +45,18 @@ static hipStream_t helper_stream()
 
 // Bin size of the tile lists: one list per tile below 2048 tiles (a 256 x 256 image has 16 bins of
 // 4 x 4, and its 1024 blend wavefronts, four per tile there, would each filter a list sixteen times
-// the tile's own: forward 0.175 ms with lists per tile, 0.186 with bins of 2 x 2, 0.208 with 4 x 4);
-// from 2048 tiles on, bins of 4 x 4 tiles (a Gaussian's rectangle then touches a few bins instead of
-// a dozen tiles, and emission and partition shrink accordingly), or of 8 x 8 where that brings the
-// lists, slot 0 included, down to the 256 that ONE partition pass handles (1920 x 1080: 135 lists
-// instead of 510; 3 M small Gaussians 0.840 -> 0.827 ms per step, 1 M large ones 1.04 -> 0.68; a
-// 3840 x 2160 image needs two passes either way and its forward is slower with the larger bins,
-// 1.24 -> 1.32 ms, because every tile filters four times as many entries).  set_list_bin overrides
-// the choice for the process.
-static std::atomic<int> g_list_bin{0};
-
-int set_list_bin(int tiles_per_side)
-{
-    if(tiles_per_side != 0 && tiles_per_side != 1 && tiles_per_side != 2 && tiles_per_side != 4 && tiles_per_side != 8)
-        return DSX_ERR_BAD_ARG;
-    g_list_bin.store(tiles_per_side, std::memory_order_relaxed);
-    return DSX_OK;
-}
-
-ListGrid list_grid(int image_width, int image_height)
+// the tile's own); from 2048 tiles on, bins of 4 x 4 tiles (a Gaussian's rectangle then touches a few
+// bins instead of a dozen tiles, and emission and partition shrink accordingly), or of 8 x 8 where
+// that brings the lists, slot 0 included, down to the 256 that ONE partition pass handles
+// (1920 x 1080: 135 lists instead of 510; a 3840 x 2160 image needs two passes either way).
+// list_bin != 0 (dsx_camera::list_bin) asks for bins of that many tiles a side instead.
+ListGrid list_grid(int image_width, int image_height, int list_bin)
 {
     ListGrid g;
     g.ntx = tiles_x(image_width);
     g.nty = tiles_y(image_height);
-    const int forced = g_list_bin.load(std::memory_order_relaxed);
-    int side = forced ? forced : 1;
-    if(!forced && g.ntx * g.nty >= 2048)
+    int side = list_bin ? list_bin : 1;
+    if(!list_bin && g.ntx * g.nty >= 2048)
     {
         auto lists = [&](int b) { return ((g.ntx + b - 1) / b) * ((g.nty + b - 1) / b); };
         side = (slot_bits(lists(4)) > 8 && slot_bits(lists(8)) <= 8) ? 8 : 4;
@@ -685,7 +670,7 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
 // depth order of the Gaussians and the scanned tile counts in that order
 // ---------------------------------------------------------------------------------------
 
-OrderLayout order_layout(int64_t n, int image_width, int image_height)
+OrderLayout order_layout(int64_t n, int image_width, int image_height, int list_bin)
 {
     auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
     OrderLayout o;
@@ -710,7 +695,7 @@ OrderLayout order_layout(int64_t n, int image_width, int image_height)
     off = align(off + (size_t)kMaxPasses32 * kBins32 * 4);
     o.sort = off;
     off = align(off + sort32_workspace(n, 32, sort32_tile_keys(n)).bytes);
-    const ListGrid g = list_grid(image_width, image_height);
+    const ListGrid g = list_grid(image_width, image_height, list_bin);
     o.cover = off;
     off += (size_t)((g.ntx + 1) * (g.nty + 1) + 1) * 4;
     o.bin_cover = off;
@@ -720,7 +705,7 @@ OrderLayout order_layout(int64_t n, int image_width, int image_height)
     o.key_count = off; // inside the region that is zeroed with the corner grids
     off = align(off + 16);
     o.ranges = off;
-    off += (size_t)(ranges_layout(g).count - (g.shift ? g.tiles() * 8 : 0)) * 4;
+    off += (size_t)ranges_layout(g).ready * 4;
     o.bytes = align(off);
     return o;
 }
@@ -899,6 +884,8 @@ struct CountsJob
     uint32_t* slot_hist; // may be null
     int32_t* ranges;
     int32_t* last;       // may be null: receives the highest occupied tile, -1 if none
+    int32_t* header;     // may be null: receives header_value (the bin shift the lists are built for)
+    int32_t header_value;
     Digits32 plan;
 };
 struct CountsJobs
@@ -1032,6 +1019,8 @@ __global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(const Counts
         ranges[tiles] = (int32_t)s_carry; // K
         if(J.last)
             *J.last = last;
+        if(J.header)
+            *J.header = J.header_value;
         for(int p = 0; p < plan.passes; ++p)
             atomicAdd(&hist[p * kBins32], negatives);
     }
@@ -1045,20 +1034,20 @@ __global__ __launch_bounds__(kCoverThreads) void tile_counts_kernel(const Counts
 void depth_order_clear_region(const dsx_camera& cam, int64_t n, void* order, uint32_t** words, int64_t* count)
 {
     // the sort's histograms, counters and look-back statuses and, right behind them, the corner grid
-    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height);
+    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height, cam.list_bin);
     const Sort32Workspace w = sort32_workspace(n, 32, sort32_tile_keys(n));
     *words = reinterpret_cast<uint32_t*>(static_cast<char*>(order) + o.sort + w.hist);
     *count = (int64_t)((w.bytes + (o.ranges - o.cover)) / 4);
 }
 
-// k_host (optional, with k_copied): receives the number of pairs as 8 bytes as soon as the
-// rectangles have been counted; k_copied is recorded behind that copy.
+// k_host (optional, with k_copied): receives the two pair counts (uint64[2]: per-tile lists, bin lists) as
+// soon as the rectangles have been counted; k_copied is recorded behind that copy.
 int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_t stream, bool already_cleared,
                        void* k_host, hipEvent_t k_copied)
 {
     if(n <= 0)
         return DSX_OK;
-    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height);
+    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height, cam.list_bin);
     char* base = static_cast<char*>(order);
     uint32_t* keys_a = reinterpret_cast<uint32_t*>(base + o.depth_keys);
     uint32_t* keys_b = reinterpret_cast<uint32_t*>(base + o.keys_alt);
@@ -1096,7 +1085,7 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
     bool k_copy_ok = true;
     {
         hipStream_t cs = side ? side : stream;
-        const ListGrid lg = list_grid(cam.image_width, cam.image_height);
+        const ListGrid lg = list_grid(cam);
         const RangesLayout rl = ranges_layout(lg);
         const int ntx = lg.ntx, nty = lg.nty;
         const int cells = (ntx + 1) * (nty + 1) + 1;
@@ -1129,10 +1118,10 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
                                reinterpret_cast<const uint2*>(base + o.rects), n, ntx, nty, lg.shift, lg.nbx, lg.nby,
                                use_lds, grid, bin_grid, reinterpret_cast<unsigned long long*>(base + o.key_count));
         }
-        // the pairs of the lists that will be built: per bin when the lists are binned
+        // both pair counts, 16 bytes: of the per-tile lists (what the reference calls K: the fine ranges
+        // and final_idx index that many pairs) and of the bin lists (zero when the lists are per tile)
         if(k_host)
-            k_copy_ok = hipMemcpyAsync(k_host, base + o.key_count + (lg.shift ? 8 : 0), 8, hipMemcpyDeviceToHost,
-                                       cs) == hipSuccess &&
+            k_copy_ok = hipMemcpyAsync(k_host, base + o.key_count, 16, hipMemcpyDeviceToHost, cs) == hipSuccess &&
                         hipEventRecord(k_copied, cs) == hipSuccess;
         {
             CountsJobs jobs;
@@ -1145,6 +1134,8 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
             fine.slot_hist = lg.shift ? nullptr : reinterpret_cast<uint32_t*>(base + o.slot_hist);
             fine.ranges = ranges + rl.fine;
             fine.last = lg.shift ? ranges + rl.last_tile : nullptr;
+            fine.header = ranges + rl.header;
+            fine.header_value = lg.shift;
             jobs.job[1] = fine;
             if(lg.shift)
             {
@@ -1157,6 +1148,7 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
                 bins.slot_hist = reinterpret_cast<uint32_t*>(base + o.slot_hist);
                 bins.ranges = ranges + rl.bins;
                 bins.last = nullptr;
+                bins.header = nullptr;
             }
             DSX_TIMED("tile_counts_kernel", cs);
             hipLaunchKernelGGL(tile_counts_kernel, dim3(lg.shift ? 2 : 1), dim3(kCoverThreads),
@@ -1200,7 +1192,7 @@ int launch_depth_order(const dsx_camera& cam, int64_t n, void* order, hipStream_
         DSX_TIMED("ordered_block_sums_kernel", stream);
         hipLaunchKernelGGL(ordered_block_sums_kernel, dim3((unsigned)blocks), dim3(kProjBlock), 0, stream,
                            reinterpret_cast<const uint2*>(base + o.rects_sorted), n,
-                           list_grid(cam.image_width, cam.image_height).shift, block_sums);
+                           list_grid(cam).shift, block_sums);
     }
     if(hipGetLastError() != hipSuccess)
         return finish(DSX_ERR_LAUNCH);
@@ -1429,16 +1421,18 @@ template <typename SlotT>
 static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_tiles, const void* order,
                            int32_t* sorted_ids, int32_t* ranges, void* workspace, hipStream_t stream)
 {
-    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height);
+    const OrderLayout o = order_layout(n, cam.image_width, cam.image_height, cam.list_bin);
     const char* obase = static_cast<const char*>(order);
-    const ListGrid lg = list_grid(cam.image_width, cam.image_height);
+    const ListGrid lg = list_grid(cam);
     const RangesLayout rl = ranges_layout(lg);
     // what the depth order left ready: everything but the part that the blend forward writes
-    const int ready_words = lg.shift ? rl.walk : rl.count;
+    const int ready_words = rl.ready;
     if(k <= 0)
     {
         // no pairs: the ranges are all zero (and no tile is occupied)
         int rc = launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), ready_words, 0u, stream);
+        if(rc == DSX_OK && lg.shift)
+            rc = launch_fill_u32(reinterpret_cast<uint32_t*>(ranges) + rl.header, 1, (uint32_t)lg.shift, stream);
         if(rc == DSX_OK && lg.shift)
             rc = launch_fill_u32(reinterpret_cast<uint32_t*>(ranges) + rl.last_tile, 1, 0xffffffffu, stream);
         return rc;
@@ -1488,7 +1482,7 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
 int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
                       int32_t* ranges, void* workspace, hipStream_t stream)
 {
-    const int num_tiles = list_grid(cam.image_width, cam.image_height).lists();
+    const int num_tiles = list_grid(cam).lists();
     if(k >= (1ll << 30))
         return DSX_ERR_TOO_LARGE;
     if(n <= 0)

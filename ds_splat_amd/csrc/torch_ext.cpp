@@ -36,7 +36,7 @@ struct Camera
 
 Camera make_camera(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
                    int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view, const at::Tensor& proj,
-                   const at::Tensor& campos, const at::Tensor& bg, const at::Device& dev)
+                   const at::Tensor& campos, const at::Tensor& bg, int64_t list_bin, const at::Device& dev)
 {
     Camera cam;
     auto prep = [&](const at::Tensor& t) { return t.to(dev, at::kFloat).contiguous(); };
@@ -57,18 +57,23 @@ Camera make_camera(int64_t height, int64_t width, double tanfovx, double tanfovy
     cam.c.proj = cam.proj.data_ptr<float>();
     cam.c.campos = cam.campos.data_ptr<float>();
     cam.c.bg = cam.bg.data_ptr<float>();
+    TORCH_CHECK(list_bin == 0 || list_bin == 1 || list_bin == 2 || list_bin == 4 || list_bin == 8,
+                "list_bin must be 0 (the library's choice), 1, 2, 4 or 8 tiles a side");
+    cam.c.list_bin = (int32_t)list_bin;
     return cam;
 }
 
 at::Tensor& pinned_key_count()
 {
-    // one pinned int64 per host thread: the landing place of the key count
-    thread_local at::Tensor slot = at::zeros({1}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
+    // two pinned int64 per host thread: the landing place of the two pair counts
+    thread_local at::Tensor slot = at::zeros({2}, at::TensorOptions().dtype(at::kLong).pinned_memory(true));
     return slot;
 }
 
 } // namespace
 
+// list_bin: tiles per side of the bins that the tile lists are built for (0: the library's choice);
+// the backward of this forward must be given the same value.
 // image[H,W,3], radii[N], splats[N,12], sorted_ids[K], ranges[dsx_ranges_count], final_T[H,W], final_idx[H,W]
 // (the 3-D covariances are not kept: the backward rebuilds them from scales and rotations, or
 // reads cov3d_precomp) and, when prepare_backward is set, the backward's gradient accumulator
@@ -77,7 +82,7 @@ at::Tensor& pinned_key_count()
 std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
                                 int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view,
                                 const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
-                                const at::Tensor& means3d, const c10::optional<at::Tensor>& scales,
+                                int64_t list_bin, const at::Tensor& means3d, const c10::optional<at::Tensor>& scales,
                                 const c10::optional<at::Tensor>& quats, const at::Tensor& opacities,
                                 const c10::optional<at::Tensor>& shs, const c10::optional<at::Tensor>& cov3d_precomp,
                                 const c10::optional<at::Tensor>& colors_precomp, bool prepare_backward,
@@ -86,7 +91,7 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
     const at::Device dev = means3d.device();
     c10::DeviceGuard guard(dev);
     Camera cam = make_camera(height, width, tanfovx, tanfovy, scale_modifier, sh_degree, max_sh_degree, view, proj,
-                             campos, bg, dev);
+                             campos, bg, list_bin, dev);
     const int64_t n = means3d.numel() / 3;
     const auto f32 = at::TensorOptions().dtype(at::kFloat).device(dev);
     const auto i32 = at::TensorOptions().dtype(at::kInt).device(dev);
@@ -96,7 +101,7 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
     at::Tensor splats = at::empty({n, DSX_SPLAT_FLOATS}, f32);
     at::Tensor radii = at::empty({n}, i32);
     at::Tensor block_sums = at::empty({std::max<int64_t>(dsx_num_blocks(n), 1)}, i32);
-    const size_t order_bytes = dsx_order_bytes(n, (int32_t)width, (int32_t)height);
+    const size_t order_bytes = dsx_order_bytes(n, (int32_t)width, (int32_t)height, cam.c.list_bin);
     at::Tensor order = at::empty({(int64_t)std::max<size_t>(order_bytes, 1)}, u8);
     at::Tensor& k_host = pinned_key_count();
     uint32_t* bs = reinterpret_cast<uint32_t*>(block_sums.data_ptr<int32_t>());
@@ -106,11 +111,11 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
                               order_bytes, k_host.data_ptr<int64_t>(), s));
     const int64_t k = *k_host.data_ptr<int64_t>();
     at::Tensor sorted_ids = at::empty({k}, i32);
-    at::Tensor ranges = at::empty({dsx_ranges_count((int32_t)width, (int32_t)height)}, i32);
+    at::Tensor ranges = at::empty({dsx_ranges_count((int32_t)width, (int32_t)height, cam.c.list_bin)}, i32);
     at::Tensor image = at::empty({height, width, 3}, f32);
     at::Tensor final_T = at::empty({height, width}, f32);
     at::Tensor final_idx = at::empty({height, width}, i32);
-    const size_t ws_bytes = dsx_workspace_bytes(n, k, (int32_t)width, (int32_t)height);
+    const size_t ws_bytes = dsx_workspace_bytes(n, k, (int32_t)width, (int32_t)height, cam.c.list_bin);
     at::Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 1)}, u8);
     at::Tensor grads = prepare_backward && n > 0 ? at::empty({(int64_t)(dsx_grads_bytes(n) / 4)}, f32) : at::Tensor();
     check(dsx_forward_finish(&cam.c, n, k, splats.data_ptr<float>(), order.data_ptr(), sorted_ids.data_ptr<int32_t>(),
@@ -126,7 +131,7 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
 std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, double tanfovy, double scale_modifier,
                                  int64_t sh_degree, int64_t max_sh_degree, const at::Tensor& view,
                                  const at::Tensor& proj, const at::Tensor& campos, const at::Tensor& bg,
-                                 int64_t num_bases, const at::Tensor& means3d, const c10::optional<at::Tensor>& scales,
+                                 int64_t list_bin, int64_t num_bases, const at::Tensor& means3d, const c10::optional<at::Tensor>& scales,
                                  const c10::optional<at::Tensor>& quats, const at::Tensor& splats,
                                  const c10::optional<at::Tensor>& cov3d_precomp, const at::Tensor& radii,
                                  const at::Tensor& ranges,
@@ -137,18 +142,18 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
     const at::Device dev = means3d.device();
     c10::DeviceGuard guard(dev);
     Camera cam = make_camera(height, width, tanfovx, tanfovy, scale_modifier, sh_degree, max_sh_degree, view, proj,
-                             campos, bg, dev);
+                             campos, bg, list_bin, dev);
     const int64_t n = means3d.numel() / 3;
     const auto f32 = at::TensorOptions().dtype(at::kFloat).device(dev);
     TORCH_CHECK(v_image.is_contiguous() && v_image.scalar_type() == at::kFloat && v_image.numel() == height * width * 3,
                 "v_image must be a contiguous float32 [H, W, 3] tensor");
-    // The lists that `ranges` and `sorted_ids` describe are per tile or per bin of tiles, as the library
-    // chose (or was told) when the forward ran; the size of `ranges` says which.  A backward that read
-    // them the other way would walk off the end of sorted_ids.
+    // The lists that `ranges` and `sorted_ids` describe are per tile or per bin of tiles, as the forward was
+    // told (list_bin); the library compares the buffer's header word with this call's bin size on the device.
     TORCH_CHECK(ranges.is_contiguous() && ranges.scalar_type() == at::kInt &&
-                    ranges.numel() == dsx_ranges_count((int32_t)width, (int32_t)height),
-                "ranges does not have the layout of this image size and of the tile lists' current bin size "
-                "(dsx_set_list_bin must not change between a forward and its backward)");
+                    ranges.numel() == dsx_ranges_count((int32_t)width, (int32_t)height, cam.c.list_bin),
+                "ranges does not have the layout of this image size and bin size (the backward must be given the "
+                "list_bin of its forward)");
+    TORCH_CHECK(sorted_ids.is_contiguous() && sorted_ids.scalar_type() == at::kInt, "sorted_ids must be int32");
     auto out = [&](int bit, std::initializer_list<int64_t> shape) {
         return (wanted >> bit) & 1 ? at::empty(shape, f32) : at::Tensor();
     };
@@ -167,7 +172,8 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
                         prepared_grads->numel() == (int64_t)(dsx_grads_bytes(n) / 4) && prepared_grads->device() == dev,
                     "prepared_grads must be the float32 accumulator of this forward (dsx_grads_bytes(N) bytes)");
     at::Tensor grads = prepared ? *prepared_grads : at::empty({(int64_t)(dsx_grads_bytes(n) / 4)}, f32);
-    check(dsx_backward(&cam.c, n, (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales), fptr(quats),
+    check(dsx_backward(&cam.c, n, sorted_ids.numel(), (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales),
+                       fptr(quats),
                        splats.data_ptr<float>(), fptr(cov3d_precomp), radii.data_ptr<int32_t>(),
                        ranges.data_ptr<int32_t>(), sorted_ids.numel() ? sorted_ids.data_ptr<int32_t>() : nullptr,
                        final_T.data_ptr<float>(), final_idx.data_ptr<int32_t>(), v_image.data_ptr<float>(),

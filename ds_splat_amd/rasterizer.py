@@ -96,8 +96,10 @@ class DsRasterizerFunction(torch.autograd.Function):
         ext = _native.load_torch_ext()
         opt = lambda t: t if t.numel() > 0 else None
         stream = torch.cuda.current_stream(means_3d.device).cuda_stream
+        # (the last entry: tiles per side of the bins of the tile lists; the backward is given the same)
         cam = (int(s.image_height), int(s.image_width), float(s.tanfovx), float(s.tanfovy), float(s.scale_modifier),
-               int(s.sh_degree), int(s.max_sh_degree), s.view_matrix, s.proj_matrix, s.campos, s.bg)
+               int(s.sh_degree), int(s.max_sh_degree), s.view_matrix, s.proj_matrix, s.campos, s.bg,
+               _native.default_list_bin())
         # a backward will follow: the forward's blend kernel, which leaves the memory system idle,
         # prepares the gradient accumulator on the side (sums zeroed, conics beside them), and the
         # first backward needs no fill and no second look at the splat records

@@ -24,7 +24,9 @@ class CameraArgs:
     """Holds the device tensors a ``dsx_camera`` points to (keeps them alive)."""
 
     def __init__(self, image_height, image_width, tanfovx, tanfovy, bg, scale_modifier, view_rowmajor,
-                 proj_rowmajor, sh_degree, max_sh_degree, campos):
+                 proj_rowmajor, sh_degree, max_sh_degree, campos, list_bin=None):
+        """list_bin: tiles per side of the bins of the tile lists (0: the library's choice by image size;
+        None: _native.default_list_bin() at the time of construction)."""
         dev = view_rowmajor.device
         f32 = lambda t: t.to(device=dev, dtype=torch.float32).contiguous()
         self.view = f32(view_rowmajor)
@@ -47,6 +49,7 @@ class CameraArgs:
         c.proj = self.proj.data_ptr()
         c.campos = self.campos.data_ptr()
         c.bg = self.bg.data_ptr()
+        c.list_bin = N.default_list_bin() if list_bin is None else int(list_bin)
         self.c = c
 
     @property
@@ -57,15 +60,30 @@ class CameraArgs:
     def num_tiles(self):
         return ((self.width + 15) // 16) * ((self.height + 15) // 16)
 
+    @property
+    def list_bin(self):
+        """what the calls are told (0: the library's choice); stages.list_bin(cam) resolves it"""
+        return int(self.c.list_bin)
 
-def camera_from_scene(sc, device, bg=None, sh_degree=None, scale_modifier=None):
+    def with_list_bin(self, list_bin):
+        """The same camera (same device tensors) asking for another bin size."""
+        other = CameraArgs.__new__(CameraArgs)
+        other.__dict__.update(self.__dict__)
+        c = N.Camera()
+        C.memmove(C.byref(c), C.byref(self.c), C.sizeof(N.Camera))
+        c.list_bin = int(list_bin)
+        other.c = c
+        return other
+
+
+def camera_from_scene(sc, device, bg=None, sh_degree=None, scale_modifier=None, list_bin=None):
     """CameraArgs for a ds_splat_amd.synthetic scene (API-convention matrices are transposed
     back to row-major here, as the rasterizer module does)."""
     return CameraArgs(sc["height"], sc["width"], sc["tanfovx"], sc["tanfovy"],
                       (sc["bg"] if bg is None else bg).to(device),
                       sc["scale_modifier"] if scale_modifier is None else scale_modifier,
                       sc["viewmatrix"].to(device).t().contiguous(), sc["projmatrix"].to(device).t().contiguous(),
-                      sc["sh_degree"] if sh_degree is None else sh_degree, 3, sc["campos"].to(device))
+                      sc["sh_degree"] if sh_degree is None else sh_degree, 3, sc["campos"].to(device), list_bin)
 
 
 def project_fwd(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, colors_precomp=None, order=None):
@@ -85,7 +103,7 @@ def project_fwd(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None,
 
 def new_order(cam, n, device):
     """The buffer that carries the depth order from the projection to the tile lists."""
-    nbytes = int(N.load().dsx_order_bytes(n, cam.width, cam.height))
+    nbytes = int(N.load().dsx_order_bytes(n, cam.width, cam.height, cam.list_bin))
     return torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=device)
 
 
@@ -111,7 +129,7 @@ def depth_order_view(n, order):
 
 def list_bin(cam):
     """Tiles per side of the bins that the tile lists of this image size are built for (1: per tile)."""
-    return int(N.load().dsx_list_bin(cam.width, cam.height))
+    return int(N.load().dsx_list_bin(cam.width, cam.height, cam.list_bin))
 
 
 def key_count(cam, n, order):
@@ -122,16 +140,17 @@ def key_count(cam, n, order):
 
 
 def split_lists(cam, lists):
-    """The parts of a `ranges` buffer (dsx_ranges_count words): dict with 'fine' [T+1] and, for
-    binned lists, 'last_tile' (int tensor [1]), 'bins' [bins+1] and 'walk' [T, 4, 2]."""
+    """The parts of a `ranges` buffer (dsx_ranges_count words): dict with 'fine' [T+1], 'header' [1]
+    (log2 of the bin side) and, for binned lists, 'last_tile' (int tensor [1]), 'bins' [bins+1] and
+    'walk' [T, 4, 2]."""
     t = cam.num_tiles
-    out = {"fine": lists[:t + 1]}
+    out = {"fine": lists[:t + 1], "header": lists[t + 1:t + 2]}
     b = list_bin(cam)
     if b > 1:
         nbx, nby = (((cam.width + 15) // 16) + b - 1) // b, (((cam.height + 15) // 16) + b - 1) // b
-        out["last_tile"] = lists[t + 1:t + 2]
-        out["bins"] = lists[t + 2:t + 2 + nbx * nby + 1]
-        out["walk"] = lists[t + 3 + nbx * nby:].view(t, 4, 2)
+        out["last_tile"] = lists[t + 2:t + 3]
+        out["bins"] = lists[t + 3:t + 3 + nbx * nby + 1]
+        out["walk"] = lists[t + 4 + nbx * nby:].view(t, 4, 2)
     return out
 
 
@@ -144,15 +163,15 @@ def tile_lists(cam, n, k, order, return_flags=False, return_lists=False):
     lib = N.load()
     dev = order.device
     sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
-    lists = torch.empty((int(lib.dsx_ranges_count(cam.width, cam.height)),), dtype=torch.int32, device=dev)
-    nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height))
+    lists = torch.empty((int(lib.dsx_ranges_count(cam.width, cam.height, cam.list_bin)),), dtype=torch.int32, device=dev)
+    nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height, cam.list_bin))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
     N.check(lib.dsx_tile_lists(cam.ref, n, k, _ptr(order), _ptr(sorted_ids), _ptr(lists), _ptr(ws), nbytes, _stream()))
     ranges = lists if return_lists else lists[:cam.num_tiles + 1]
     if not return_flags:
         return sorted_ids, ranges
     p_a, p_b = C.c_void_p(), C.c_void_p()
-    N.check(lib.dsx_sort_flags(n, k, cam.width, cam.height, _ptr(order), _ptr(ws) if k > 0 else None,
+    N.check(lib.dsx_sort_flags(n, k, cam.width, cam.height, cam.list_bin, _ptr(order), _ptr(ws) if k > 0 else None,
                                C.byref(p_a), C.byref(p_b)))
     torch.cuda.synchronize()
     read = lambda t, p: 0 if not p.value else int(t.view(torch.int32)[(p.value - t.data_ptr()) // 4].item())
@@ -203,21 +222,24 @@ def tile_ranges(sorted_keys, num_tiles):
 
 
 def blend_fwd(cam, ranges, sorted_ids, splats):
+    """ranges: the whole `ranges` buffer of tile_lists(..., return_lists=True) for this camera's bin size,
+    or, for per-tile lists, any tensor that starts with the T + 1 per-tile ranges."""
     lib = N.load()
+    n, k = splats.shape[0], sorted_ids.numel()
     dev = ranges.device
     image = torch.empty((cam.height, cam.width, 3), dtype=torch.float32, device=dev)
     final_T = torch.empty((cam.height, cam.width), dtype=torch.float32, device=dev)
     final_idx = torch.empty((cam.height, cam.width), dtype=torch.int32, device=dev)
-    N.check(lib.dsx_blend_fwd(cam.ref, _ptr(ranges), _ptr(sorted_ids), _ptr(splats), _ptr(image), _ptr(final_T),
-                              _ptr(final_idx), _stream()))
+    N.check(lib.dsx_blend_fwd(cam.ref, n, k, _ptr(ranges), _ptr(sorted_ids), _ptr(splats), _ptr(image),
+                              _ptr(final_T), _ptr(final_idx), _stream()))
     return image, final_T, final_idx
 
 
 def blend_bwd(cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image):
     lib = N.load()
     grads = torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=splats.device)
-    N.check(lib.dsx_blend_bwd(cam.ref, n, _ptr(ranges), _ptr(sorted_ids), _ptr(splats), _ptr(final_T),
-                              _ptr(final_idx), _ptr(v_image), _ptr(grads), _stream()))
+    N.check(lib.dsx_blend_bwd(cam.ref, n, sorted_ids.numel(), _ptr(ranges), _ptr(sorted_ids), _ptr(splats),
+                              _ptr(final_T), _ptr(final_idx), _ptr(v_image), _ptr(grads), _stream()))
     return grads
 
 
@@ -255,10 +277,10 @@ _pinned = threading.local()
 
 
 def _pinned_i64():
-    """One pinned int64 per host thread: the landing place of the key count."""
+    """Two pinned int64 per host thread: the landing place of the two pair counts."""
     t = getattr(_pinned, "slot", None)
     if t is None:
-        t = torch.zeros((1,), dtype=torch.int64, pin_memory=True)
+        t = torch.zeros((2,), dtype=torch.int64, pin_memory=True)
         _pinned.slot = t
     return t
 
@@ -267,7 +289,7 @@ class ForwardState:
     """What the forward keeps for the backward (the reference saves the analogous tensors
     on the autograd context, ds_splat/rasterizer.py:47-64)."""
     __slots__ = ("splats", "radii", "cov3d", "sorted_ids", "lists", "ranges", "final_T", "final_idx", "num_keys",
-                 "grads")
+                 "num_keys_per_tile", "list_bin", "grads")
 
 
 def sort_flag_indices(cam, n, k, order, workspace):
@@ -275,7 +297,7 @@ def sort_flag_indices(cam, n, k, order, workspace):
     the give-up flags of the two chained scans."""
     lib = N.load()
     p_a, p_b = C.c_void_p(), C.c_void_p()
-    N.check(lib.dsx_sort_flags(n, k, cam.width, cam.height, _ptr(order), _ptr(workspace) if k > 0 else None,
+    N.check(lib.dsx_sort_flags(n, k, cam.width, cam.height, cam.list_bin, _ptr(order), _ptr(workspace) if k > 0 else None,
                                C.byref(p_a), C.byref(p_b)))
     ia = (p_a.value - order.data_ptr()) // 4 if p_a.value else None
     ib = (p_b.value - workspace.data_ptr()) // 4 if p_b.value else None
@@ -303,18 +325,20 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
                                     _ptr(cov3d_precomp), _ptr(colors_precomp), _ptr(st.splats), _ptr(st.radii),
                                     _ptr(st.cov3d), _ptr(block_sums), _ptr(order), order.numel(),
                                     _ptr(k_host), stream))
-    k = int(k_host.item())
+    k = int(k_host[0].item())
     st.num_keys = k
+    st.num_keys_per_tile = int(k_host[1].item())
+    st.list_bin = cam.list_bin
     if after_project is not None:
         after_project(order, n, k)
     st.sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
     # the whole `ranges` buffer, and its first T+1 words: the per-tile ranges as the reference defines them
-    st.lists = torch.empty((int(lib.dsx_ranges_count(cam.width, cam.height)),), dtype=torch.int32, device=dev)
+    st.lists = torch.empty((int(lib.dsx_ranges_count(cam.width, cam.height, cam.list_bin)),), dtype=torch.int32, device=dev)
     st.ranges = st.lists[:cam.num_tiles + 1]
     image = torch.empty((cam.height, cam.width, 3), dtype=torch.float32, device=dev)
     st.final_T = torch.empty((cam.height, cam.width), dtype=torch.float32, device=dev)
     st.final_idx = torch.empty((cam.height, cam.width), dtype=torch.int32, device=dev)
-    nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height))
+    nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height, cam.list_bin))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
     st.grads = new_accumulator(n, dev) if prepare_grads else None
     N.check(lib.dsx_forward_finish(cam.ref, n, k, _ptr(st.splats), _ptr(order), _ptr(st.sorted_ids),
@@ -328,14 +352,14 @@ def backward(cam, st, num_bases, means3d, scales, quats, v_image):
     n = means3d.shape[0]
     dev = means3d.device
     o = _bwd_outputs(n, num_bases, dev)
-    if st.lists.numel() != int(lib.dsx_ranges_count(cam.width, cam.height)):
-        raise RuntimeError("the forward built its tile lists for another bin size (dsx_set_list_bin must not change "
-                           "between a forward and its backward)")
+    if cam.list_bin != st.list_bin:
+        raise RuntimeError("the forward built its tile lists for list_bin = %d, this camera asks for %d (a backward "
+                           "must be given the list_bin of its forward)" % (st.list_bin, cam.list_bin))
     # an accumulator that the forward prepared serves one backward; after that it holds sums
     prepared = getattr(st, "grads", None) is not None
     grads = st.grads if prepared else new_accumulator(n, dev)
     st.grads = None
-    N.check(lib.dsx_backward(cam.ref, n, num_bases, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(st.splats),
+    N.check(lib.dsx_backward(cam.ref, n, st.sorted_ids.numel(), num_bases, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(st.splats),
                              _ptr(st.cov3d), _ptr(st.radii), _ptr(st.lists), _ptr(st.sorted_ids), _ptr(st.final_T),
                              _ptr(st.final_idx), _ptr(v_image), _ptr(grads), int(prepared), _ptr(o["v_mean3d"]),
                              _ptr(o["v_means2d"]), _ptr(o["v_shs"]), _ptr(o["v_colors"]), _ptr(o["v_opacity"]),

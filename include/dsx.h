@@ -6,13 +6,16 @@
  * The library allocates nothing on the device: outputs and workspace are the caller's.
  * All functions return 0 on success or a negative dsx_status; dsx_error_string() explains it.
  * Functions are re-entrant: different streams / devices may be driven concurrently by different
- * host threads (each call uses the current HIP device).  Process-wide state, all of it behind
+ * host threads (each call uses the current HIP device), and nothing that a call computes depends on
+ * a process-wide setting: the bin size of the tile lists travels in dsx_camera::list_bin and, on the
+ * device, in the header word of the `ranges` buffer.  What the process does share, all of it behind
  * locks or atomics: (1) the optional per-kernel timing trace (dsx_trace_enable / dsx_trace_read),
  * a list behind a mutex, off by default; (2) one helper stream per device, created on first use
  * and kept until the process ends: dsx_depth_order / dsx_forward_project fork onto it and join
- * before they return, so that the tile counting runs beside the depth sort — callers on
+ * before they return, so that the tile counting runs beside the depth sort; callers on
  * different streams of one device share it and their forked parts serialise there; (3) the
- * blend-kernel form override of dsx_set_blend_pixels_per_lane; (4) the device address of the
+ * blend-kernel form override of dsx_set_blend_pixels_per_lane, a diagnostic that changes no result
+ * of the forward and only the order of the backward's sums; (4) the device address of the
  * built-in scratch of dsx_backward_static, looked up once per device.
  *
  * What each entry point replaces in the reference (deepsense-ai/ds-splat) is cited as
@@ -42,13 +45,17 @@ typedef enum dsx_status
     DSX_ERR_BAD_ARG = -1,      /* NULL where data is required, negative size, bad degree ... */
     DSX_ERR_LAUNCH = -2,       /* hipGetLastError() after a launch reported a failure       */
     DSX_ERR_RUNTIME = -3,      /* a HIP runtime call (memcpy, sync, event) failed           */
-    DSX_ERR_TOO_LARGE = -4,    /* sizes beyond 32-bit indexing of keys (K >= 2^30)          */
+    DSX_ERR_TOO_LARGE = -4,    /* 2^30 pairs or more in the lists that are built, or 2^31   */
+                               /* or more in the per-tile lists (the reference's K)         */
     DSX_ERR_WORKSPACE = -5,    /* workspace smaller than dsx_workspace_bytes() asks for     */
     DSX_ERR_STATIC_LIMIT = -6  /* n beyond DSX_STATIC_MAX_GAUSSIANS (dsx_backward_static)   */
 } dsx_status;
 
 /* Mirrors TorchRasterizationSettings, cpp/ds_cuda_rasterizer/rasterizer_torch.hpp:7-22.
- * `prefiltered` and `debug` are carried by the reference but never read; they are omitted. */
+ * `prefiltered` and `debug` are carried by the reference but never read; they are omitted.
+ * list_bin has no counterpart there: the tile lists are built per BIN of list_bin x list_bin tiles
+ * (1, 2, 4 or 8; 0 = the library's choice for the image size, see dsx_list_bin).  Every call that
+ * belongs to one forward and its backward must be given the same value. */
 typedef struct dsx_camera
 {
     int32_t image_height;
@@ -62,6 +69,7 @@ typedef struct dsx_camera
     const float* proj;      /* device float[16], row-major world->clip              */
     const float* campos;    /* device float[3]                                      */
     const float* bg;        /* device float[3]                                      */
+    int32_t list_bin;       /* tiles per side of a list's bin: 0 (automatic), 1, 2, 4, 8 */
 } dsx_camera;
 
 /*
@@ -81,8 +89,10 @@ typedef struct dsx_camera
  */
 
 const char* dsx_error_string(int status);
-/* 100 * major + minor.  200: the `ranges` buffer has dsx_ranges_count words and the accumulator
- * dsx_grads_bytes bytes (100 had tiles + 1 words and n * 12 floats). */
+/* 100 * major + minor.  300: the bin size of the tile lists is an argument (dsx_camera::list_bin and
+ * the size helpers) instead of a process-wide setting; the `ranges` buffer carries it in a header word;
+ * the blend entry points and the backward are told n and k and follow no id or list position beyond
+ * them; dsx_forward_project returns both pair counts.  (200 had dsx_set_list_bin.) */
 int dsx_version(void);
 /* bytes of the accumulator that dsx_forward_finish prepares and dsx_backward uses:
  * n * DSX_GRAD_FLOATS * 4 for the records + n bytes rounded up to 16 */
@@ -94,30 +104,31 @@ int64_t dsx_num_blocks(int64_t n);
 int32_t dsx_num_tiles(int32_t width, int32_t height);
 int32_t dsx_sort_passes(int32_t num_tiles);
 /* The tile lists of the whole forward (dsx_forward_project / dsx_forward_finish / dsx_backward,
- * dsx_depth_order / dsx_tile_lists) are built per BIN of b x b tiles, b = 1, 2, 4 or 8: a Gaussian
- * enters the list of every bin that its tile rectangle touches, and a blend tile walks its bin's
- * list and keeps the entries whose rectangle contains the tile.  With b = 1 the lists are the
- * reference's own (sorted_ids is the value array of its sorted keys, bit for bit); with b > 1 the
- * same entries reach every pixel in the same order, final_idx holds the same indices, and emission
- * and partition handle a fraction of the pairs.  dsx_list_bin says which b the library uses for an
- * image size (1 below 2048 tiles; above, 8 where that brings the lists down to the 256 slots of a
- * single partition pass and 4 does not, else 4); dsx_set_list_bin forces one for the whole process
- * (0: back to the library's choice) — not between the two halves of a forward or between a
- * forward and its backward.  dsx_ranges_count: int32 words of the `ranges` buffer of those entry
- * points: tiles + 1 words of per-tile ranges as the reference defines them and, for b > 1, the
- * highest occupied tile, the bins' ranges and 8 words per tile that the blend forward leaves for
- * the backward.  No counterpart in the reference. */
-int32_t dsx_list_bin(int32_t width, int32_t height);
-int dsx_set_list_bin(int tiles_per_side);
-int64_t dsx_ranges_count(int32_t width, int32_t height);
+ * dsx_depth_order / dsx_tile_lists / dsx_blend_fwd / dsx_blend_bwd) are built per BIN of b x b tiles,
+ * b = 1, 2, 4 or 8: a Gaussian enters the list of every bin that its tile rectangle touches, and a
+ * blend tile walks its bin's list and keeps the entries whose rectangle contains the tile.  With
+ * b = 1 the lists are the reference's own (sorted_ids is the value array of its sorted keys, bit for
+ * bit); with b > 1 the same entries reach every pixel in the same order, final_idx holds the same
+ * indices, and emission and partition handle a fraction of the pairs.  b is dsx_camera::list_bin, or,
+ * when that is 0, the library's choice for the image size: 1 below 2048 tiles; above, 8 where that
+ * brings the lists down to the 256 slots of a single partition pass and 4 does not, else 4.
+ * dsx_list_bin(width, height, list_bin) returns the b that a call with this list_bin uses (0 for a
+ * list_bin that is none of 0, 1, 2, 4, 8).
+ * dsx_ranges_count: int32 words of the `ranges` buffer of those entry points: tiles + 1 words of
+ * per-tile ranges as the reference defines them (cpp/rasterizer_torch.cu:23-42), one header word
+ * (log2 of b: the blend kernels walk nothing when it is not the b they were launched for) and, for
+ * b > 1, the highest occupied tile, the bins' ranges and 8 words per tile that the blend forward
+ * leaves for the backward.  No counterpart in the reference. */
+int32_t dsx_list_bin(int32_t width, int32_t height, int32_t list_bin);
+int64_t dsx_ranges_count(int32_t width, int32_t height, int32_t list_bin);
 /* bytes of `workspace` dsx_forward_finish / dsx_tile_lists need for k keys */
-size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height);
+size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height, int32_t list_bin);
 /* bytes of `workspace` dsx_sort_pairs needs for k keys, and dsx_sort_pairs_u32 for count pairs */
 size_t dsx_sort_workspace_bytes(int64_t k, int32_t num_tiles);
 size_t dsx_sort_u32_workspace_bytes(int64_t count, int32_t key_bits);
 /* bytes of the per-Gaussian `order` buffer that carries the depth order from the projection
  * (dsx_project_fwd / dsx_forward_project) to the tile lists (dsx_tile_lists / dsx_forward_finish) */
-size_t dsx_order_bytes(int64_t n, int32_t width, int32_t height);
+size_t dsx_order_bytes(int64_t n, int32_t width, int32_t height, int32_t list_bin);
 
 /* ------------------------------------------------------------------------------------ */
 /* Per-stage entry points (each one individually parity-tested and timed)                */
@@ -129,8 +140,9 @@ size_t dsx_order_bytes(int64_t n, int32_t width, int32_t height);
  * Gaussian counts as zero, cpp/rasterizer_torch.cu:99-104).  shs may be NULL iff
  * colors_precomp is given; scales/quats may be NULL iff cov3d_precomp is given (then cov3d
  * receives a copy).  cov3d may be NULL: it is then not stored (the reference keeps it for its
- * backward, cpp/rasterizer_torch.cu:207; dsx_gaussian_bwd can do without).  order (may be NULL): buffer of dsx_order_bytes(n, W, H) that also receives each
- * Gaussian's depth bits and packed tile rectangle, the input of dsx_depth_order. */
+ * backward, cpp/rasterizer_torch.cu:207; dsx_gaussian_bwd can do without).  order (may be NULL):
+ * buffer of dsx_order_bytes(n, W, H, cam->list_bin) that also receives each Gaussian's depth bits and
+ * packed tile rectangle, the input of dsx_depth_order. */
 int dsx_project_fwd(const dsx_camera* cam, int64_t n, const float* means3d, const float* scales,
                     const float* quats, const float* opacities, const float* shs,
                     const float* cov3d_precomp, const float* colors_precomp, float* splats,
@@ -163,9 +175,11 @@ int dsx_sort_pairs(int64_t k, int32_t num_tiles, int64_t* keys, int32_t* values,
 int dsx_tile_ranges(int64_t k, const int64_t* sorted_keys, int32_t num_tiles, int32_t* ranges,
                     void* stream);
 
-/* Stages 2+3, fast route — the same sorted_ids[k] and ranges[T+1] as dsx_emit_keys +
- * dsx_sort_pairs + dsx_tile_ranges (i.e. as calculate_keys_and_indices_kernel, thrust::sort_by_key
- * and identify_tile_ranges, cpp/rasterizer_torch.cu:70-104) without sorting K 64-bit keys: the
+/* Stages 2+3, fast route — with cam->list_bin = 1 the same sorted_ids[k] and ranges[T+1] as
+ * dsx_emit_keys + dsx_sort_pairs + dsx_tile_ranges (i.e. as calculate_keys_and_indices_kernel,
+ * thrust::sort_by_key and identify_tile_ranges, cpp/rasterizer_torch.cu:70-104) without sorting K
+ * 64-bit keys; with larger bins the same per-tile ranges and the lists per bin (see dsx_list_bin),
+ * which dsx_blend_fwd / dsx_blend_bwd walk when they are given the same cam->list_bin.  The
  * order (tile, depth bits, Gaussian index) is produced by (1) a stable sort of the n Gaussians by
  * their 32 depth bits, (2) emission of (tile slot, Gaussian) pairs in that order, (3) a stable
  * partition of the k pairs by tile slot.
@@ -175,10 +189,12 @@ int dsx_tile_ranges(int64_t k, const int64_t* sorted_keys, int32_t num_tiles, in
  * dsx_depth_order: step (1) on an `order` buffer the projection has filled; it also leaves the
  * scanned tile counts of the depth-ordered 256-Gaussian blocks, the number of pairs of every
  * tile and the digit histograms of the tile slots (from the rectangles by a 2-D prefix sum of
- * their corners: no pair is enumerated) in the buffer.
+ * their corners: no pair is enumerated) in the buffer.  The number of pairs k of the lists that
+ * dsx_tile_lists will build is the last entry of the block offsets (dsx_order_view).
  * dsx_order_view: device pointers into the buffer (depth order uint32[n], block offsets
  * uint32[dsx_num_blocks(n)+1] whose last entry is K), for inspection.
- * dsx_tile_lists: steps (2) and (3) and the ranges. */
+ * dsx_tile_lists: steps (2) and (3) and the ranges: sorted_ids[k], ranges[dsx_ranges_count(W, H,
+ * cam->list_bin)] (everything but the part that the blend forward writes). */
 int dsx_sort_pairs_u32(int64_t count, int32_t key_bits, uint32_t* keys, uint32_t* values,
                        void* workspace, size_t workspace_bytes, void* stream);
 int dsx_depth_order(const dsx_camera* cam, int64_t n, void* order, size_t order_bytes, void* stream);
@@ -192,8 +208,8 @@ int dsx_order_view(int64_t n, const void* order, const uint32_t** depth_order,
  * dsx_forward_finish, for callers that want to check after synchronising.  Either output may
  * be NULL; an address is NULL when its buffer is NULL or empty.  No counterpart in the
  * reference (thrust's sort has no such wait). */
-int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t height, const void* order,
-                   const void* workspace, const uint32_t** depth_sort_flag,
+int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t height, int32_t list_bin,
+                   const void* order, const void* workspace, const uint32_t** depth_sort_flag,
                    const uint32_t** partition_flag);
 int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const void* order,
                    int32_t* sorted_ids, int32_t* ranges, void* workspace, size_t workspace_bytes,
@@ -201,15 +217,22 @@ int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const void* orde
 
 /* Stage 4 — replaces rasterizer_cuda_forward + render_image_kernel,
  * cpp/rasterizer_torch.cu:44-68, cpp/rasterizer_kernels.cu:341-431.
- * image[H*W*3] (HWC, background not composited), final_T[H*W], final_idx[H*W]. */
-int dsx_blend_fwd(const dsx_camera* cam, const int32_t* ranges, const int32_t* sorted_ids,
-                  const float* splats, float* image, float* final_T, int32_t* final_idx,
-                  void* stream);
+ * image[H*W*3] (HWC, background not composited), final_T[H*W], final_idx[H*W].
+ * ranges / sorted_ids[k]: what dsx_tile_lists wrote for the same cam->list_bin (the kernel adds the
+ * part of `ranges` that the backward reads when the lists are per bin); with cam->list_bin = 1 (or 0
+ * on an image below 2048 tiles) ranges may also be the num_tiles + 1 words of dsx_tile_ranges and
+ * sorted_ids the values of dsx_sort_pairs.  n: Gaussians behind `splats`.  An id of the lists is
+ * taken only up to n - 1 and a list position only inside [0, k): lists in disorder give a wrong
+ * image, not a fetch outside the arrays; a `ranges` buffer whose header names another bin size
+ * than this call's gives a NaN image. */
+int dsx_blend_fwd(const dsx_camera* cam, int64_t n, int64_t k, int32_t* ranges, const int32_t* sorted_ids,
+                  const float* splats, float* image, float* final_T, int32_t* final_idx, void* stream);
 
 /* Stage 5a — replaces rasterize_backward_tensor + rasterize_backward_kernel,
  * cpp/gsplat/bindings.cu:140-194, cpp/gsplat/backward.cu:25-202.  grads[n*12] is zeroed by
- * the call and then accumulated with float atomics.  v_image[H*W*3]. */
-int dsx_blend_bwd(const dsx_camera* cam, int64_t n, const int32_t* ranges,
+ * the call and then accumulated with float atomics.  v_image[H*W*3].  ranges, sorted_ids, n, k: as
+ * for dsx_blend_fwd, after it has run on them. */
+int dsx_blend_bwd(const dsx_camera* cam, int64_t n, int64_t k, const int32_t* ranges,
                   const int32_t* sorted_ids, const float* splats, const float* final_T,
                   const int32_t* final_idx, const float* v_image, float* grads, void* stream);
 
@@ -245,8 +268,11 @@ int dsx_gaussian_bwd(const dsx_camera* cam, int64_t n, int32_t num_bases, const 
  * and two device drains at cpp/rasterizer_torch.cu:95-104; K is summed from the tile rectangles
  * by the first kernel that runs beside the depth sort) and, overlapping that read-back, the depth
  * order.  block_sums[dsx_num_blocks(n)] receives the tile count of each 256-Gaussian block
- * (not scanned).  order: device buffer of dsx_order_bytes(n, W, H).  *num_keys (host; pinned
- * memory lets the copy overlap) receives K. */
+ * (not scanned).  order: device buffer of dsx_order_bytes(n, W, H, cam->list_bin).  num_keys (host,
+ * TWO entries; pinned memory lets the copy overlap): [0] receives k, the number of pairs of the lists
+ * that dsx_forward_finish will build (entries of sorted_ids); [1] the number of pairs of the per-tile
+ * lists, the reference's K (equal to [0] when the lists are per tile), which the per-tile ranges and
+ * final_idx index.  DSX_ERR_TOO_LARGE when [0] >= 2^30 or [1] >= 2^31. */
 int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
                         const float* scales, const float* quats, const float* opacities,
                         const float* shs, const float* cov3d_precomp, const float* colors_precomp,
@@ -258,9 +284,9 @@ int dsx_forward_project(const dsx_camera* cam, int64_t n, const float* means3d,
  * outputs that backward needs; workspace as dsx_workspace_bytes(n, k, W, H).  If one of the two
  * sorts gave up a bounded wait (see dsx_sort_flags) the image is written as NaN: a failure
  * shows without a read-back of the flags.
- * The blend kernels of dsx_forward_finish and dsx_backward take an id from the lists only up to
- * n - 1 (larger or negative ones read as n - 1): lists in disorder give a wrong image or gradient,
- * not a fetch outside the splat records.  (dsx_blend_fwd is not told n and trusts its lists.)
+ * The blend kernels take an id from the lists only up to n - 1 (larger or negative ones read as
+ * n - 1) and a list position only inside [0, k): lists in disorder give a wrong image or gradient,
+ * not a fetch outside the splat records or sorted_ids.
  * grads_to_prepare (may be NULL; 16-byte aligned, dsx_grads_bytes(n) bytes): the accumulator that
  * a dsx_backward of this forward will use.  The blend kernel, which leaves the memory system idle,
  * prepares it on the side (the nine sums zeroed, each Gaussian's conic in the three spare places,
@@ -272,13 +298,15 @@ int dsx_forward_finish(const dsx_camera* cam, int64_t n, int64_t k, const float*
                        float* final_T, int32_t* final_idx, void* workspace,
                        size_t workspace_bytes, float* grads_to_prepare, void* stream);
 
-/* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316. grads is scratch of
+/* rasterizer_backward_deepsense, cpp/rasterizer_torch.cu:263-316.  k: entries of sorted_ids (the k
+ * of the forward); ranges: the buffer that dsx_forward_finish filled, for the same cam->list_bin (a
+ * buffer whose header names another bin size is not walked: the gradients are then zero).  grads is scratch of
  * dsx_grads_bytes(n) bytes, 16-byte aligned; grads_prepared != 0 says that dsx_forward_finish has
  * prepared it (true for one call: this one leaves sums in it).  The outputs are as for
  * dsx_gaussian_bwd: zero wherever the blend backward added no term to a Gaussian's record (most
  * of a dense scene), written by the blend kernel's wavefronts on their way out; the per-Gaussian
  * kernel then works on the marked Gaussians only. */
-int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
+int dsx_backward(const dsx_camera* cam, int64_t n, int64_t k, int32_t num_bases, const float* means3d,
                  const float* scales, const float* quats, const float* splats, const float* cov3d,
                  const int32_t* radii, const int32_t* ranges, const int32_t* sorted_ids,
                  const float* final_T, const int32_t* final_idx, const float* v_image,
@@ -298,8 +326,8 @@ int dsx_backward(const dsx_camera* cam, int64_t n, int32_t num_bases, const floa
  * share the one array: calls that overlap on a GPU (two streams, two host threads) race — keep
  * them on one stream or serialise them.  The array's device address is looked up on the first
  * call on each device: make that first call outside a graph capture. */
-int dsx_backward_static(const dsx_camera* cam, int64_t n, int32_t num_bases, const float* means3d,
-                        const float* scales, const float* quats, const float* splats,
+int dsx_backward_static(const dsx_camera* cam, int64_t n, int64_t k, int32_t num_bases,
+                        const float* means3d, const float* scales, const float* quats, const float* splats,
                         const float* cov3d, const int32_t* radii, const int32_t* ranges,
                         const int32_t* sorted_ids, const float* final_T, const int32_t* final_idx,
                         const float* v_image, float* v_mean3d, float* v_means2d, float* v_shs,
@@ -322,7 +350,7 @@ int dsx_forward_core(const float* means3d, const float* shs, const float* opacit
 /* reference (its test harness times whole calls on the host, tests/rasterizer_test.cpp:    */
 /* 112-143).  While enabled, every kernel launch of the library records a start/stop event  */
 /* pair; dsx_trace_read waits for them, returns up to max_entries (name, ms) records in     */
-/* launch order and clears the trace.  This is the only process-wide state of the library.  */
+/* launch order and clears the trace (process-wide, like the rest of the list at the top).  */
 /* ------------------------------------------------------------------------------------ */
 typedef struct dsx_trace_entry
 {

@@ -35,13 +35,14 @@ def blend_form():
 
 @pytest.fixture
 def list_bin():
-    """Returns a function that forces the bin size of the tile lists (1, 2, 4 or 8 tiles a side; 0: the
-    library's choice) for the rest of the test; the library's own choice is restored afterwards."""
+    """Returns a function that sets the bin size of the tile lists (1, 2, 4 or 8 tiles a side; 0: the
+    library's choice) that this package's callers ask for by default, for the rest of the test; the
+    library's own choice is restored afterwards.  (The native library has no such setting: the Python
+    callers pass the value with every call.)"""
     from ds_splat_amd import _native
-    lib = _native.load()
 
     def force(tiles_per_side):
-        _native.check(lib.dsx_set_list_bin(int(tiles_per_side)))
+        _native.set_default_list_bin(int(tiles_per_side))
 
     yield force
-    _native.check(lib.dsx_set_list_bin(0))
+    _native.set_default_list_bin(0)

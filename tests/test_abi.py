@@ -26,19 +26,6 @@ def test_library_exports_every_declared_symbol():
         assert getattr(lib, name) is not None
 
 
-def test_probe_library_exports_what_its_header_declares():
-    """include/dsx_probe.h: the benchmark's streaming probe lives in a library of its own."""
-    import ctypes as C
-    text = open(os.path.join(ROOT, "include", "dsx_probe.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    names = sorted(set(re.findall(r"\b(dsxp_[a-z0-9_]+)\s*\(", text)))
-    assert names == ["dsxp_stream_probe"]
-    lib = C.CDLL(os.path.join(ROOT, "ds_splat_amd", "lib", "libdsx_probe.so"))
-    for name in names:
-        assert getattr(lib, name) is not None
-    assert lib.dsxp_stream_probe(None, None, C.c_size_t(16), 2, None, None) == -1     # no launch without buffers
-
-
 def test_torch_binding_loads_and_links_the_library():
     from ds_splat_amd import _native
     ext = _native.load_torch_ext()
@@ -55,26 +42,28 @@ def test_host_helpers():
     assert lib.dsx_num_tiles(40, 30) == 6
     # 32 depth bits + bits for tile ids 0..T (slot 0 = negative keys), at most 9 bits a pass
     assert lib.dsx_sort_passes(8160) == 5 and lib.dsx_sort_passes(255) == 5 and lib.dsx_sort_passes(32400) == 6
-    assert lib.dsx_workspace_bytes(0, 0, 64, 64) >= 0
+    assert lib.dsx_workspace_bytes(0, 0, 64, 64, 0) >= 0
     # tile lists: two slot buffers (16-bit slots up to 65534 lists, else 32-bit) and one id buffer
-    assert (1 << 20) * 8 < lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080) < (1 << 20) * 9
-    assert lib.dsx_set_list_bin(1) == 0
-    assert (1 << 20) * 12 < lib.dsx_workspace_bytes(0, 1 << 20, 16400, 1040) < (1 << 20) * 13
-    # bins of the tile lists: 4 x 4 tiles from 2048 tiles on, unless forced; the `ranges` buffer grows with them
-    assert lib.dsx_list_bin(1920, 1080) == 1 and lib.dsx_ranges_count(1920, 1080) == 8160 + 1
-    assert lib.dsx_set_list_bin(0) == 0 and lib.dsx_set_list_bin(3) == -1
+    assert (1 << 20) * 8 < lib.dsx_workspace_bytes(0, 1 << 20, 1920, 1080, 0) < (1 << 20) * 9
+    assert (1 << 20) * 12 < lib.dsx_workspace_bytes(0, 1 << 20, 16400, 1040, 1) < (1 << 20) * 13
+    # bins of the tile lists: an argument of every call (0: the library's choice); the `ranges` buffer is the
+    # per-tile ranges and a header word, and grows with the bins
+    assert lib.dsx_list_bin(1920, 1080, 1) == 1 and lib.dsx_ranges_count(1920, 1080, 1) == 8160 + 2
+    assert lib.dsx_list_bin(1920, 1080, 3) == 0 and lib.dsx_ranges_count(1920, 1080, 3) == 0
+    assert lib.dsx_order_bytes(100, 1920, 1080, 5) == 0 and lib.dsx_workspace_bytes(0, 10, 1920, 1080, -1) == 0
     # per tile below 2048 tiles; 8 x 8 where that needs one partition pass and 4 x 4 two (1080p: 135 against
     # 510 lists); 4 x 4 where it fits one pass itself (128 lists) or where both need two (4K: 510 against 2040)
-    assert lib.dsx_list_bin(1920, 1080) == 8 and lib.dsx_list_bin(1024, 512) == 4 and lib.dsx_list_bin(1024, 496) == 1
-    assert lib.dsx_list_bin(3840, 2160) == 4 and lib.dsx_set_list_bin(8) == 0 and lib.dsx_list_bin(640, 480) == 8
-    assert lib.dsx_set_list_bin(0) == 0
-    assert lib.dsx_ranges_count(1920, 1080) == (8160 + 1) + 1 + (15 * 9 + 1) + 8 * 8160
-    assert lib.dsx_ranges_count(240, 240) == 225 + 1
+    assert lib.dsx_list_bin(1920, 1080, 0) == 8 and lib.dsx_list_bin(1024, 512, 0) == 4
+    assert lib.dsx_list_bin(1024, 496, 0) == 1 and lib.dsx_list_bin(3840, 2160, 0) == 4
+    assert lib.dsx_list_bin(640, 480, 8) == 8 and lib.dsx_list_bin(640, 480, 0) == 1
+    assert lib.dsx_ranges_count(1920, 1080, 0) == (8160 + 1) + 1 + 1 + (15 * 9 + 1) + 8 * 8160
+    assert lib.dsx_ranges_count(1920, 1080, 8) == lib.dsx_ranges_count(1920, 1080, 0)
+    assert lib.dsx_ranges_count(240, 240, 0) == 225 + 2
     assert lib.dsx_sort_workspace_bytes(1 << 20, 8160) > (1 << 20) * 12
     assert lib.dsx_sort_u32_workspace_bytes(1 << 20, 32) > (1 << 20) * 8
     # order buffer: 4 uint32 arrays and two uint2 arrays per Gaussian
-    assert lib.dsx_order_bytes(1 << 20, 1920, 1080) > (1 << 20) * 32
-    assert lib.dsx_order_bytes(0, 3840, 2160) - lib.dsx_order_bytes(0, 16, 16) >= 241 * 136 * 4 - 512
+    assert lib.dsx_order_bytes(1 << 20, 1920, 1080, 0) > (1 << 20) * 32
+    assert lib.dsx_order_bytes(0, 3840, 2160, 0) - lib.dsx_order_bytes(0, 16, 16, 0) >= 241 * 136 * 4 - 512
     assert b"workspace" in lib.dsx_error_string(-5)
     assert lib.dsx_error_string(0) == b"ok"
 
@@ -90,11 +79,12 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.dsx_sort_pairs_u32(10, 33, 1, 1, 1, 0, None) == -1
     assert lib.dsx_sort_pairs_u32(10, 32, 1, 1, 1, 0, None) == -5
     assert lib.dsx_depth_order(None, 10, None, 0, None) == -1
-    assert lib.dsx_sort_flags(-1, 0, 16, 16, None, None, None, None) == -1
-    assert lib.dsx_sort_flags(10, 10, 16, 16, None, None, None, None) == 0
+    assert lib.dsx_sort_flags(-1, 0, 16, 16, 0, None, None, None, None) == -1
+    assert lib.dsx_sort_flags(10, 10, 16, 16, 3, None, None, None, None) == -1
+    assert lib.dsx_sort_flags(10, 10, 16, 16, 0, None, None, None, None) == 0
     # with a well-formed camera (its pointers are only compared with null before these checks fail)
     import ctypes as C
-    cam = _native.Camera(64, 64, 0.5, 0.5, 1.0, 3, 3, 8, 8, 8, 8)
+    cam = _native.Camera(64, 64, 0.5, 0.5, 1.0, 3, 3, 8, 8, 8, 8, 0)
     ref = C.byref(cam)
     fake = 16   # any non-null address: nothing is launched
     # the per-Gaussian backward needs the stored covariances or scales + rotations to rebuild them
@@ -104,8 +94,25 @@ def test_bad_arguments_are_rejected_without_touching_the_gpu():
     assert lib.dsx_gaussian_bwd(ref, 10, 17, fake, fake, fake, fake, None, fake, fake, *([None] * 8), None) == -1
     # the forward's first half wants a place for K; the backward its saved tensors
     assert lib.dsx_forward_project(ref, 10, *([fake] * 7), fake, fake, None, fake, fake, 1 << 20, None, None) == -1
-    assert lib.dsx_backward(ref, 10, 16, fake, fake, fake, fake, None, fake, None, fake, fake, fake, fake, fake, 0,
+    assert lib.dsx_backward(ref, 10, 5, 16, fake, fake, fake, fake, None, fake, None, fake, fake, fake, fake, fake, 0,
                             *([None] * 8), None) == -1
+    # list positions and ids are bounded by what the caller says it holds: a backward with entries but no
+    # sorted_ids, negative counts, and counts beyond 32-bit indexing are refused before anything is launched
+    full = [fake, fake, fake, fake, None, fake, fake]          # means3d .. radii, ranges
+    tail = [fake, fake, fake, fake, 0] + [None] * 8 + [None]    # final_T, final_idx, v_image, grads, prepared, outputs, stream
+    assert lib.dsx_backward(ref, 10, 5, 16, *full, None, *tail) == -1
+    assert lib.dsx_backward(ref, 10, -1, 16, *full, fake, *tail) == -1
+    assert lib.dsx_backward(ref, 10, 1 << 30, 16, *full, fake, *tail) == -4
+    assert lib.dsx_blend_fwd(ref, 10, 5, fake, None, fake, fake, fake, fake, None) == -1
+    assert lib.dsx_blend_fwd(ref, -1, 5, fake, fake, fake, fake, fake, fake, None) == -1
+    assert lib.dsx_blend_fwd(ref, 10, 1 << 31, fake, fake, fake, fake, fake, fake, None) == -4
+    assert lib.dsx_blend_bwd(ref, 10, 1 << 31, fake, fake, fake, fake, fake, fake, fake, None) == -4
+    assert lib.dsx_blend_bwd(ref, 10, 5, fake, None, fake, fake, fake, fake, fake, None) == -1
+    # a bin size that is none of 0, 1, 2, 4, 8 is a bad camera
+    bad = _native.Camera(64, 64, 0.5, 0.5, 1.0, 3, 3, 8, 8, 8, 8, 3)
+    assert lib.dsx_depth_order(C.byref(bad), 10, fake, 1 << 20, None) == -1
+    assert lib.dsx_blend_fwd(C.byref(bad), 10, 5, fake, fake, fake, fake, fake, fake, None) == -1
+    assert b"2^31" in lib.dsx_error_string(-4) and b"2^30" in lib.dsx_error_string(-4)
 
 
 def test_python_api_surface():

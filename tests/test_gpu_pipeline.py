@@ -284,10 +284,11 @@ def test_backward_twice_through_the_api_gives_the_same_gradients():
         assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * max(1.0, float(a.abs().max())))
 
 
-def test_inria_adaptor_composites_the_background_and_keeps_the_gradients():
-    """Channel-first image = HWC image + final_T * bg; gradients equal those of the wrapped API
-    for the same upstream gradient (the backward kernel's background term is the derivative of
-    exactly that product)."""
+def test_inria_adaptor_composites_the_background_and_keeps_the_gradients(oracle):
+    """Channel-first image = the oracle's image + the oracle's final_T * bg (the reference's forward leaves the
+    background out, cpp/rasterizer_kernels.cu:417-422, and its backward differentiates exactly that
+    product); gradients against the oracle's backward with the same background, and equal to those of the
+    wrapped API for the same upstream gradient."""
     from ds_splat_amd import inria_compat, stages
     sc = make_scene("cfg1", n=20000, width=320, height=200, sh_degree=3)
     bg = (0.3, 0.6, 0.1)
@@ -309,8 +310,23 @@ def test_inria_adaptor_composites_the_background_and_keeps_the_gradients():
     want = image.detach() + st.final_T.unsqueeze(-1) * torch.tensor(bg, device=DEV).view(1, 1, 3)
     assert torch.allclose(color.detach().permute(1, 2, 0), want, rtol=0, atol=1e-6)
     assert (st.final_T > 0.5).any() and float((color.detach().permute(1, 2, 0) - image.detach()).abs().max()) > 0.05
+    # against the CPU oracle: its image and final_T, composited here
+    img_o, radii_o, S, B = oracle_run(oracle, sc, 2.0, bg=np.asarray(bg, np.float32))
+    assert (radii2.cpu().numpy() == radii_o).all()
+    ok = S["margin"] > 1e-4
+    assert ok.mean() > 0.98
+    want_o = img_o + S["final_T"][..., None] * np.asarray(bg, np.float32).reshape(1, 1, 3)
+    got = color.detach().permute(1, 2, 0).cpu().numpy()
+    np.testing.assert_allclose(got[ok], want_o[ok], rtol=1e-4, atol=1e-5)
+    assert float(np.abs(want_o - img_o)[ok].max()) > 0.05          # the background does show
     color.backward(t["v_image"].permute(2, 0, 1))
     torch.cuda.synchronize()
+    fT, fidx, _ = gpu_forward_state(sc, 2.0)
+    gok = comparable_gaussians(S, B, sc["width"], fT, fidx)
+    got_grads = {"v_mean3d": p["means"].grad, "v_shs": p["shs"].grad, "v_opacity": p["opac"].grad,
+                 "v_scale": p["scales"].grad, "v_quat": p["rots"].grad}
+    check_grads_against_bounds({k: v.cpu().numpy() for k, v in got_grads.items()}, B, B["bounds"], gok,
+                               "inria adaptor")
     for k in p:
         a, b = leaves[k].grad, p[k].grad
         assert torch.allclose(a, b, rtol=1e-3, atol=1e-4 * max(1.0, float(a.abs().max()))), k
@@ -654,27 +670,91 @@ def test_a_sort_that_gave_up_poisons_the_image():
     assert torch.isnan(image).all()
 
 
-def test_backward_refuses_lists_of_another_bin_size(list_bin):
-    """The bin size of the tile lists is process-wide state for tests; if it changes between a forward
-    and its backward, the saved lists no longer mean what the backward's kernels would take them for
-    (per-tile ranges run far past the end of per-bin ids).  The binding sees it from the size of
-    `ranges` and raises before anything is launched."""
+def test_backward_uses_the_bin_size_of_its_own_forward(oracle, list_bin):
+    """The bin size of the tile lists is an argument of every native call and the autograd context keeps the one
+    its forward used: changing the package's default between a forward and its backward changes nothing for that
+    backward (gradients against the oracle)."""
     from ds_splat import GaussianRasterizationSettings, GaussianRasterizer
     sc = make_scene("cfg1", n=20000, width=640, height=360, sh_degree=3)
+    img_o, radii_o, S, B = oracle_run(oracle, sc, 2.0)
     t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
     settings = GaussianRasterizationSettings(
         image_height=sc["height"], image_width=sc["width"], tanfovx=sc["tanfovx"], tanfovy=sc["tanfovy"], bg=t["bg"],
         scale_modifier=1.0, viewmatrix=t["viewmatrix"], projmatrix=t["projmatrix"], sh_degree=sc["sh_degree"],
         max_sh_degree=3, campos=t["campos"], prefiltered=False, debug=False)
+    fT, fidx, _ = gpu_forward_state(sc, 2.0)
+    gok = comparable_gaussians(S, B, sc["width"], fT, fidx)
     for before, after in ((4, 1), (1, 4), (4, 8)):
         list_bin(before)
         means = t["means_3d"].clone().requires_grad_(True)
+        scales = (t["scales"] * 2.0).requires_grad_(True)
         image, _ = GaussianRasterizer(settings)(means, torch.zeros_like(means), t["shs"], None, t["opacities"],
-                                                t["scales"], t["rotations"], None)
+                                                scales, t["rotations"], None)
         list_bin(after)
-        with pytest.raises(RuntimeError, match="dsx_set_list_bin must not change"):
-            image.backward(t["v_image"])
+        image.backward(t["v_image"])
         torch.cuda.synchronize()
+        check_grads_against_bounds({"v_mean3d": means.grad.cpu().numpy(), "v_scale": scales.grad.cpu().numpy()}, B,
+                                   B["bounds"], gok, "bins %d then %d" % (before, after))
+
+
+def test_lists_of_another_bin_size_are_not_walked(list_bin):
+    """A `ranges` buffer carries the bin size it was built for in its header word; a blend launch that is told
+    another one (a caller's mix-up: the C ABI cannot see it on the host) reads no further: the forward stage
+    writes a NaN image, the backward leaves every gradient zero, and nothing is fetched outside the buffers."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg1", n=20000, width=640, height=360, sh_degree=3)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    for built, told in ((4, 1), (1, 4), (4, 8), (8, 2)):
+        cam = stages.camera_from_scene(sc, DEV, list_bin=built)
+        image, st = stages.forward(cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
+        assert int(stages.split_lists(cam, st.lists)["header"].item()) == {1: 0, 2: 1, 4: 2, 8: 3}[built]
+        assert torch.isfinite(image).all() and float(image.max()) > 0
+        other = cam.with_list_bin(told)
+        # the stage forward on the wrong layout: NaN image (the buffer is as long as the larger layout wants)
+        pad = torch.zeros(max(int(_ranges_words(other)), st.lists.numel()) + 8, dtype=torch.int32, device=DEV)
+        pad[:st.lists.numel()] = st.lists
+        img2, _, _ = stages.blend_fwd(other, pad, st.sorted_ids, st.splats)
+        torch.cuda.synchronize()
+        # (the stage entry takes per-tile ranges without a header too, dsx_tile_ranges' own, so it cannot refuse
+        # when it is told "per tile": positions are clamped and the image is merely wrong)
+        assert told == 1 or torch.isnan(img2).all(), (built, told)
+        # the whole backward on the wrong layout: zeros
+        st.lists = pad
+        st.list_bin = told
+        out = stages.backward(other, st, 16, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["v_image"])
+        torch.cuda.synchronize()
+        for key in ("v_mean3d", "v_shs", "v_opacity", "v_scale", "v_quat"):
+            assert float(out[key].abs().max()) == 0.0, (built, told, key)
+
+
+def _ranges_words(cam):
+    from ds_splat_amd import _native
+    return _native.load().dsx_ranges_count(cam.width, cam.height, cam.list_bin)
+
+
+def test_list_positions_beyond_the_ids_are_not_followed():
+    """Ranges whose ends lie beyond the entries of sorted_ids (a `ranges` buffer of another forward, a k that is
+    too small): the blend kernels clamp every position to [0, k) and give wrong numbers, not a fetch outside
+    sorted_ids.  Runs the stage entry points and the whole backward on per-tile and on binned lists."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg1", n=20000, width=640, height=360, sh_degree=3)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    for bins in (1, 4):
+        cam = stages.camera_from_scene(sc, DEV, list_bin=bins)
+        image, st = stages.forward(cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
+        k = st.sorted_ids.numel()
+        parts = stages.split_lists(cam, st.lists)
+        which = "fine" if bins == 1 else "bins"
+        assert int(parts[which][-1].item()) == k
+        # only the first third of the ids is handed over, with the full ranges
+        short = st.sorted_ids[:k // 3].clone()
+        img2, fT2, fidx2 = stages.blend_fwd(cam, st.lists, short, st.splats)
+        torch.cuda.synchronize()
+        assert torch.isfinite(img2).all()
+        st.sorted_ids = short
+        out = stages.backward(cam, st, 16, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["v_image"])
+        torch.cuda.synchronize()
+        assert all(torch.isfinite(out[key]).all() for key in ("v_mean3d", "v_shs", "v_scale"))
 
 
 def test_api_rejects_bad_inputs_with_the_reference_messages():

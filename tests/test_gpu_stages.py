@@ -410,7 +410,7 @@ def test_blend_fwd_vs_oracle(oracle, n, W, H, scale_mul, pixels_per_lane, blend_
     st_ = _stages()
     sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=31 + n, scale_mul=scale_mul)
     oracle.free(st)
-    cam = st_.camera_from_scene(sc, DEV)
+    cam = st_.camera_from_scene(sc, DEV, list_bin=1)       # the oracle's lists are the reference's: one per tile
     splats = dev(pack_splats(S, radii, A["opacities"]))
     image, final_T, final_idx = st_.blend_fwd(cam, dev(S["ranges"]), dev(S["sorted_ids"]), splats)
     torch.cuda.synchronize()
@@ -433,7 +433,7 @@ def test_blend_bwd_vs_oracle(oracle, n, W, H, scale_mul, bg, pixels_per_lane, bl
     s.bg[:] = list(bg)
     B = oracle.blend_bwd(s, S["ranges"], S["sorted_ids"], S["means2d"], S["conic"], S["rgb"], A["opacities"],
                          S["final_T"], S["final_idx"], A["v_image"])
-    cam = st_.camera_from_scene(sc, DEV, bg=torch.tensor(bg, dtype=torch.float32))
+    cam = st_.camera_from_scene(sc, DEV, bg=torch.tensor(bg, dtype=torch.float32), list_bin=1)
     splats = dev(pack_splats(S, radii, A["opacities"]))
     grads = st_.blend_bwd(cam, n, dev(S["ranges"]), dev(S["sorted_ids"]), splats, dev(S["final_T"]),
                           dev(S["final_idx"]), dev(A["v_image"]))

@@ -28,7 +28,7 @@ def _backward_both_ways(oracle, n, W, H, camera, seed):
     # the entry point under test: same arguments, no accumulator
     out = stages._bwd_outputs(n, 16, torch.device(DEV))
     p = lambda x: None if x is None else C.c_void_p(x.data_ptr())
-    rc = lib.dsx_backward_static(cam.ref, n, 16, p(t["means_3d"]), p(scales), p(t["rotations"]), p(st.splats), None,
+    rc = lib.dsx_backward_static(cam.ref, n, st.sorted_ids.numel(), 16, p(t["means_3d"]), p(scales), p(t["rotations"]), p(st.splats), None,
                                  p(st.radii), p(st.lists), p(st.sorted_ids), p(st.final_T), p(st.final_idx),
                                  p(t["v_image"]), p(out["v_mean3d"]), p(out["v_means2d"]), p(out["v_shs"]),
                                  p(out["v_colors"]), p(out["v_opacity"]), p(out["v_scale"]), p(out["v_quat"]),
@@ -66,7 +66,7 @@ def test_backward_static_matches_backward_twice_in_a_row(oracle):
 def test_backward_static_rejects_more_gaussians_than_its_scratch_holds():
     from ds_splat_amd import _native
     lib = _native.load()
-    cam = _native.Camera(64, 64, 0.5, 0.5, 1.0, 3, 3, 8, 8, 8, 8)
+    cam = _native.Camera(64, 64, 0.5, 0.5, 1.0, 3, 3, 8, 8, 8, 8, 0)
     fake = 16
-    rc = lib.dsx_backward_static(C.byref(cam), 524288 + 1, 16, *([fake] * 11), *([None] * 8), None)
+    rc = lib.dsx_backward_static(C.byref(cam), 524288 + 1, 5, 16, *([fake] * 11), *([None] * 8), None)
     assert rc == -6 and b"524288" in lib.dsx_error_string(rc)
