@@ -83,6 +83,7 @@ SIGNATURES["dsx_trace_read"] = (C.c_int, [C.POINTER(TraceEntry), C.c_int])
 SIGNATURES["dsx_set_blend_pixels_per_lane"] = (C.c_int, [C.c_int])
 SIGNATURES["dsx_list_bin"] = (_I32, [_I32, _I32, _I32])
 SIGNATURES["dsx_ranges_count"] = (_I64, [_I32, _I32, _I32])
+SIGNATURES["dsx_sorted_ids_count"] = (_I64, [_I64, _I32, _I32, _I32])
 SIGNATURES["dsx_grads_bytes"] = (C.c_size_t, [_I64])
 
 _lib = None

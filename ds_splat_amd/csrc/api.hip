@@ -151,7 +151,8 @@ extern "C" size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32
     (void)n;
     if(!valid_list_bin(list_bin))
         return 0;
-    return lists_workspace(k < 0 ? 0 : k, list_grid(width, height, list_bin).lists()).bytes;
+    const ListGrid lg = list_grid(width, height, list_bin);
+    return lists_workspace(k < 0 ? 0 : k, lg.lists(), lg.shift != 0).bytes;
 }
 
 extern "C" int32_t dsx_list_bin(int32_t width, int32_t height, int32_t list_bin)
@@ -159,6 +160,13 @@ extern "C" int32_t dsx_list_bin(int32_t width, int32_t height, int32_t list_bin)
     if(!valid_list_bin(list_bin))
         return 0;
     return 1 << list_grid(width < 0 ? 0 : width, height < 0 ? 0 : height, list_bin).shift;
+}
+
+extern "C" int64_t dsx_sorted_ids_count(int64_t k, int32_t width, int32_t height, int32_t list_bin)
+{
+    if(!valid_list_bin(list_bin) || k < 0)
+        return 0;
+    return list_grid(width < 0 ? 0 : width, height < 0 ? 0 : height, list_bin).shift ? 2 * k : k;
 }
 
 extern "C" size_t dsx_grads_bytes(int64_t n)
@@ -398,8 +406,9 @@ extern "C" int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t heigh
         *partition_flag = nullptr;
         if(workspace && k > 0)
         {
-            const int tiles = list_grid(width, height, list_bin).lists();
-            const ListsWorkspace lw = lists_workspace(k, tiles);
+            const ListGrid lg = list_grid(width, height, list_bin);
+            const int tiles = lg.lists();
+            const ListsWorkspace lw = lists_workspace(k, tiles, lg.shift != 0);
             const Sort32Workspace w = sort32_workspace(k, slot_bits(tiles), kListSortTile);
             *partition_flag =
                 reinterpret_cast<const uint32_t*>(static_cast<const char*>(workspace) + lw.sort + w.counters) + w.passes;
@@ -421,7 +430,7 @@ extern "C" int dsx_tile_lists(const dsx_camera* cam, int64_t n, int64_t k, const
     {
         if(!order || !sorted_ids || !workspace)
             return DSX_ERR_BAD_ARG;
-        if(workspace_bytes < lists_workspace(k, list_grid(*cam).lists()).bytes)
+        if(workspace_bytes < lists_workspace(k, list_grid(*cam).lists(), list_grid(*cam).shift != 0).bytes)
             return DSX_ERR_WORKSPACE;
     }
     return launch_tile_lists(*cam, n, k, order, sorted_ids, ranges, workspace, as_stream(stream));
@@ -653,9 +662,9 @@ extern "C" int dsx_forward_core(const float* means3d, const float* shs, const fl
     char* buf2 = nullptr;
     if(rc == DSX_OK)
     {
-        const size_t ws = lists_workspace(k, list_grid(cam).lists()).bytes;
+        const size_t ws = lists_workspace(k, list_grid(cam).lists(), list_grid(cam).shift != 0).bytes;
         const size_t o_ids = align(ws);
-        if(hipMallocAsync(reinterpret_cast<void**>(&buf2), o_ids + (size_t)k * 4 + 256, s) != hipSuccess)
+        if(hipMallocAsync(reinterpret_cast<void**>(&buf2), o_ids + (size_t)dsx_sorted_ids_count(k, image_width, image_height, 0) * 4 + 256, s) != hipSuccess)
             rc = DSX_ERR_RUNTIME;
         else
             rc = dsx_forward_finish(&cam, n, k, reinterpret_cast<float*>(buf + o_splats), buf + o_order,

@@ -118,7 +118,7 @@ struct BinLists
     const int32_t* fine;      // int32[tiles + 1]
     const int32_t* last_tile; // highest occupied tile (-1: none)
     const int32_t* bins;      // int32[bins + 1]
-    int32_t* walk;            // int32[tiles * 8]: per tile and band, (last blended position in the bin list, its index in the tile's list)
+    int32_t* walk;            // int32[tiles * 8]: per tile and band of four rows, where the forward's scan of the bin list stopped and how many of the tile's entries it had met by then
     int shift, nbx, nty;
 };
 
@@ -161,14 +161,16 @@ __device__ __forceinline__ TileSource tile_source(const BinLists& L, int tile, i
     return t;
 }
 
-// does the entry's tile rectangle (recomputed from the splat record exactly as the projection
-// computed it) contain the source tile?
-__device__ __forceinline__ bool entry_in_tile(const TileSource& t, float px, float py, float radius_bits, int ntx, int nty)
+// Every pair of a bin list carries, in the high half of its key word, which tiles of the bin the
+// Gaussian's rectangle covers: bit x for the columns, bit 8 + y for the rows (a rectangle is the
+// product of a column range and a row range).  The two bits of the tile this wavefront takes its
+// entries for; 0 when every entry belongs (the list of negative depths).
+__device__ __forceinline__ uint32_t tile_bits_of(const TileSource& t, int shift)
 {
     if(t.sx < 0)
-        return true;
-    const TileRect r = tile_rect(px, py, __float_as_int(radius_bits), ntx, nty);
-    return t.sx >= r.sx && t.sx < r.ex && t.sy >= r.sy && t.sy < r.ey;
+        return 0u;
+    const int side = (1 << shift) - 1;
+    return (1u << (t.sx & side)) | (256u << (t.sy & side));
 }
 
 // number of set bits of a wavefront mask below this lane
@@ -191,11 +193,19 @@ constexpr int kBwdFourPixelsFrom = 1600;
 // wavefronts per tile, each with one band of four rows and one pixel per lane; a tile's walk is
 // then four times shorter in time, which is what counts when the launch cannot fill the chip.
 constexpr int kFwdBatch = 128; // sorted entries staged in LDS per round (two per lane)
+constexpr int kScanGroups = 4; // groups of 64 positions of a bin's list whose loads are in flight together
 
 // 8 wavefronts per SIMD (at most 64 VGPRs): all tiles of a 1080p image are resident at once
-// kBinned: the entries come out of the list of the tile's bin (BinLists); an entry belongs to the
-// tile if its tile rectangle contains it, and final_idx still receives the reference's index (the
-// tile's range start plus the entry's rank among the tile's own entries).
+// kBinned: the entries come out of the list of the tile's bin (BinLists).  The wavefront first
+// FILTERS the bin's list: 64 positions at a time it reads the pair's id and key word (two coalesced
+// 4-byte loads, the next 64 already in flight), tests the two bits of its tile in the key's mask,
+// and packs the ids of its own entries into a queue in LDS (the staging arrays' memory, which is
+// free between two rounds) until more than 64 are there or the list ends.  Only those are then gathered,
+// tested for reach and staged as with per-tile lists, so a tile pays a dozen instructions per 64
+// entries of its bin's list instead of a gather and a rectangle test per entry; a scene whose
+// pixels do not saturate early, where every tile reads its bin's whole list, costs a few percent
+// more than with per-tile lists instead of twice as much.  final_idx still receives the
+// reference's index: the tile's range start plus the entry's rank among the tile's own entries.
 template <int kFwdPix, bool kBinned>
 __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))) void blend_fwd_kernel(const int32_t* __restrict__ ranges,
                                                              const int32_t* __restrict__ ids,
@@ -213,6 +223,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic a, conic b
     __shared__ float4 s_b[kFwdBatch]; // conic c, opacity, red, green
     __shared__ float s_c[kFwdBatch];  // blue
+    // the queue of the tile's own entries (binned lists) lives in s_a between two rounds: up to 128 ids
+    int* const s_queue = reinterpret_cast<int*>(s_a);
 
     const int lane = threadIdx.x;
     const int tile = kFwdPix == 4 ? blockIdx.x : blockIdx.x >> 2;
@@ -247,8 +259,6 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     }
     start = min(max(start, 0), k);
     end = min(max(end, 0), k);
-    int seen = 0;     // entries of the tile's own list met so far (binned lists)
-    int pos_hi = -1;  // position of the last entry that any pixel blended (binned lists)
 
     // A pixel that has stopped (or lies outside the image) gets NaN as its row coordinate: its
     // exponent is then NaN, the test `power < 0` fails whatever the entry holds, and the loop
@@ -269,55 +279,109 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
         last[p] = 0;
     }
 
-    // the Gaussian ids of a round are fetched one round ahead: the gather of the splat records then
-    // waits for one memory round trip instead of two in a row
+    // per-tile lists: the Gaussian ids of a round are fetched one round ahead: the gather of the
+    // splat records then waits for one memory round trip instead of two in a row
     int g_ahead[kFwdBatch / DSX_WAVE];
-#pragma unroll
-    for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
+    // binned lists: the scan of the bin's list
+    const uint32_t tile_bits = kBinned ? tile_bits_of(src, lists.shift) << 16 : 0u; // (in the key word's high half)
+    const int32_t* const keys = ids + k; // the pairs' key words lie behind the ids (binned lists)
+    int scan = start;  // next position of the bin's list to look at
+    int seen = 0;      // entries of the tile's own list found so far
+    if(!kBinned)
     {
-        const int e = start + h * DSX_WAVE + lane;
-        g_ahead[h] = e < end ? ids[e] : 0;
+#pragma unroll
+        for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
+        {
+            const int e = start + h * DSX_WAVE + lane;
+            g_ahead[h] = e < end ? ids[e] : 0;
+        }
     }
-    for(int b = start; b < end; b += kFwdBatch)
+    int index_base = kBinned ? src.fine_base : start; // what final_idx records for the first entry of the round
+    for(int b = start;; b += kFwdBatch)
     {
         if(alive == 0)
             break;
-        if(kBinned && seen >= src.count) // the bin's list goes on, the tile's own has ended
-            break;
+        int batch; // entries of this round
         __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
+        if(kBinned)
+        {
+            // Another 64 positions are taken only while all of them would still fit the round, and a
+            // tile whose own entries have all been found looks no further.  The loads of four such
+            // groups are issued together (the scan is bound by their latency, not by its dozen
+            // instructions per group); groups that the round has no room for are read again by the next.
+            int count = 0;
+            while(count <= kFwdBatch - DSX_WAVE && scan < end && seen < src.count)
+            {
+                int id[kScanGroups], key[kScanGroups];
+#pragma unroll
+                for(int j = 0; j < kScanGroups; ++j)
+                {
+                    const int e = scan + j * DSX_WAVE + lane;
+                    id[j] = e < end ? ids[e] : 0;
+                    key[j] = e < end ? keys[e] : 0;
+                }
+#pragma unroll
+                for(int j = 0; j < kScanGroups; ++j)
+                {
+                    if(count <= kFwdBatch - DSX_WAVE && scan < end && seen < src.count) // (uniform)
+                    {
+                        const bool member = scan + lane < end && (((uint32_t)key[j]) & tile_bits) == tile_bits;
+                        const uint64_t m = __ballot(member);
+                        if(member)
+                            s_queue[count + bits_below_lane(m)] = id[j];
+                        const int found = __popcll(m);
+                        count += found;
+                        seen += found;
+                        scan += DSX_WAVE;
+                    }
+                }
+            }
+            if(count == 0)
+                break;
+            __syncthreads();
+            batch = count;
+#pragma unroll
+            for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
+                g_ahead[h] = h * DSX_WAVE + lane < batch ? s_queue[h * DSX_WAVE + lane] : 0;
+            __syncthreads(); // the queue has been read: its memory now takes the staged records
+        }
+        else
+        {
+            if(b >= end)
+                break;
+            batch = min(end - b, kFwdBatch);
+        }
         uint64_t todo[kFwdBatch / DSX_WAVE]; // entries of this round that can touch the tile
-        uint64_t members[kFwdBatch / DSX_WAVE]; // entries of this round that belong to the tile (binned lists)
-        int seen_before[kFwdBatch / DSX_WAVE];  // entries of the tile's own list before each half of the round
 #pragma unroll
         for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
         {
             const int slot = h * DSX_WAVE + lane;
-            const int e = b + slot;
             bool useful = false;
-            bool member = false;
             // (an id is taken for what it is only up to the last Gaussian: lists that a failed sort or a
             // caller's mix-up left in disorder then give a wrong image, not a fetch outside the records)
             const int g = (int)min((uint32_t)g_ahead[h], last_id);
-            g_ahead[h] = e + kFwdBatch < end ? ids[e + kFwdBatch] : 0;
-            if(e < end)
+            if(slot < batch)
             {
                 const float4* rec = splats + 3 * (int64_t)g;
                 const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
                 s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
                 s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
-                member = !kBinned || entry_in_tile(src, q0.x, q0.y, q0.w, ntx, lists.nty);
-                useful = member && entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
+                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
             }
             todo[h] = __ballot(useful);
-            if(kBinned)
-            {
-                members[h] = __ballot(member);
-                seen_before[h] = seen;
-                seen += __popcll(members[h]);
-            }
         }
         __syncthreads();
+        if(!kBinned)
+        {
+            // the next round's ids: in flight while this round's entries are blended
+#pragma unroll
+            for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
+            {
+                const int e = b + kFwdBatch + h * DSX_WAVE + lane;
+                g_ahead[h] = e < end ? ids[e] : 0;
+            }
+        }
 #pragma unroll
         for(int h = 0; h < kFwdBatch / DSX_WAVE; ++h)
         {
@@ -332,12 +396,9 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                 const float4 A = s_a[i];
                 const float4 B = s_b[i];
                 const float C = s_c[i];
-                // what final_idx records for this entry: its position in the sorted key array
-                // (binned lists: the tile's range start plus the entry's rank among the tile's own
-                // entries, counted on the scalar unit from the round's membership mask)
-                const int entry_index =
-                    kBinned ? src.fine_base + seen_before[h] + __popcll(members[h] & ((1ull << bit) - 1ull)) : b + i;
-                uint64_t m_applied = 0;
+                // what final_idx records for this entry: its position in the sorted key array (binned
+                // lists: the tile's range start plus the entry's rank among the tile's own entries)
+                const int entry_index = index_base + i;
                 const ExponentX ex = exponent_x(A.z, A.w, pxf - A.x);
 #pragma unroll
                 for(int p = 0; p < kFwdPix; ++p)
@@ -362,13 +423,10 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                     last[p] = apply ? entry_index : last[p];
                     pyf[p] = stop ? __builtin_nanf("") : pyf[p];
                     alive -= __popcll(m_stop);
-                    if(kBinned)
-                        m_applied |= m_pass & ~m_low;
                 }
-                if(kBinned)
-                    pos_hi = m_applied ? b + i : pos_hi; // (scalar unit)
             }
         }
+        index_base += batch;
     }
 
     // A sort pass that gave up waiting on its predecessor (bounded wait, never seen to happen)
@@ -395,26 +453,18 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
     }
     if(kBinned && layout_ok)
     {
-        // for the backward: where this wavefront's walk ended, as a position in the bin's list and
-        // as an index in the sorted key array (-1, -1 if it blended nothing).  The four-pixel form
-        // speaks for the whole tile and marks the other three bands as empty.
-        int top = -1;
-#pragma unroll
-        for(int p = 0; p < kFwdPix; ++p)
-            top = max(top, last[p]);
-#pragma unroll
-        for(int o = 32; o > 0; o >>= 1)
-            top = max(top, __shfl_xor(top, o, DSX_WAVE));
-        if(pos_hi < 0)
-            top = -1;
+        // for the backward: where this wavefront's scan of the bin's list stopped and how many of the
+        // tile's entries it had met by then (everything that any of its pixels blended lies below).
+        // The four-pixel form speaks for the whole tile and marks the other three bands as empty.
         int32_t* w = lists.walk + (int64_t)tile * 8;
+        const int stopped = min(scan, end);
         if(kFwdPix == 4)
         {
             if(lane < 8)
-                w[lane] = lane == 0 ? pos_hi : (lane == 1 ? top : -1);
+                w[lane] = lane == 0 ? stopped : (lane == 1 ? seen : (lane & 1 ? 0 : -1));
         }
         else if(lane < 2)
-            w[2 * band + lane] = lane == 0 ? pos_hi : top;
+            w[2 * band + lane] = lane == 0 ? stopped : seen;
     }
     // A side job for the memory system, which this kernel leaves idle: every wavefront prepares
     // its share of the backward's gradient accumulator, twelve floats per Gaussian: the nine sums
@@ -587,9 +637,10 @@ constexpr int kBwdBatch = 128; // sorted entries staged in LDS per round (two pe
 // (tile, entry).  Compared with four wavefronts of one pixel per lane this does one
 // cross-lane reduction per entry instead of four and needs no LDS accumulators or barriers.
 // (kBwdPix = 1: four wavefronts per tile with one band of four rows each, as in the forward)
-// kBinned: the entries come out of the list of the tile's bin; the forward left, per tile and band,
-// the bin-list position where its walk ended and that entry's index in the sorted key array, from
-// which every entry met on the way down gets its own index (final_idx is compared with those).
+// kBinned: the entries come out of the list of the tile's bin, filtered into a queue as in the forward
+// but downwards; the forward left, per tile and band, the bin-list position where its scan stopped and
+// the number of the tile's entries it had met by then, from which every entry met on the way down
+// gets its index in the sorted key array (final_idx is compared with those).
 template <int kBwdPix, bool kBinned>
 __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const int32_t* __restrict__ ranges, const int32_t* __restrict__ ids, const float4* __restrict__ splats,
@@ -601,6 +652,8 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     __shared__ float4 s_b[kBwdBatch]; // conic c, opacity, red, green
     __shared__ float s_c[kBwdBatch];  // blue
     __shared__ int s_id[kBwdBatch];
+    // the queue of the tile's own entries (binned lists) lives in s_a between two rounds, as in the forward
+    int* const s_queue = reinterpret_cast<int*>(s_a);
 
     const int lane = threadIdx.x;
     const int tile = kBwdPix == 4 ? blockIdx.x : blockIdx.x >> 2;
@@ -638,63 +691,123 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
         m = max(m, bin_final[p]);
     }
 
+    // last entry (as an index in the sorted key array) that any pixel of this wavefront blended
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1)
+        m = max(m, __shfl_xor(m, o, DSX_WAVE));
+
     // lists that were built for another bin size than this launch assumes are not read (see the forward)
     const bool layout_ok = header == nullptr || *header == header_shift;
     int start = 0, hi = -1;
     TileSource src = {};
-    int index_hi = 0; // index (in the sorted key array) of the entry at position hi (binned lists)
-    int above = 0;    // entries of the tile's own list met so far, from the top (binned lists)
+    // binned lists: the scan of the bin's list, downwards from where the forward's scan stopped
+    uint32_t my_bits = 0u; // the two bits of this wavefront's tile in a pair's key word (high half)
+    int pos = -1;       // next position of the bin's list to look at
+    int rank_next = -1; // rank, in the tile's own list, of the next of its entries to be found
+    int idx_next = 0;   // index (in the sorted key array) of the next entry that is handed to the blend
     if(kBinned && layout_ok)
     {
-        // the forward's walk of this tile ended at position hi of the bin's list, on the entry
-        // with index index_hi (the larger of the four bands' figures: both grow together)
+        // The forward's scan of the bin's list stopped at position w[0] after meeting w[1] of the
+        // tile's entries (the larger of the four bands' figures: both grow together); everything
+        // that was blended lies below, and the entries are taken from there downwards.  An entry's
+        // index is the tile's range start plus its rank; those above the last blended one (m) are
+        // not even queued, so the entries that are handed on have consecutive indices.
         src = tile_source(lists, tile, ntx);
-        start = src.start;
+        my_bits = tile_bits_of(src, lists.shift) << 16;
+        start = max(src.start, 0);
         const int32_t* w = lists.walk + (int64_t)tile * 8;
-        hi = max(max(w[0], w[2]), max(w[4], w[6]));
-        index_hi = max(max(w[1], w[3]), max(w[5], w[7]));
-        if(src.count <= 0)
-            hi = -1;
-        hi = min(hi, k - 1); // (positions outside sorted_ids are not followed, as in the forward)
-        start = max(start, 0);
+        const int stopped = max(max(w[0], w[2]), max(w[4], w[6]));
+        const int seen = max(max(w[1], w[3]), max(w[5], w[7]));
+        // (positions outside sorted_ids are not followed, as in the forward)
+        pos = min(stopped, min(src.end, k)) - 1;
+        rank_next = min(seen, src.count) - 1;
+        idx_next = min(m, src.fine_base + rank_next);
+        if(src.count <= 0 || idx_next < src.fine_base) // nothing of this tile was blended
+            pos = start - 1;
     }
     else if(layout_ok)
     {
         start = max(ranges[tile], 0);
         const int end = min(ranges[tile + 1], k);
-        // last entry any pixel of this tile blended
-#pragma unroll
-        for(int o = 32; o > 0; o >>= 1)
-            m = max(m, __shfl_xor(m, o, DSX_WAVE));
         hi = min(end - 1, m);
     }
 
-    // (ids one round ahead, as in the forward)
     int g_ahead[kBwdBatch / DSX_WAVE];
+    const int32_t* const keys = ids + k; // the pairs' key words lie behind the ids (binned lists)
+    if(!kBinned)
+    {
+        // (ids one round ahead, as in the forward)
 #pragma unroll
-    for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
-    {
-        const int e = hi - (h * DSX_WAVE + lane);
-        g_ahead[h] = e >= start ? ids[e] : 0;
+        for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
+        {
+            const int e = hi - (h * DSX_WAVE + lane);
+            g_ahead[h] = e >= start ? ids[e] : 0;
+        }
     }
-    for(int top = hi; top >= start; top -= kBwdBatch)
+    for(int top = hi;; top -= kBwdBatch)
     {
-        if(kBinned && index_hi - above < src.fine_base) // every entry of the tile's own list has been met
-            break;
+        int batch;     // entries of this round
+        int idx_first; // index (in the sorted key array) of the round's first entry; the others follow downwards
         __syncthreads(); // single wavefront: orders the LDS reads of the last round before these writes
+        if(kBinned)
+        {
+            // (four groups of 64 positions in flight at a time, as in the forward)
+            int count = 0;
+            while(count <= kBwdBatch - DSX_WAVE && pos >= start && rank_next >= 0)
+            {
+                int id[kScanGroups], key[kScanGroups];
+#pragma unroll
+                for(int j = 0; j < kScanGroups; ++j)
+                {
+                    const int e = pos - j * DSX_WAVE - lane;
+                    id[j] = e >= start ? ids[e] : 0;
+                    key[j] = e >= start ? keys[e] : 0;
+                }
+#pragma unroll
+                for(int j = 0; j < kScanGroups; ++j)
+                {
+                    if(count <= kBwdBatch - DSX_WAVE && pos >= start && rank_next >= 0) // (uniform)
+                    {
+                        const bool member = pos - lane >= start && (((uint32_t)key[j]) & my_bits) == my_bits;
+                        const uint64_t mm = __ballot(member);
+                        // lower lanes hold higher positions: this entry's rank is the next one less the members before it
+                        const int rank = rank_next - bits_below_lane(mm);
+                        const bool keep = member && src.fine_base + rank <= m;
+                        const uint64_t mk = __ballot(keep);
+                        if(keep)
+                            s_queue[count + bits_below_lane(mk)] = id[j];
+                        count += __popcll(mk);
+                        rank_next -= __popcll(mm);
+                        pos -= DSX_WAVE;
+                    }
+                }
+            }
+            if(count == 0)
+                break;
+            __syncthreads();
+            batch = count;
+#pragma unroll
+            for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
+                g_ahead[h] = h * DSX_WAVE + lane < batch ? s_queue[h * DSX_WAVE + lane] : 0;
+            __syncthreads(); // the queue has been read: its memory now takes the staged records
+            idx_first = idx_next;
+            idx_next -= batch;
+        }
+        else
+        {
+            if(top < start)
+                break;
+            batch = min(top - start + 1, kBwdBatch);
+            idx_first = top;
+        }
         uint64_t todo[kBwdBatch / DSX_WAVE]; // entries of this round that can touch the tile
-        uint64_t members[kBwdBatch / DSX_WAVE]; // entries of this round that belong to the tile (binned lists)
-        int above_before[kBwdBatch / DSX_WAVE]; // entries of the tile's own list above each half of the round
 #pragma unroll
         for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
         {
             const int slot = h * DSX_WAVE + lane;
-            const int e = top - slot;
             bool useful = false;
-            bool member = false;
             const int g = (int)min((uint32_t)g_ahead[h], last_id); // (as in the forward)
-            g_ahead[h] = e - kBwdBatch >= start ? ids[e - kBwdBatch] : 0;
-            if(e >= start)
+            if(slot < batch)
             {
                 const float4* rec = splats + 3 * (int64_t)g;
                 const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
@@ -702,28 +815,28 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
                 s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
                 s_id[slot] = g;
-                member = !kBinned || entry_in_tile(src, q0.x, q0.y, q0.w, ntx, lists.nty);
-                useful = member && entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
+                useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
             }
             todo[h] = __ballot(useful);
-            if(kBinned)
-            {
-                members[h] = __ballot(member);
-                above_before[h] = above;
-                above += __popcll(members[h]);
-            }
         }
         __syncthreads();
+        if(!kBinned)
+        {
+            // the next round's ids: in flight while this round's entries are blended
+#pragma unroll
+            for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
+            {
+                const int e = top - kBwdBatch - (h * DSX_WAVE + lane);
+                g_ahead[h] = e >= start ? ids[e] : 0;
+            }
+        }
 #pragma unroll
         for(int h = 0; h < kBwdBatch / DSX_WAVE; ++h)
         for(uint64_t mask = todo[h]; mask != 0; mask &= mask - 1)
         {
             const int bit = __builtin_ctzll(mask);
             const int t = h * DSX_WAVE + bit;
-            // binned lists: lower slots are higher positions, so the entry's index is the top one's
-            // less the tile's entries met above it (scalar unit)
-            const int idx =
-                kBinned ? index_hi - above_before[h] - __popcll(members[h] & ((1ull << bit) - 1ull)) : top - t;
+            const int idx = idx_first - t; // the entry's index in the sorted key array (scalar unit)
             const float4 A = s_a[t];
             const float4 B = s_b[t];
             // the exponent exactly as the forward computed it (pixel - mean); sigma = -exponent

@@ -264,14 +264,15 @@ OrderLayout order_layout(int64_t n, int image_width = 0, int image_height = 0, i
 // Workspace of the tile lists for k keys.
 struct ListsWorkspace
 {
-    size_t slots_a; // uint32[k]
-    size_t slots_b; // uint32[k]
+    size_t slots_a; // uint16 / uint32[k]
+    size_t slots_b; // the same (per-tile lists only)
     size_t ids_alt; // int32[k]
     size_t sort;    // Sort32Workspace
     size_t bytes;
     int passes;
 };
-ListsWorkspace lists_workspace(int64_t k, int num_tiles);
+// binned: lists per bin (32-bit slot words that carry the tile masks and end in the caller's buffer)
+ListsWorkspace lists_workspace(int64_t k, int num_tiles, bool binned);
 
 // launchers (each returns a dsx_status)
 int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_a, uint32_t* keys_b,

@@ -1212,7 +1212,13 @@ constexpr int kEmitWindows = DSX_EMIT_WINDOWS; // windows of 256 outputs per rou
 constexpr int kEmitChunkMax = 4096;            // outputs per workgroup: at most this many ...
 constexpr int kEmitWorkgroups = 4096;          // ... and fewer when that leaves less than this many workgroups
 
-template <typename SlotT>
+// kMasks (lists per bin, SlotT = uint32_t): the high half of a pair's slot word says which tiles of the
+// bin the Gaussian's rectangle covers, bit x for the columns and bit 8 + y for the rows of the bin
+// (a rectangle is the product of a column range and a row range).  The partition sorts by the low bits
+// only and carries the rest along; the blend kernels pick a tile's entries out of its bin's list by
+// testing the tile's two bits.  Pairs of negative depth (slot 0, one list for the whole image) carry
+// all sixteen bits.
+template <typename SlotT, bool kMasks>
 __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t* __restrict__ order,
                                                                   const uint2* __restrict__ rects_sorted,
                                                                   const uint32_t* __restrict__ block_offsets,
@@ -1227,6 +1233,7 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
     // per Gaussian of the block: x = first output, y = slot of the rectangle's first tile (0 for
     // negative depths), z = width (0 marks a negative depth: every pair goes to slot 0), w = id
     __shared__ uint4 s_rec[kProjBlock];
+    __shared__ uint2 s_rect[kMasks ? kProjBlock : 1]; // the tile rectangles themselves (for the masks)
     __shared__ __attribute__((aligned(16))) uint32_t wave_tot[kProjBlock / DSX_WAVE];
     __shared__ uint32_t s_mark[kEmitWindows * kProjBlock];
     __shared__ __attribute__((aligned(16))) uint32_t s_wave_max[kEmitWindows][kProjBlock / DSX_WAVE];
@@ -1297,6 +1304,8 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
             rec.y = negative ? 0u : first_y * (uint32_t)ntx + first_x + 1u;
             rec.z = negative ? 0u : w;
             rec.w = g;
+            if(kMasks)
+                s_rect[tid] = r;
         }
         const uint32_t incl = wave_incl_scan32(count, lane);
         if(lane == 63)
@@ -1368,7 +1377,7 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
                     const uint4 own = s_rec[owner]; // one 16-byte LDS read per output
                     const uint32_t r = j - own.x;
                     const uint32_t w = own.z;
-                    uint32_t slot = 0;
+                    uint32_t slot = kMasks ? 0xffff0000u : 0u;
                     if(w)
                     {
                         // r / w by a float reciprocal (r < 2^24 tiles per Gaussian), corrected by one step
@@ -1379,6 +1388,21 @@ __global__ __launch_bounds__(kProjBlock) void emit_ordered_kernel(const uint32_t
                             ++ry;
                         const uint32_t rx = r - ry * w;
                         slot = own.y + ry * (uint32_t)ntx + rx;
+                        if(kMasks)
+                        {
+                            // the rectangle's columns and rows inside this bin, as bit ranges [lo, hi]
+                            const uint2 tr = s_rect[owner];
+                            const int side = 1 << shift;
+                            const int tsx = (int)(tr.x & 0xffffu), tsy = (int)(tr.x >> 16);
+                            const int tw = (int)(tr.y & 0xffffu), th = (int)((tr.y >> 16) & 0x7fffu);
+                            const int x0 = (int)(((uint32_t)tsx >> shift) + rx) << shift; // the bin's first column
+                            const int y0 = (int)(((uint32_t)tsy >> shift) + ry) << shift;
+                            const int xlo = max(tsx - x0, 0), xhi = min(tsx + tw - 1 - x0, side - 1);
+                            const int ylo = max(tsy - y0, 0), yhi = min(tsy + th - 1 - y0, side - 1);
+                            const uint32_t xm = ((2u << xhi) - 1u) & ~((1u << xlo) - 1u);
+                            const uint32_t ym = ((2u << yhi) - 1u) & ~((1u << ylo) - 1u);
+                            slot |= (xm | (ym << 8)) << 16;
+                        }
                     }
                     slots[base + j] = (SlotT)slot;
                     ids[base + j] = (int32_t)own.w;
@@ -1397,17 +1421,19 @@ static bool slots_are_u16(int num_tiles)
     return num_tiles + 1 <= 65535;
 }
 
-ListsWorkspace lists_workspace(int64_t k, int num_tiles)
+// binned: the slot words are 32 bits (slot in the low half, the tile mask in the high half) and the
+// sorted ones end in the caller's buffer, behind the ids
+ListsWorkspace lists_workspace(int64_t k, int num_tiles, bool binned)
 {
     auto align = [](size_t x) { return (x + 255) & ~(size_t)255; };
     ListsWorkspace w;
-    const size_t slot_bytes = slots_are_u16(num_tiles) ? 2 : 4;
+    const size_t slot_bytes = (binned || !slots_are_u16(num_tiles)) ? 4 : 2;
     w.passes = digits32(slot_bits(num_tiles)).passes;
     size_t off = 0;
     w.slots_a = off;
     off = align(off + (size_t)k * slot_bytes);
     w.slots_b = off;
-    off = align(off + (size_t)k * slot_bytes);
+    off = align(off + (binned ? 0 : (size_t)k * slot_bytes));
     w.ids_alt = off;
     off = align(off + (size_t)k * 4);
     w.sort = off;
@@ -1416,8 +1442,8 @@ ListsWorkspace lists_workspace(int64_t k, int num_tiles)
     return w;
 }
 
-// num_tiles: lists that the pairs are partitioned into (tiles, or bins when the lists are binned)
-template <typename SlotT>
+// num_tiles: lists that the pairs are partitioned into (tiles, or bins when the lists are binned: kMasks)
+template <typename SlotT, bool kMasks>
 static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_tiles, const void* order,
                            int32_t* sorted_ids, int32_t* ranges, void* workspace, hipStream_t stream)
 {
@@ -1437,17 +1463,20 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
             rc = launch_fill_u32(reinterpret_cast<uint32_t*>(ranges) + rl.last_tile, 1, 0xffffffffu, stream);
         return rc;
     }
-    const ListsWorkspace w = lists_workspace(k, num_tiles);
+    const ListsWorkspace w = lists_workspace(k, num_tiles, kMasks);
     const int bits = slot_bits(num_tiles);
     char* base = static_cast<char*>(workspace);
-    SlotT* slots_a = reinterpret_cast<SlotT*>(base + w.slots_a);
-    SlotT* slots_b = reinterpret_cast<SlotT*>(base + w.slots_b);
     uint32_t* ids_final = reinterpret_cast<uint32_t*>(sorted_ids);
     uint32_t* ids_other = reinterpret_cast<uint32_t*>(base + w.ids_alt);
-    // ping-pong parity: start so that the last pass lands the ids in the caller's buffer
+    // ping-pong parity: start so that the last pass lands the ids in the caller's buffer (and, for
+    // binned lists, the slot words with their masks right behind them)
     const bool even = (w.passes % 2) == 0;
     uint32_t* vals_a = even ? ids_final : ids_other;
     uint32_t* vals_b = even ? ids_other : ids_final;
+    SlotT* slots_final = kMasks ? reinterpret_cast<SlotT*>(ids_final + k) : reinterpret_cast<SlotT*>(base + w.slots_b);
+    SlotT* slots_other = reinterpret_cast<SlotT*>(base + w.slots_a);
+    SlotT* slots_a = (kMasks && even) ? slots_final : slots_other;
+    SlotT* slots_b = (kMasks && even) ? slots_other : slots_final;
     int rc = DSX_OK;
     const Sort32Workspace sw = sort32_workspace(k, bits, kListSortTile);
     {
@@ -1455,8 +1484,8 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
         // outputs per workgroup: a multiple of 256 between 256 and kEmitChunkMax
         const int64_t want = (k + kEmitWorkgroups - 1) / kEmitWorkgroups;
         const int chunk = (int)min((int64_t)kEmitChunkMax, ((want + kProjBlock - 1) / kProjBlock) * kProjBlock);
-        hipLaunchKernelGGL(emit_ordered_kernel<SlotT>, dim3((unsigned)((k + chunk - 1) / chunk)), dim3(kProjBlock),
-                           0, stream, reinterpret_cast<const uint32_t*>(obase + o.ids_a),
+        hipLaunchKernelGGL((emit_ordered_kernel<SlotT, kMasks>), dim3((unsigned)((k + chunk - 1) / chunk)),
+                           dim3(kProjBlock), 0, stream, reinterpret_cast<const uint32_t*>(obase + o.ids_a),
                            reinterpret_cast<const uint2*>(obase + o.rects_sorted),
                            reinterpret_cast<const uint32_t*>(obase + o.block_sums), n, k,
                            lg.shift ? lg.nbx : lg.ntx, lg.shift, slots_a, reinterpret_cast<int32_t*>(vals_a),
@@ -1466,13 +1495,17 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
     DSX_LAUNCH_CHECK();
     SlotT* ko;
     uint32_t* vo;
-    // the sorted slots themselves are not needed: the ranges are known already
-    rc = sort32_passes<SlotT, kListSortThreads, kListSortItems>(k, bits, slots_a, vals_a, slots_b, vals_b, false, false,
-                                                                base + w.sort, "onesweep32_kernel<tile partition>",
-                                                                stream, &ko, &vo, nullptr, nullptr,
+    // per-tile lists: the sorted slots themselves are not needed (the ranges are known already);
+    // binned lists: they are kept for their masks
+    rc = sort32_passes<SlotT, kListSortThreads, kListSortItems>(k, bits, slots_a, vals_a, slots_b, vals_b, false,
+                                                                kMasks, base + w.sort,
+                                                                "onesweep32_kernel<tile partition>", stream, &ko, &vo,
+                                                                nullptr, nullptr,
                                                                 reinterpret_cast<const uint32_t*>(obase + o.slot_hist));
     if(rc)
         return rc;
+    if(kMasks && ko != slots_final)
+        return DSX_ERR_RUNTIME;
     return vo == ids_final ? DSX_OK : DSX_ERR_RUNTIME;
 }
 
@@ -1482,14 +1515,21 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
 int launch_tile_lists(const dsx_camera& cam, int64_t n, int64_t k, const void* order, int32_t* sorted_ids,
                       int32_t* ranges, void* workspace, hipStream_t stream)
 {
-    const int num_tiles = list_grid(cam).lists();
+    const ListGrid lg = list_grid(cam);
+    const int num_tiles = lg.lists();
     if(k >= (1ll << 30))
         return DSX_ERR_TOO_LARGE;
     if(n <= 0)
         k = 0;
+    if(lg.shift)
+    {
+        if(num_tiles + 1 > 65535) // (the slot shares its word with the 16-bit mask)
+            return DSX_ERR_TOO_LARGE;
+        return tile_lists_impl<uint32_t, true>(cam, n, k, num_tiles, order, sorted_ids, ranges, workspace, stream);
+    }
     if(slots_are_u16(num_tiles))
-        return tile_lists_impl<uint16_t>(cam, n, k, num_tiles, order, sorted_ids, ranges, workspace, stream);
-    return tile_lists_impl<uint32_t>(cam, n, k, num_tiles, order, sorted_ids, ranges, workspace, stream);
+        return tile_lists_impl<uint16_t, false>(cam, n, k, num_tiles, order, sorted_ids, ranges, workspace, stream);
+    return tile_lists_impl<uint32_t, false>(cam, n, k, num_tiles, order, sorted_ids, ranges, workspace, stream);
 }
 
 } // namespace dsx

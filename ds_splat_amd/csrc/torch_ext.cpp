@@ -74,7 +74,7 @@ at::Tensor& pinned_key_count()
 
 // list_bin: tiles per side of the bins that the tile lists are built for (0: the library's choice);
 // the backward of this forward must be given the same value.
-// image[H,W,3], radii[N], splats[N,12], sorted_ids[K], ranges[dsx_ranges_count], final_T[H,W], final_idx[H,W]
+// image[H,W,3], radii[N], splats[N,12], sorted_ids[dsx_sorted_ids_count(K)], ranges[dsx_ranges_count], final_T[H,W], final_idx[H,W]
 // (the 3-D covariances are not kept: the backward rebuilds them from scales and rotations, or
 // reads cov3d_precomp) and, when prepare_backward is set, the backward's gradient accumulator
 // (dsx_grads_bytes(N) bytes as float32), which the blend kernel prepares on the side: sums zeroed,
@@ -110,7 +110,7 @@ std::vector<at::Tensor> forward(int64_t height, int64_t width, double tanfovx, d
                               splats.data_ptr<float>(), radii.data_ptr<int32_t>(), nullptr, bs, order.data_ptr(),
                               order_bytes, k_host.data_ptr<int64_t>(), s));
     const int64_t k = *k_host.data_ptr<int64_t>();
-    at::Tensor sorted_ids = at::empty({k}, i32);
+    at::Tensor sorted_ids = at::empty({dsx_sorted_ids_count(k, (int32_t)width, (int32_t)height, cam.c.list_bin)}, i32);
     at::Tensor ranges = at::empty({dsx_ranges_count((int32_t)width, (int32_t)height, cam.c.list_bin)}, i32);
     at::Tensor image = at::empty({height, width, 3}, f32);
     at::Tensor final_T = at::empty({height, width}, f32);
@@ -154,6 +154,10 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
                 "ranges does not have the layout of this image size and bin size (the backward must be given the "
                 "list_bin of its forward)");
     TORCH_CHECK(sorted_ids.is_contiguous() && sorted_ids.scalar_type() == at::kInt, "sorted_ids must be int32");
+    // pairs in sorted_ids: the buffer holds k ids and, for lists per bin, k more words
+    const int64_t words_per_pair = dsx_sorted_ids_count(1, (int32_t)width, (int32_t)height, cam.c.list_bin);
+    TORCH_CHECK(words_per_pair > 0 && sorted_ids.numel() % words_per_pair == 0, "sorted_ids has the wrong size");
+    const int64_t k = sorted_ids.numel() / words_per_pair;
     auto out = [&](int bit, std::initializer_list<int64_t> shape) {
         return (wanted >> bit) & 1 ? at::empty(shape, f32) : at::Tensor();
     };
@@ -172,7 +176,7 @@ std::vector<at::Tensor> backward(int64_t height, int64_t width, double tanfovx, 
                         prepared_grads->numel() == (int64_t)(dsx_grads_bytes(n) / 4) && prepared_grads->device() == dev,
                     "prepared_grads must be the float32 accumulator of this forward (dsx_grads_bytes(N) bytes)");
     at::Tensor grads = prepared ? *prepared_grads : at::empty({(int64_t)(dsx_grads_bytes(n) / 4)}, f32);
-    check(dsx_backward(&cam.c, n, sorted_ids.numel(), (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales),
+    check(dsx_backward(&cam.c, n, k, (int32_t)num_bases, means3d.data_ptr<float>(), fptr(scales),
                        fptr(quats),
                        splats.data_ptr<float>(), fptr(cov3d_precomp), radii.data_ptr<int32_t>(),
                        ranges.data_ptr<int32_t>(), sorted_ids.numel() ? sorted_ids.data_ptr<int32_t>() : nullptr,

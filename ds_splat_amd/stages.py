@@ -162,12 +162,14 @@ def tile_lists(cam, n, k, order, return_flags=False, return_lists=False):
     `ranges` buffer (see split_lists) instead of its first T+1 words."""
     lib = N.load()
     dev = order.device
-    sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
+    sorted_ids = new_sorted_ids(cam, k, dev)
     lists = torch.empty((int(lib.dsx_ranges_count(cam.width, cam.height, cam.list_bin)),), dtype=torch.int32, device=dev)
     nbytes = int(lib.dsx_workspace_bytes(n, k, cam.width, cam.height, cam.list_bin))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=dev)
     N.check(lib.dsx_tile_lists(cam.ref, n, k, _ptr(order), _ptr(sorted_ids), _ptr(lists), _ptr(ws), nbytes, _stream()))
     ranges = lists if return_lists else lists[:cam.num_tiles + 1]
+    if not return_lists:
+        sorted_ids = sorted_ids[:k]      # the ids alone (binned lists carry a word of tile masks per pair behind them)
     if not return_flags:
         return sorted_ids, ranges
     p_a, p_b = C.c_void_p(), C.c_void_p()
@@ -176,6 +178,12 @@ def tile_lists(cam, n, k, order, return_flags=False, return_lists=False):
     torch.cuda.synchronize()
     read = lambda t, p: 0 if not p.value else int(t.view(torch.int32)[(p.value - t.data_ptr()) // 4].item())
     return sorted_ids, ranges, (read(order, p_a), read(ws, p_b))
+
+
+def new_sorted_ids(cam, k, device):
+    """The `sorted_ids` buffer for k pairs: k ids and, for binned lists, k more words (the pairs' tile masks)."""
+    words = int(N.load().dsx_sorted_ids_count(k, cam.width, cam.height, cam.list_bin))
+    return torch.empty((words,), dtype=torch.int32, device=device)
 
 
 def sort_pairs_u32(keys, values, key_bits=32):
@@ -221,11 +229,16 @@ def tile_ranges(sorted_keys, num_tiles):
     return ranges
 
 
+def _pairs_in(cam, sorted_ids):
+    """number of pairs k that a `sorted_ids` buffer of this camera's bin size holds"""
+    return sorted_ids.numel() // (2 if list_bin(cam) > 1 else 1)
+
+
 def blend_fwd(cam, ranges, sorted_ids, splats):
-    """ranges: the whole `ranges` buffer of tile_lists(..., return_lists=True) for this camera's bin size,
-    or, for per-tile lists, any tensor that starts with the T + 1 per-tile ranges."""
+    """ranges, sorted_ids: the whole buffers of tile_lists(..., return_lists=True) for this camera's bin size,
+    or, for per-tile lists, any tensor that starts with the T + 1 per-tile ranges and the ids."""
     lib = N.load()
-    n, k = splats.shape[0], sorted_ids.numel()
+    n, k = splats.shape[0], _pairs_in(cam, sorted_ids)
     dev = ranges.device
     image = torch.empty((cam.height, cam.width, 3), dtype=torch.float32, device=dev)
     final_T = torch.empty((cam.height, cam.width), dtype=torch.float32, device=dev)
@@ -238,7 +251,7 @@ def blend_fwd(cam, ranges, sorted_ids, splats):
 def blend_bwd(cam, n, ranges, sorted_ids, splats, final_T, final_idx, v_image):
     lib = N.load()
     grads = torch.empty((n, N.GRAD_FLOATS), dtype=torch.float32, device=splats.device)
-    N.check(lib.dsx_blend_bwd(cam.ref, n, sorted_ids.numel(), _ptr(ranges), _ptr(sorted_ids), _ptr(splats),
+    N.check(lib.dsx_blend_bwd(cam.ref, n, _pairs_in(cam, sorted_ids), _ptr(ranges), _ptr(sorted_ids), _ptr(splats),
                               _ptr(final_T), _ptr(final_idx), _ptr(v_image), _ptr(grads), _stream()))
     return grads
 
@@ -288,8 +301,8 @@ def _pinned_i64():
 class ForwardState:
     """What the forward keeps for the backward (the reference saves the analogous tensors
     on the autograd context, ds_splat/rasterizer.py:47-64)."""
-    __slots__ = ("splats", "radii", "cov3d", "sorted_ids", "lists", "ranges", "final_T", "final_idx", "num_keys",
-                 "num_keys_per_tile", "list_bin", "grads")
+    __slots__ = ("splats", "radii", "cov3d", "sorted_ids", "ids", "lists", "ranges", "final_T", "final_idx",
+                 "num_keys", "num_keys_per_tile", "list_bin", "grads")
 
 
 def sort_flag_indices(cam, n, k, order, workspace):
@@ -331,7 +344,9 @@ def forward(cam, means3d, scales, quats, opacities, shs, cov3d_precomp=None, col
     st.list_bin = cam.list_bin
     if after_project is not None:
         after_project(order, n, k)
-    st.sorted_ids = torch.empty((k,), dtype=torch.int32, device=dev)
+    # (binned lists: k ids and, behind them, k words of tile masks; st.ids is the ids alone)
+    st.sorted_ids = new_sorted_ids(cam, k, dev)
+    st.ids = st.sorted_ids[:k]
     # the whole `ranges` buffer, and its first T+1 words: the per-tile ranges as the reference defines them
     st.lists = torch.empty((int(lib.dsx_ranges_count(cam.width, cam.height, cam.list_bin)),), dtype=torch.int32, device=dev)
     st.ranges = st.lists[:cam.num_tiles + 1]
@@ -359,7 +374,7 @@ def backward(cam, st, num_bases, means3d, scales, quats, v_image):
     prepared = getattr(st, "grads", None) is not None
     grads = st.grads if prepared else new_accumulator(n, dev)
     st.grads = None
-    N.check(lib.dsx_backward(cam.ref, n, st.sorted_ids.numel(), num_bases, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(st.splats),
+    N.check(lib.dsx_backward(cam.ref, n, _pairs_in(cam, st.sorted_ids), num_bases, _ptr(means3d), _ptr(scales), _ptr(quats), _ptr(st.splats),
                              _ptr(st.cov3d), _ptr(st.radii), _ptr(st.lists), _ptr(st.sorted_ids), _ptr(st.final_T),
                              _ptr(st.final_idx), _ptr(v_image), _ptr(grads), int(prepared), _ptr(o["v_mean3d"]),
                              _ptr(o["v_means2d"]), _ptr(o["v_shs"]), _ptr(o["v_colors"]), _ptr(o["v_opacity"]),

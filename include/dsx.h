@@ -121,6 +121,11 @@ int32_t dsx_sort_passes(int32_t num_tiles);
  * leaves for the backward.  No counterpart in the reference. */
 int32_t dsx_list_bin(int32_t width, int32_t height, int32_t list_bin);
 int64_t dsx_ranges_count(int32_t width, int32_t height, int32_t list_bin);
+/* int32 words of the `sorted_ids` buffer for k pairs: k ids and, for b > 1, behind them one word per
+ * pair whose high half says which tiles of the bin the pair's Gaussian covers (the blend kernels pick
+ * a tile's entries out of its bin's list by it): 2 k words.  Wherever this header says sorted_ids[k],
+ * the buffer has this many words and k is still the number of pairs. */
+int64_t dsx_sorted_ids_count(int64_t k, int32_t width, int32_t height, int32_t list_bin);
 /* bytes of `workspace` dsx_forward_finish / dsx_tile_lists need for k keys */
 size_t dsx_workspace_bytes(int64_t n, int64_t k, int32_t width, int32_t height, int32_t list_bin);
 /* bytes of `workspace` dsx_sort_pairs needs for k keys, and dsx_sort_pairs_u32 for count pairs */

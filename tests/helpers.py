@@ -153,9 +153,11 @@ def tile_rects(S, radii, width, height):
 
 def expected_bin_lists(S, radii, width, height, bin_side):
     """What binned tile lists must hold, from the oracle's stage-1 results: (ids, bin_ranges,
-    last_tile).  Slot 0 (positions [0, bin_ranges[0])) is the oracle's own list of pairs with a
+    last_tile, masks).  Slot 0 (positions [0, bin_ranges[0])) is the oracle's own list of pairs with a
     negative depth; the list of a bin holds every Gaussian of non-negative depth (the last Gaussian
-    excepted: it never emits) whose tile rectangle touches the bin, once, by (depth bits, index)."""
+    excepted: it never emits) whose tile rectangle touches the bin, once, by (depth bits, index).
+    masks: per pair, which tiles of the bin the Gaussian's rectangle covers: bit x for the bin's columns,
+    bit 8 + y for its rows; all sixteen bits for the pairs of slot 0."""
     n = len(radii)
     ntx, nty = (width + 15) // 16, (height + 15) // 16
     nbx, nby = (ntx + bin_side - 1) // bin_side, (nty + bin_side - 1) // bin_side
@@ -170,14 +172,21 @@ def expected_bin_lists(S, radii, width, height, bin_side):
     order = np.lexsort((np.arange(n), bits))                # by depth bits, then index
     order = order[pos[order]]
     per_bin = [[] for _ in range(nbx * nby)]
+    per_bin_masks = [[] for _ in range(nbx * nby)]
     for g in order.tolist():
         for by in range(sy[g] // bin_side, (ey[g] - 1) // bin_side + 1):
             for bx in range(sx[g] // bin_side, (ex[g] - 1) // bin_side + 1):
                 per_bin[by * nbx + bx].append(g)
+                xm = sum(1 << (x - bx * bin_side) for x in range(max(sx[g], bx * bin_side), min(ex[g], (bx + 1) * bin_side)))
+                ym = sum(1 << (y - by * bin_side) for y in range(max(sy[g], by * bin_side), min(ey[g], (by + 1) * bin_side)))
+                per_bin_masks[by * nbx + bx].append(xm | (ym << 8))
     ids = [S["sorted_ids"][:negatives].astype(np.int64)]
+    masks = [np.full(negatives, 0xffff, np.int64)]
     ranges = [negatives]
-    for lst in per_bin:
+    for lst, ms in zip(per_bin, per_bin_masks):
         ids.append(np.asarray(lst, np.int64))
+        masks.append(np.asarray(ms, np.int64))
         ranges.append(ranges[-1] + len(lst))
     last_rows = np.where(pos, (ey - 1) * ntx + (ex - 1), -1)
-    return np.concatenate(ids), np.asarray(ranges, np.int64), int(last_rows.max()) if n else -1
+    return (np.concatenate(ids), np.asarray(ranges, np.int64), int(last_rows.max()) if n else -1,
+            np.concatenate(masks))

@@ -253,7 +253,7 @@ def test_backward_takes_ids_only_up_to_the_last_gaussian():
     args = (t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
     _, st = stages.forward(cam, *args)
     bad = torch.tensor([0x7fffffff, -1, n, 1 << 30, -(1 << 31)], dtype=torch.int32, device=DEV)
-    st.sorted_ids[::5] = bad[torch.arange(st.sorted_ids[::5].numel(), device=DEV) % 5]
+    st.ids[::5] = bad[torch.arange(st.ids[::5].numel(), device=DEV) % 5]
     o = stages.backward(cam, st, 16, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["v_image"])
     torch.cuda.synchronize()
     # the replaced entries all read as Gaussian n - 1: it is marked, and nothing outside the arrays was touched
@@ -742,12 +742,14 @@ def test_list_positions_beyond_the_ids_are_not_followed():
     for bins in (1, 4):
         cam = stages.camera_from_scene(sc, DEV, list_bin=bins)
         image, st = stages.forward(cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"], t["shs"])
-        k = st.sorted_ids.numel()
+        k = st.num_keys
         parts = stages.split_lists(cam, st.lists)
         which = "fine" if bins == 1 else "bins"
         assert int(parts[which][-1].item()) == k
-        # only the first third of the ids is handed over, with the full ranges
-        short = st.sorted_ids[:k // 3].clone()
+        # only the first third of the pairs is handed over (ids and, for binned lists, their mask words), with
+        # the full ranges
+        third = k // 3
+        short = torch.cat([st.sorted_ids[:third], st.sorted_ids[k:k + third]]) if bins > 1 else st.sorted_ids[:third].clone()
         img2, fT2, fidx2 = stages.blend_fwd(cam, st.lists, short, st.splats)
         torch.cuda.synchronize()
         assert torch.isfinite(img2).all()

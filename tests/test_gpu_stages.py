@@ -354,7 +354,7 @@ def test_binned_tile_lists_vs_oracle(oracle, list_bin, bin_side, n, W, H, scale_
     sc, A, s, img, radii, st, S = oracle_scene(oracle, n=n, W=W, H=H, seed=11 + n, scale_mul=scale_mul,
                                                flip_behind=flip, giants=giants, camera=camera)
     oracle.free(st)
-    want_ids, want_bins, want_last = expected_bin_lists(S, radii, W, H, bin_side)
+    want_ids, want_bins, want_last, want_masks = expected_bin_lists(S, radii, W, H, bin_side)
     cam = st_.camera_from_scene(sc, DEV)
     assert st_.list_bin(cam) == bin_side
     order = st_.new_order(cam, n, DEV)
@@ -370,7 +370,14 @@ def test_binned_tile_lists_vs_oracle(oracle, list_bin, bin_side, n, W, H, scale_
     assert (parts["fine"].cpu().numpy() == S["ranges"]).all()
     assert int(parts["last_tile"].item()) == want_last
     assert (parts["bins"].cpu().numpy() == want_bins).all()
-    assert (ids.cpu().numpy() == want_ids).all()
+    # the buffer: k ids and, behind them, one word per pair: its slot (bin + 1; 0 = negative depths) in the low
+    # half, the tiles of the bin that its Gaussian covers in the high half
+    assert ids.numel() == 2 * k
+    assert (ids[:k].cpu().numpy() == want_ids).all()
+    words = ids[k:].cpu().numpy().astype(np.int64) & 0xffffffff
+    assert ((words >> 16) == want_masks).all()
+    want_slots = np.repeat(np.arange(len(want_bins)), np.diff(np.concatenate([[0], want_bins])))
+    assert ((words & 0xffff) == want_slots).all()
     if flip:
         assert want_bins[0] > 0
 

@@ -28,7 +28,7 @@ def _backward_both_ways(oracle, n, W, H, camera, seed):
     # the entry point under test: same arguments, no accumulator
     out = stages._bwd_outputs(n, 16, torch.device(DEV))
     p = lambda x: None if x is None else C.c_void_p(x.data_ptr())
-    rc = lib.dsx_backward_static(cam.ref, n, st.sorted_ids.numel(), 16, p(t["means_3d"]), p(scales), p(t["rotations"]), p(st.splats), None,
+    rc = lib.dsx_backward_static(cam.ref, n, st.num_keys, 16, p(t["means_3d"]), p(scales), p(t["rotations"]), p(st.splats), None,
                                  p(st.radii), p(st.lists), p(st.sorted_ids), p(st.final_T), p(st.final_idx),
                                  p(t["v_image"]), p(out["v_mean3d"]), p(out["v_means2d"]), p(out["v_shs"]),
                                  p(out["v_colors"]), p(out["v_opacity"]), p(out["v_scale"]), p(out["v_quat"]),
