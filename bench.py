@@ -313,7 +313,13 @@ def main():
         "config": {"workload": "%s: %d Gaussians, %dx%d, SH degree %d, %s" %
                                (spec.name, n, W, H, sc["sh_degree"], "forward+backward" if do_backward else "forward"),
                    "num_keys": int(k), "num_keys_per_tile_lists": k_per_tile, "tiles": int(tiles),
-                   "list_bin_tiles": list_bin, "lists": int(lists), "gaussians_with_gradient": marked},
+                   "list_bin_tiles": list_bin, "lists": int(lists), "gaussians_with_gradient": marked,
+                   # (from the CPU oracle's counters, when it ran: pixel-entry pairs that the blend kernels
+                   # walk, and those among them that are blended)
+                   "pairs_walked_fwd": int(counters.pairs_fwd) if counters is not None else None,
+                   "pairs_blended_fwd": int(counters.pairs_fwd_applied) if counters is not None else None,
+                   "pairs_walked_bwd": int(counters.pairs_bwd) if counters is not None else None,
+                   "pairs_valid_bwd": int(counters.pairs_bwd_valid) if counters is not None else None},
         "mpix_per_s": round(W * H / (ms_per_step * 1e-3) / 1e6, 1),
         "ms_per_step_with_kernel_events": round(ms_per_step_traced, 4),
         # the host's share of a step (enqueue + the wait for the pair count) and the device's (sum of the

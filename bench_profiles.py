@@ -6,23 +6,23 @@ and the instruction counters come from separate rocprofv3 runs of the same scrip
 reads their CSV files and writes a short markdown table and, for the traffic, a JSON record that
 bench.py quotes as `roofline.traffic` (with the commit the counters were taken at).
 
-    # on the MI355X box, repository root (each counter set in a run of its own):
+    # on the MI355X box, repository root (each counter set in a run of its own; W = cfg1 .. cfg4, dense):
     export TMPDIR=/tmp
-    rocprofv3 --kernel-trace --stats --output-format csv -d out/prof -o bench -- \\
-        python3 bench.py --steps 20 --warmup 5 --no-cpu-baseline
-    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out/pmc_fetch -o f -- \\
-        python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe > out/pmc_fetch.json
-    rocprofv3 --pmc WRITE_SIZE --output-format csv -d out/pmc_write -o w -- \\
-        python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe
+    rocprofv3 --kernel-trace --stats --output-format csv -d out/W/prof -o bench -- \\
+        python3 bench.py --workload W --steps 20 --warmup 5 --no-cpu-baseline
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out/W/pmc_fetch -o f -- \\
+        python3 bench.py --workload W --steps 2 --warmup 1 --no-cpu-baseline --copy-probe > out/W/pmc_fetch.json
+    rocprofv3 --pmc WRITE_SIZE --output-format csv -d out/W/pmc_write -o w -- \\
+        python3 bench.py --workload W --steps 2 --warmup 1 --no-cpu-baseline --copy-probe
     rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_INSTS_SALU \\
-        SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT --output-format csv -d out/pmc_sq -o s -- \\
-        python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline
+        SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT --output-format csv -d out/W/pmc_sq -o s -- \\
+        python3 bench.py --workload W --steps 2 --warmup 1 --no-cpu-baseline
 
     # anywhere the CSV files are (the commit is read from git when --commit is not given):
-    python3 bench_profiles.py stats   out/prof --name bench_cfg2_fwd_bwd_kernel_stats
-    python3 bench_profiles.py traffic out/pmc_fetch out/pmc_write --bench-json out/pmc_fetch.json \\
-        --name cfg2_hbm_traffic_per_kernel
-    python3 bench_profiles.py sq      out/pmc_sq out/prof --name cfg2_sq_counters_per_kernel
+    python3 bench_profiles.py stats   out/W/prof --workload W --name W_kernel_stats
+    python3 bench_profiles.py traffic out/W/pmc_fetch out/W/pmc_write --bench-json out/W/pmc_fetch.json \\
+        --workload W --name W_hbm_traffic_per_kernel
+    python3 bench_profiles.py sq      out/W/pmc_sq out/W/prof --workload W --name W_sq_counters_per_kernel
 """
 import argparse
 import collections
@@ -40,18 +40,26 @@ PROFILES = os.path.join(ROOT, "profiles")
 
 # the commands whose output this tool reads; {dir} is the directory that the tool was given
 STATS_CMD = ("rocprofv3 --kernel-trace --stats --output-format csv -d {dir} -o bench -- "
-             "python3 bench.py --steps 20 --warmup 5 --no-cpu-baseline")
+             "python3 bench.py --workload {workload} --steps 20 --warmup 5 --no-cpu-baseline")
 FETCH_CMD = ("rocprofv3 --pmc FETCH_SIZE --output-format csv -d {dir} -o f -- "
-             "python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe")
+             "python3 bench.py --workload {workload} --steps 2 --warmup 1 --no-cpu-baseline --copy-probe")
 WRITE_CMD = ("rocprofv3 --pmc WRITE_SIZE --output-format csv -d {dir} -o w -- "
-             "python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline --copy-probe")
+             "python3 bench.py --workload {workload} --steps 2 --warmup 1 --no-cpu-baseline --copy-probe")
 SQ_CMD = ("rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_INSTS_SALU "
           "SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT --output-format csv -d {dir} -o s -- "
-          "python3 bench.py --steps 2 --warmup 1 --no-cpu-baseline")
+          "python3 bench.py --workload {workload} --steps 2 --warmup 1 --no-cpu-baseline")
 
 
-def command(template, directory):
-    return template.format(dir=os.path.normpath(directory))
+def command(template, directory, workload="cfg2"):
+    return template.format(dir=os.path.normpath(directory), workload=workload)
+
+
+def workload_title(workload):
+    sys.path.insert(0, ROOT)
+    from ds_splat_amd.synthetic import WORKLOADS
+    w = WORKLOADS[workload]
+    return "%s: %d Gaussians, %dx%d, SH degree %d, %s" % (w.name, w.n, w.width, w.height, w.sh_degree,
+                                                           "forward + backward" if w.backward else "forward")
 
 
 def short_name(kernel):
@@ -73,7 +81,10 @@ def trace_name(short):
     """The name the library's own event trace (and bench.py's JSON line) uses for a kernel."""
     base = short.split("<")[0]
     if base == "onesweep32_kernel":
-        return "onesweep32_kernel<tile partition>" if "unsigned short" in short else "onesweep32_kernel<sort>"
+        # the depth sort of the Gaussians carries their rectangles through the passes (last template argument;
+        # images of more than 255 tiles a side excepted); the tile partition, with 16-bit slots per tile or 32-bit
+        # slot words per bin, carries nothing
+        return "onesweep32_kernel<sort>" if short.rstrip().endswith("true>") else "onesweep32_kernel<tile partition>"
     return base
 
 
@@ -127,8 +138,10 @@ def cmd_stats(args):
     if trace:
         for r in csv.DictReader(open(sorted(trace)[-1])):
             med[r["Kernel_Name"]].append(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]))
-    lines = ["# %s" % args.title, "", "Commit: %s" % (args.commit or git_commit()), "",
-             "Command (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "", "    " + command(STATS_CMD, args.dir), "",
+    lines = ["# Kernel statistics, bench.py (%s)" % workload_title(args.workload), "",
+             "Commit: %s" % (args.commit or git_commit()), "",
+             "Command (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "",
+             "    " + command(STATS_CMD, args.dir, args.workload), "",
              "rocprofv3 kernel statistics (all launches of the run, warm-up included; the median is taken from the",
              "kernel trace of the same run):", "",
              "| kernel | calls | total ms | avg us | median us | % |", "|---|---|---|---|---|---|"]
@@ -171,9 +184,10 @@ def cmd_traffic(args):
     lines = ["# HBM traffic per launch (FETCH_SIZE / WRITE_SIZE), %s" % cfg["workload"], "",
              "Commit: %s" % commit, "",
              "Commands (on the MI355X box, repository root, after `export TMPDIR=/tmp`; one counter per run):", "",
-             "    " + command(FETCH_CMD, args.fetch_dir), "    " + command(WRITE_CMD, args.write_dir),
-             "    python3 bench_profiles.py traffic %s %s --bench-json <the first run's JSON line> --name %s" % (
-                 os.path.normpath(args.fetch_dir), os.path.normpath(args.write_dir), args.name),
+             "    " + command(FETCH_CMD, args.fetch_dir, args.workload),
+             "    " + command(WRITE_CMD, args.write_dir, args.workload),
+             "    python3 bench_profiles.py traffic %s %s --bench-json <the first run's JSON line> --workload %s --name %s" % (
+                 os.path.normpath(args.fetch_dir), os.path.normpath(args.write_dir), args.workload, args.name),
              "",
              "Calibration: `--copy-probe` runs one 1 GiB device-to-device copy (`%s`, reads 1048576 KiB, writes 1048576 KiB)." % copy,
              "The counters read FETCH_SIZE = %.1f KiB and WRITE_SIZE = %.1f KiB for it, so the scale factors are %.4f (fetch) and %.4f (write)." % (
@@ -212,9 +226,11 @@ def cmd_sq(args):
     d = counters_per_kernel(args.sq_dir)
     times = kernel_times_ms(args.stats_dir)
     avg = lambda x: sum(x) / len(x)
-    lines = ["# SQ counters per kernel (VALU issue, LDS bank conflicts)", "", "Commit: %s" % (args.commit or git_commit()), "",
-             "Commands (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "", "    " + command(SQ_CMD, args.sq_dir),
-             "    " + command(STATS_CMD, args.stats_dir) + "    # the `kernel ms` column", "",
+    lines = ["# SQ counters per kernel (VALU issue, LDS bank conflicts), %s" % workload_title(args.workload), "",
+             "Commit: %s" % (args.commit or git_commit()), "",
+             "Commands (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "",
+             "    " + command(SQ_CMD, args.sq_dir, args.workload),
+             "    " + command(STATS_CMD, args.stats_dir, args.workload) + "    # the `kernel ms` column", "",
              "Averages per launch. A wave64 VALU instruction occupies its SIMD for 4 clocks, so the chip (256 CU x 4 SIMD at 2.4 GHz)",
              "issues at most 614 G wave-instructions/s: `VALU floor` = SQ_INSTS_VALU / 614e9 is the time the kernel's VALU",
              "instructions alone need (quarter-rate instructions such as exp and rcp count once here, so the true floor is higher);",
@@ -240,7 +256,6 @@ def main():
     p = sub.add_parser("stats", help="kernel statistics of a --kernel-trace --stats run")
     p.add_argument("dir")
     p.add_argument("--name", required=True)
-    p.add_argument("--title", default="Kernel statistics, bench.py (cfg2: 3 M Gaussians, 1920x1080, SH 3, forward + backward)")
     p.add_argument("--commit")
     p.set_defaults(fn=cmd_stats)
     p = sub.add_parser("traffic", help="HBM bytes per launch from a FETCH_SIZE run and a WRITE_SIZE run")
@@ -256,6 +271,8 @@ def main():
     p.add_argument("--name", required=True)
     p.add_argument("--commit")
     p.set_defaults(fn=cmd_sq)
+    for p in sub.choices.values():
+        p.add_argument("--workload", default="cfg2", help="the bench.py workload the runs were made with")
     args = ap.parse_args()
     args.fn(args)
 
