@@ -848,3 +848,70 @@ def test_non_finite_gaussians_are_culled_and_leave_the_rest_alone():
     assert img_n.shape == img_c.shape and torch.equal(radii_n > 0, (radii_c > 0) | torch.isin(
         torch.arange(20000, device=DEV), bad.to(DEV)) & (radii_n > 0))
 
+
+
+def test_forward_refuses_more_per_tile_pairs_than_32_bits_index():
+    """Lists per bin hold a fraction of the pairs of per-tile lists, but the per-tile ranges, final_idx and the
+    scan records still index the per-tile pairs as int32: 300 K Gaussians that each cover the whole 1920 x 1080
+    image make 2.4 G per-tile pairs (beyond 2^31) and only 40 M pairs of the 8 x 8 bins (well below the 2^30 that
+    the partition sorts).  The forward must say DSX_ERR_TOO_LARGE after its first half, not wrap the indices."""
+    from ds_splat_amd import stages
+    n = 300_000
+    sc = make_scene("cfg1", n=n, width=1920, height=1080, sh_degree=0)
+    sc["means_3d"][:, :2] *= 0.02                      # all near the optical axis
+    sc["scales"] = torch.full_like(sc["scales"], 40.0)  # ... and far larger than the frustum
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    cam = stages.camera_from_scene(sc, DEV)
+    assert stages.list_bin(cam) == 8
+    with pytest.raises(RuntimeError, match="too many"):
+        stages.forward(cam, t["means_3d"], t["scales"], t["rotations"], t["opacities"], t["shs"])
+    torch.cuda.synchronize()
+    # the same scene cut to a tenth fits both limits and renders
+    m = n // 10
+    image, st = stages.forward(cam, t["means_3d"][:m].contiguous(), t["scales"][:m].contiguous(),
+                               t["rotations"][:m].contiguous(), t["opacities"][:m].contiguous(),
+                               t["shs"][:m].contiguous())
+    torch.cuda.synchronize()
+    assert st.num_keys_per_tile == (m - 1) * 8160 and st.num_keys == (m - 1) * 135
+    assert torch.isfinite(image).all()
+
+
+@pytest.mark.parametrize("bins", [0, 2, 8])
+def test_stage_entry_points_chain_on_binned_lists(oracle, bins):
+    """The documented chain of stage entry points (projection, depth order, tile lists, blend forward, blend
+    backward) on an image whose lists the library builds per bin of tiles: the same camera goes to every call,
+    the whole `ranges` and `sorted_ids` buffers go from dsx_tile_lists to the blend stages, and the results are
+    the oracle's."""
+    from ds_splat_amd import stages
+    sc = make_scene("cfg1", n=40000, width=1280, height=720, sh_degree=3, seed=77)      # 3600 tiles
+    img_o, radii_o, S, B = oracle_run(oracle, sc, 2.0)
+    t = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in sc.items()}
+    cam = stages.camera_from_scene(sc, DEV, list_bin=bins)
+    assert stages.list_bin(cam) == (4 if bins == 0 else bins)
+    n = sc["n"]
+    order = stages.new_order(cam, n, DEV)
+    splats, radii, cov3d, _ = stages.project_fwd(cam, t["means_3d"], t["scales"] * 2.0, t["rotations"], t["opacities"],
+                                                 t["shs"], order=order)
+    stages.depth_order(cam, n, order)
+    torch.cuda.synchronize()
+    k = stages.key_count(cam, n, order)
+    ids, lists = stages.tile_lists(cam, n, k, order, return_lists=True)
+    image, final_T, final_idx = stages.blend_fwd(cam, lists, ids, splats)
+    grads = stages.blend_bwd(cam, n, lists, ids, splats, final_T, final_idx, t["v_image"])
+    torch.cuda.synchronize()
+    assert (radii.cpu().numpy() == radii_o).all()
+    assert (lists[:cam.num_tiles + 1].cpu().numpy() == S["ranges"]).all()
+    ok = S["margin"] > 1e-4
+    assert ok.mean() > 0.98
+    np.testing.assert_allclose(image.cpu().numpy()[ok], img_o[ok], rtol=1e-4, atol=1e-5)
+    assert (final_idx.cpu().numpy()[ok] == S["final_idx"][ok]).all()
+    # the nine screen-space sums against the oracle's blend backward, each within 1e-4 of the summed magnitudes
+    # of its terms, for the Gaussians that no borderline decision touches
+    A = arrays(sc)
+    Bb = oracle.blend_bwd(scene_settings(sc), S["ranges"], S["sorted_ids"], S["means2d"], S["conic"], S["rgb"],
+                          A["opacities"], S["final_T"], S["final_idx"], A["v_image"])
+    gok = comparable_gaussians(S, Bb, sc["width"], final_T.cpu().numpy(), final_idx.cpu().numpy())
+    want = np.concatenate([Bb["v_xy"], Bb["v_conic"], Bb["v_opacity"].reshape(n, 1), Bb["v_rgb"]], axis=1).astype(np.float64)
+    err = np.abs(grads.cpu().numpy()[:, :9].astype(np.float64) - want)[gok]
+    bound = (1e-4 * Bb["abs_sums"].astype(np.float64) + 1e-7)[gok]
+    assert gok.mean() > 0.5 and (err <= bound).all(), float((err / bound).max())
