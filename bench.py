@@ -45,11 +45,13 @@ def measured_traffic(workload, num_keys):
                                     "scale_fetch": rec.get("scale_fetch"), "scale_write": rec.get("scale_write")}
 
 
-def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters, marked, carries_rects=True):
+def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters, marked, carries_rects=True, binned=True):
     """(bound, work per launch, unit): algorithmic HBM bytes or FP32 operations per launch.
     k: pairs of the tile lists as built (per bin of tiles); lists: how many lists they are partitioned into;
-    marked: Gaussians whose accumulator record received a term in the blend backward."""
-    slot_bytes = 2 if lists + 1 <= 65535 else 4
+    marked: Gaussians whose accumulator record received a term in the blend backward;
+    binned: the lists are per bin of tiles (a pair's slot word then has 32 bits, half of them the mask of the
+    bin's tiles that its Gaussian covers, and the sorted words are kept for the blend kernels)."""
+    slot_bytes = 4 if binned else (2 if lists + 1 <= 65535 else 4)
     if kernel == "project_fwd_kernel":
         # inputs 44 + 12c bytes, outputs radii + splat record + depth key + tile rectangle (the 3-D
         # covariance is not stored on this path: the backward rebuilds it)
@@ -73,6 +75,8 @@ def algorithmic_work(kernel, n, k, pixels, lists, coeffs, counters, marked, carr
     if kernel == "onesweep32_kernel<tile partition>":
         # tile partition: slot + id in and out, except that the last pass writes no slots (average per launch)
         passes = 1 if lists + 1 <= 256 else (2 if lists + 1 <= 65536 else 3)
+        if binned:
+            return "hbm", 2 * (slot_bytes + 4) * k, "B"
         return "hbm", (2 * (slot_bytes + 4) * passes - slot_bytes) * k / passes, "B"
     if kernel == "blend_fwd_kernel" and counters is not None:
         rej = counters.pairs_fwd - counters.pairs_fwd_applied
@@ -267,7 +271,7 @@ def main():
         launches_per_step = cnt / args.steps
         avg = tot / cnt
         bound, work, unit = algorithmic_work(name, n, k, W * H, lists, coeffs, counters, marked,
-                                             (W + 15) // 16 <= 255 and (H + 15) // 16 <= 255)
+                                             (W + 15) // 16 <= 255 and (H + 15) // 16 <= 255, list_bin > 1)
         table.append((tot / args.steps, name, avg, launches_per_step, bound, work, unit))
     table.sort(reverse=True)
     measured, traffic_source = measured_traffic(spec.name, k) if args.n is None else ({}, None)

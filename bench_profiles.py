@@ -23,6 +23,7 @@ bench.py quotes as `roofline.traffic` (with the commit the counters were taken a
     python3 bench_profiles.py traffic out/W/pmc_fetch out/W/pmc_write --bench-json out/W/pmc_fetch.json \\
         --workload W --name W_hbm_traffic_per_kernel
     python3 bench_profiles.py sq      out/W/pmc_sq out/W/prof --workload W --name W_sq_counters_per_kernel
+    # (optional, `mem`: vector-memory instructions and L2 atomics per kernel; its command is in the summary it writes)
 """
 import argparse
 import collections
@@ -48,6 +49,11 @@ WRITE_CMD = ("rocprofv3 --pmc WRITE_SIZE --output-format csv -d {dir} -o w -- "
 SQ_CMD = ("rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_INSTS_SALU "
           "SQ_INSTS_LDS SQ_LDS_BANK_CONFLICT --output-format csv -d {dir} -o s -- "
           "python3 bench.py --workload {workload} --steps 2 --warmup 1 --no-cpu-baseline")
+
+
+MEM_CMD = ("rocprofv3 --pmc SQ_WAVES SQ_INSTS_VMEM_WR SQ_INSTS_VMEM_RD SQ_INSTS_BRANCH TCC_ATOMIC_sum "
+           "TCP_TCC_ATOMIC_WITHOUT_RET_REQ_sum --output-format csv -d {dir} -o m -- "
+           "python3 bench.py --workload {workload} --steps 2 --warmup 1 --no-cpu-baseline")
 
 
 def command(template, directory, workload="cfg2"):
@@ -165,7 +171,8 @@ def algorithmic_bytes(bench):
               "ordered_block_sums_kernel", "emit_ordered_kernel", "onesweep32_kernel<tile partition>"):
         bound, work, _ = bench_module.algorithmic_work(k, n, cfg["num_keys"], w * h, cfg["lists"], (deg + 1) ** 2, None,
                                                        cfg.get("gaussians_with_gradient", 0),
-                                                       (w + 15) // 16 <= 255 and (h + 15) // 16 <= 255)
+                                                       (w + 15) // 16 <= 255 and (h + 15) // 16 <= 255,
+                                                       cfg.get("list_bin_tiles", 1) > 1)
         if bound == "hbm":
             out[k] = work
     return out, n
@@ -250,6 +257,35 @@ def cmd_sq(args):
     write(args.name, lines)
 
 
+def cmd_mem(args):
+    """Vector-memory instructions and atomics per kernel: how many atomic requests the blend backward sends
+    (one instruction per blended (tile, entry) with nine active lanes) and what share of its time they are."""
+    d = counters_per_kernel(args.mem_dir)
+    times = kernel_times_ms(args.stats_dir)
+    avg = lambda x: sum(x) / len(x) if x else 0.0
+    lines = ["# Vector-memory instructions and L2 atomics per kernel, %s" % workload_title(args.workload), "",
+             "Commit: %s" % (args.commit or git_commit()), "",
+             "Commands (on the MI355X box, repository root, after `export TMPDIR=/tmp`):", "",
+             "    " + command(MEM_CMD, args.mem_dir, args.workload),
+             "    " + command(STATS_CMD, args.stats_dir, args.workload) + "    # the `kernel ms` column", "",
+             "Averages per launch. `VMEM write inst` counts stores and atomics (the blend backward issues one atomic",
+             "instruction per blended (tile, entry), nine lanes active, plus one byte store for the Gaussian's mark, and at",
+             "its end the stores of the zeros); `L2 atomic requests` is TCC_ATOMIC summed over the L2 channels.", "",
+             "| kernel | waves | VMEM read inst / wave | VMEM write inst / wave | branches / wave | TCP atomic requests | L2 atomic requests | L2 atomics / us | kernel ms |",
+             "|---|---|---|---|---|---|---|---|---|"]
+    for k in sorted(d, key=lambda k: -avg(d[k]["TCC_ATOMIC_sum"])):
+        c = d[k]
+        if "at::" in k or k.startswith("__amd") or not c["SQ_WAVES"] or k not in times:
+            continue
+        waves = avg(c["SQ_WAVES"])
+        atom = avg(c["TCC_ATOMIC_sum"])
+        lines.append("| %s | %d | %.1f | %.1f | %.1f | %.4g | %.4g | %.0f | %.3f |" % (
+            k, waves, avg(c["SQ_INSTS_VMEM_RD"]) / waves, avg(c["SQ_INSTS_VMEM_WR"]) / waves,
+            avg(c["SQ_INSTS_BRANCH"]) / waves, avg(c["TCP_TCC_ATOMIC_WITHOUT_RET_REQ_sum"]), atom,
+            atom / (times[k] * 1e3), times[k]))
+    write(args.name, lines)
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -271,6 +307,12 @@ def main():
     p.add_argument("--name", required=True)
     p.add_argument("--commit")
     p.set_defaults(fn=cmd_sq)
+    p = sub.add_parser("mem", help="vector-memory instructions and atomics per kernel")
+    p.add_argument("mem_dir")
+    p.add_argument("stats_dir")
+    p.add_argument("--name", required=True)
+    p.add_argument("--commit")
+    p.set_defaults(fn=cmd_mem)
     for p in sub.choices.values():
         p.add_argument("--workload", default="cfg2", help="the bench.py workload the runs were made with")
     args = ap.parse_args()
