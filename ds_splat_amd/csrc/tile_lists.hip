@@ -12,6 +12,7 @@
 // once and moved twice, instead of 12 bytes moved five times.
 #include "dsx_common.h"
 
+#include <algorithm>
 #include <mutex>
 
 namespace dsx
@@ -58,8 +59,12 @@ ListGrid list_grid(int image_width, int image_height, int list_bin)
     int side = list_bin ? list_bin : 1;
     if(!list_bin && g.ntx * g.nty >= 2048)
     {
-        auto lists = [&](int b) { return ((g.ntx + b - 1) / b) * ((g.nty + b - 1) / b); };
-        side = (slot_bits(lists(4)) > 8 && slot_bits(lists(8)) <= 8) ? 8 : 4;
+        auto lists = [&](int64_t b) { return ((g.ntx + b - 1) / b) * ((g.nty + b - 1) / b); };
+        side = (slot_bits((int)std::min<int64_t>(lists(4), 1 << 30)) > 8 && slot_bits((int)lists(8)) <= 8) ? 8 : 4;
+        // (a bin's slot shares its 32-bit word with the 16-bit tile mask: at most 65534 bins; images beyond
+        // that, hundreds of megapixels, get larger bins or, failing that, per-tile lists with 32-bit slots)
+        if(lists(side) + 1 > 65535)
+            side = lists(8) + 1 <= 65535 ? 8 : 1;
     }
     g.shift = side == 8 ? 3 : (side == 4 ? 2 : (side == 2 ? 1 : 0));
     g.nbx = (g.ntx + side - 1) / side;

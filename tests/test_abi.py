@@ -56,6 +56,8 @@ def test_host_helpers():
     assert lib.dsx_list_bin(1920, 1080, 0) == 8 and lib.dsx_list_bin(1024, 512, 0) == 4
     assert lib.dsx_list_bin(1024, 496, 0) == 1 and lib.dsx_list_bin(3840, 2160, 0) == 4
     assert lib.dsx_list_bin(640, 480, 8) == 8 and lib.dsx_list_bin(640, 480, 0) == 1
+    # a bin's slot shares its word with the tile mask (at most 65534 bins): larger bins, then per-tile lists
+    assert lib.dsx_list_bin(16400, 16400, 0) == 8 and lib.dsx_list_bin(40000, 40000, 0) == 1
     assert lib.dsx_ranges_count(1920, 1080, 0) == (8160 + 1) + 1 + 1 + (15 * 9 + 1) + 8 * 8160
     assert lib.dsx_ranges_count(1920, 1080, 8) == lib.dsx_ranges_count(1920, 1080, 0)
     assert lib.dsx_ranges_count(240, 240, 0) == 225 + 2
