@@ -207,8 +207,8 @@ inline bool valid_list_bin(int b)
 //   last_tile[1]      highest tile that holds a pair of non-negative depth, -1 if none
 //   bins[bins + 1]    ranges of the bin lists inside sorted_ids
 //   walk[tiles * 8]   written by the blend forward for the backward: per tile and band of four
-//                     rows, the position in the bin list of the last entry any of its pixels
-//                     blended, and that entry's index in the per-tile list
+//                     rows, the position in the bin's list where the forward's scan stopped and
+//                     the number of the tile's own entries it had met by then
 struct RangesLayout
 {
     int fine, header, last_tile, bins, walk, count;

@@ -111,7 +111,8 @@ int32_t dsx_sort_passes(int32_t num_tiles);
  * bit); with b > 1 the same entries reach every pixel in the same order, final_idx holds the same
  * indices, and emission and partition handle a fraction of the pairs.  b is dsx_camera::list_bin, or,
  * when that is 0, the library's choice for the image size: 1 below 2048 tiles; above, 8 where that
- * brings the lists down to the 256 slots of a single partition pass and 4 does not, else 4.
+ * brings the lists down to the 256 slots of a single partition pass and 4 does not, else 4 (and
+ * never more than 65534 bins: an image of hundreds of megapixels gets 8, or per-tile lists).
  * dsx_list_bin(width, height, list_bin) returns the b that a call with this list_bin uses (0 for a
  * list_bin that is none of 0, 1, 2, 4, 8).
  * dsx_ranges_count: int32 words of the `ranges` buffer of those entry points: tiles + 1 words of
