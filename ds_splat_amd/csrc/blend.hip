@@ -11,10 +11,14 @@ namespace dsx
 
 constexpr float kAlphaThreshold = 1.0f / 255.0f;
 
-// exp through the hardware base-2 exponential (the reference is built with fast-math)
-__device__ __forceinline__ float fast_exp(float x)
+// exp through the hardware base-2 exponential (the reference is built with fast-math).  The
+// factor log2(e) is not applied per pixel: the three conic coefficients are multiplied by it
+// once, when an entry is staged in LDS, so the quadratic form below comes out in base 2.
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+__device__ __forceinline__ float exp2_of(float x)
 {
-    return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
+    return __builtin_amdgcn_exp2f(x);
 }
 
 // The exponent of a splat at a pixel, -1/2 (a dx^2 + c dy^2) - b dx dy with d = pixel - mean, in
@@ -23,22 +27,24 @@ __device__ __forceinline__ float fast_exp(float x)
 // resulting alpha with 1/255 on their own.  If they disagreed on a borderline entry, the backward
 // would rebuild the transmittance of every entry in front of it from a final value that does
 // (or does not) contain its factor: an error of alpha in all their gradients at that pixel.
+// (The halves are taken by the caller: a_half = -a/2 and c_half = c/2, exact scalings, so it does
+// not matter to the bits whether they are applied per entry or once when the entry is staged.)
 struct ExponentX
 {
     float ax, bx; // -1/2 a dx^2 and b dx
 };
-__device__ __forceinline__ ExponentX exponent_x(float a, float b, float dx)
+__device__ __forceinline__ ExponentX exponent_x(float a_half, float b, float dx)
 {
 #pragma clang fp contract(off)
     ExponentX r;
     r.bx = b * dx;
-    r.ax = -0.5f * a * dx * dx;
+    r.ax = a_half * dx * dx;
     return r;
 }
-__device__ __forceinline__ float exponent_xy(ExponentX x, float c, float dy)
+__device__ __forceinline__ float exponent_xy(ExponentX x, float c_half, float dy)
 {
 #pragma clang fp contract(off)
-    const float inner = __builtin_fmaf(0.5f * c, dy, x.bx);
+    const float inner = __builtin_fmaf(c_half, dy, x.bx);
     return __builtin_fmaf(-inner, dy, x.ax);
 }
 
@@ -220,8 +226,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                                                              uint8_t* __restrict__ prep_marks,
                                                              const BinLists lists)
 {
-    __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic a, conic b
-    __shared__ float4 s_b[kFwdBatch]; // conic c, opacity, red, green
+    __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic -a/2, conic b (a, b, c times log2 e)
+    __shared__ float4 s_b[kFwdBatch]; // conic c/2, opacity, red, green
     __shared__ float s_c[kFwdBatch];  // blue
     // the queue of the tile's own entries (binned lists) lives in s_a between two rounds: up to 128 ids
     int* const s_queue = reinterpret_cast<int*>(s_a);
@@ -364,8 +370,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             {
                 const float4* rec = splats + 3 * (int64_t)g;
                 const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
-                s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
-                s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
+                s_a[slot] = make_float4(q0.x, q0.y, q1.x * (-0.5f * kLog2e), q1.y * kLog2e);
+                s_b[slot] = make_float4(q1.z * (0.5f * kLog2e), q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
                 useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
             }
@@ -405,10 +411,11 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                 {
                     const float power = exponent_xy(ex, B.x, pyf[p] - A.y);
                     // (a NaN opacity gives alpha = 0.999 here as in the reference: fminf drops the NaN)
-                    const float alpha = fminf(0.999f, B.y * fast_exp(power));
+                    const float alpha = fminf(0.999f, B.y * exp2_of(power));
                     // the three decisions as wavefront masks (each is its compare's own result register),
                     // combined on the scalar unit and handed back to the lanes as conditions
-                    const float Tn = (1.0f - alpha) * T[p];
+                    // (1 - alpha) T in one rounding
+                    const float Tn = __builtin_fmaf(-alpha, T[p], T[p]);
                     const uint64_t m_pass = __builtin_amdgcn_ballot_w64(power < 0.0f) &
                                             __builtin_amdgcn_ballot_w64(alpha >= kAlphaThreshold);
                     const uint64_t m_low = __builtin_amdgcn_ballot_w64(Tn < 0.0001f);
@@ -648,8 +655,8 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const float* __restrict__ bg, float* grads, uint8_t* marks, int W, int H, int ntx, uint32_t last_id, int k,
     const int32_t* __restrict__ header, int header_shift, const BinLists lists, const ZeroJobs zeros)
 {
-    __shared__ float4 s_a[kBwdBatch]; // pixel x, pixel y, conic a, conic b
-    __shared__ float4 s_b[kBwdBatch]; // conic c, opacity, red, green
+    __shared__ float4 s_a[kBwdBatch]; // pixel x, pixel y, conic -a/2, conic b (a, b, c times log2 e)
+    __shared__ float4 s_b[kBwdBatch]; // conic c/2, opacity, red, green
     __shared__ float s_c[kBwdBatch];  // blue
     __shared__ int s_id[kBwdBatch];
     // the queue of the tile's own entries (binned lists) lives in s_a between two rounds, as in the forward
@@ -811,8 +818,8 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             {
                 const float4* rec = splats + 3 * (int64_t)g;
                 const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
-                s_a[slot] = make_float4(q0.x, q0.y, q1.x, q1.y);
-                s_b[slot] = make_float4(q1.z, q1.w, q2.x, q2.y);
+                s_a[slot] = make_float4(q0.x, q0.y, q1.x * (-0.5f * kLog2e), q1.y * kLog2e);
+                s_b[slot] = make_float4(q1.z * (0.5f * kLog2e), q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
                 s_id[slot] = g;
                 useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
@@ -852,7 +859,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             {
                 dy[p] = pyf[p] - A.y;
                 const float power = exponent_xy(ex, B.x, dy[p]);
-                vis[p] = fast_exp(power);
+                vis[p] = exp2_of(power);
                 alpha[p] = fminf(0.99f, B.y * vis[p]);
                 m_valid[p] = __builtin_amdgcn_ballot_w64(idx <= bin_final[p]) &
                              __builtin_amdgcn_ballot_w64(!(power > 0.0f)) &
@@ -895,8 +902,13 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             const float dx = -dxf;
             S0 *= -B.y;
             S1 *= B.y;
-            g[0] = A.z * dx * S0 + A.w * S1;     // v_sigma (a dx + b dy)
-            g[1] = A.w * dx * S0 + B.x * S1;     // v_sigma (b dx + c dy)
+            // (the staged coefficients are -a/2, b and c/2 times log2(e): the factors are taken out of the
+            // two sums that use them; A.z * dxf and A.w * dxf are the exponent's own first products)
+            {
+#pragma clang fp contract(off)
+                g[0] = __builtin_fmaf(A.w, S1 * kLn2, (A.z * dxf) * (S0 * (2.0f * kLn2)));  // v_sigma (a dx + b dy)
+                g[1] = __builtin_fmaf(B.x, S1 * (2.0f * kLn2), -((A.w * dxf) * (S0 * kLn2))); // v_sigma (b dx + c dy)
+            }
             g[2] = 0.5f * dx * dx * S0;
             g[3] = dx * S1;
             g[4] = -0.5f * B.y * S2;
