@@ -409,7 +409,7 @@ extern "C" int dsx_sort_flags(int64_t n, int64_t k, int32_t width, int32_t heigh
             const ListGrid lg = list_grid(width, height, list_bin);
             const int tiles = lg.lists();
             const ListsWorkspace lw = lists_workspace(k, tiles, lg.shift != 0);
-            const Sort32Workspace w = sort32_workspace(k, slot_bits(tiles), kListSortTile);
+            const Sort32Workspace w = sort32_workspace(k, slot_bits(tiles), sort32_tile_keys(k));
             *partition_flag =
                 reinterpret_cast<const uint32_t*>(static_cast<const char*>(workspace) + lw.sort + w.counters) + w.passes;
         }

@@ -98,37 +98,30 @@ SortWorkspace sort_workspace(int64_t k, int num_tiles);
 // ---- 32-bit radix sort (depth order of the Gaussians, tile partition of the tile lists) ----
 constexpr int kBits32 = 8;
 constexpr int kBins32 = 1 << kBits32;
-// Two geometries of the same pass kernel: the depth sort of the N Gaussians (few keys: 8192-key
-// tiles so that the launch fills the chip) and the partition of the K pairs (12288-key tiles of
-// 1024 threads, two blocks per compute unit: the look-back traffic falls with the number of
-// tiles).  A tile must stay below 65536 keys (positions inside a tile are kept as 16 bits).
-#ifndef DSX_NSORT_THREADS
-#define DSX_NSORT_THREADS 512
-#endif
-#ifndef DSX_NSORT_ITEMS
-#define DSX_NSORT_ITEMS 16
-#endif
-#ifndef DSX_KSORT_THREADS
-#define DSX_KSORT_THREADS 1024
-#endif
-#ifndef DSX_KSORT_ITEMS
-#define DSX_KSORT_ITEMS 12
-#endif
-constexpr int kDepthSortThreads = DSX_NSORT_THREADS;
-constexpr int kDepthSortItems = DSX_NSORT_ITEMS;
-constexpr int kDepthSortTile = kDepthSortThreads * kDepthSortItems;
-// From this many keys on, the sort of (uint32 key, uint32 value) pairs uses the partition's
-// larger tiles too: its passes are bound by the chained scan over the tiles (all of them are
-// resident at once), which is shorter with fewer tiles (3 M keys: 0.028 -> 0.024 ms per pass);
-// smaller inputs keep the small tiles so that the launch still covers the chip.
-constexpr int64_t kLargeTileSortFrom = 1500000;
-constexpr int kListSortThreads = DSX_KSORT_THREADS;
-constexpr int kListSortItems = DSX_KSORT_ITEMS;
-constexpr int kListSortTile = kListSortThreads * kListSortItems;
+// One pass kernel, workgroups of 1024 threads, and a family of tile sizes: 1, 2, 3, 4, 6, 8 or 12 keys
+// per thread.  A pass is a chained scan over its tiles, all resident at once, and takes about as long as
+// one tile's own serial work (every thread ranks its keys one after the other) plus the chain: the
+// fastest tile size is the smallest that still leaves at most one tile per compute unit (measured at
+// 16 K to 3 M keys: 1 M keys take 0.094 ms in 8192-key tiles of 512 threads, 0.075 in 4096-key ones of
+// 1024, 0.125 in 1024-key ones; 16 K keys 0.074 against 0.034).  Beyond 12 keys per thread registers
+// run out, so larger inputs get more tiles than compute units.  A tile must stay below 65536 keys
+// (positions inside a tile are kept as 16 bits).
+constexpr int kSortThreads32 = 1024;
+constexpr int kSortItemsMax32 = 12;
+constexpr int kSortTilesWanted32 = 256; // compute units of an MI355X
+inline int sort32_items(int64_t count)
+{
+    const int64_t want = (count + (int64_t)kSortThreads32 * kSortTilesWanted32 - 1) / ((int64_t)kSortThreads32 * kSortTilesWanted32);
+    const int family[] = {1, 2, 3, 4, 6, 8, kSortItemsMax32};
+    for(int items : family)
+        if(items >= want)
+            return items;
+    return kSortItemsMax32;
+}
 constexpr int kMaxPasses32 = 4;
 inline int sort32_tile_keys(int64_t count)
 {
-    return count >= kLargeTileSortFrom ? kListSortTile : kDepthSortTile;
+    return kSortThreads32 * sort32_items(count);
 }
 // depth key of a Gaussian that emits no (tile, Gaussian) pair; as a float it is a NaN, which no
 // emitting Gaussian has (a NaN depth fails the frustum test)

@@ -216,8 +216,8 @@ constexpr int kSpinLimit32 = 1 << 18; // bounded wait: a stuck predecessor ends 
 #endif
 constexpr int kLookBatch32 = DSX_LOOK32;
 
-static_assert(kDepthSortThreads >= kBins32 && kListSortThreads >= kBins32, "one thread per digit");
-static_assert(kDepthSortTile <= 65535 && kListSortTile <= 65535, "u16 ranks");
+static_assert(kSortThreads32 >= kBins32, "one thread per digit");
+static_assert(kSortThreads32 * kSortItemsMax32 <= 65535, "u16 ranks");
 
 // A tile rectangle as the projection packs it (16-bit fields) in 32 bits: 8 bits each for first
 // column, first row, width and height, for images of at most 255 x 255 tiles.  The depth's sign
@@ -649,26 +649,29 @@ int launch_sort32(int64_t count, int key_bits, uint32_t* keys_a, uint32_t* vals_
                            reinterpret_cast<uint32_t*>(static_cast<char*>(sort_ws) + w.hist));
     }
     DSX_LAUNCH_CHECK();
-    const bool large = sort32_tile_keys(count) == kListSortTile;
-    if(carry_a && carry_b && gather_src && gather_dst)
+    const bool carry = carry_a && carry_b && gather_src && gather_dst;
+#define DSX_SORT32_ITEMS(ITEMS)                                                                                       \
+    case ITEMS:                                                                                                       \
+        return carry ? sort32_passes<uint32_t, kSortThreads32, ITEMS, true>(                                          \
+                           count, key_bits, keys_a, vals_a, keys_b, vals_b, iota_values, keep_keys, sort_ws,          \
+                           "onesweep32_kernel<sort>", stream, keys_out, vals_out, gather_src, gather_dst, nullptr,    \
+                           carry_a, carry_b)                                                                          \
+                     : sort32_passes<uint32_t, kSortThreads32, ITEMS>(count, key_bits, keys_a, vals_a, keys_b, vals_b, \
+                                                                      iota_values, keep_keys, sort_ws,                \
+                                                                      "onesweep32_kernel<sort>", stream, keys_out,    \
+                                                                      vals_out, gather_src, gather_dst)
+    switch(sort32_items(count))
     {
-        if(large)
-            return sort32_passes<uint32_t, kListSortThreads, kListSortItems, true>(
-                count, key_bits, keys_a, vals_a, keys_b, vals_b, iota_values, keep_keys, sort_ws,
-                "onesweep32_kernel<sort>", stream, keys_out, vals_out, gather_src, gather_dst, nullptr, carry_a, carry_b);
-        return sort32_passes<uint32_t, kDepthSortThreads, kDepthSortItems, true>(
-            count, key_bits, keys_a, vals_a, keys_b, vals_b, iota_values, keep_keys, sort_ws, "onesweep32_kernel<sort>",
-            stream, keys_out, vals_out, gather_src, gather_dst, nullptr, carry_a, carry_b);
+        DSX_SORT32_ITEMS(1);
+        DSX_SORT32_ITEMS(2);
+        DSX_SORT32_ITEMS(3);
+        DSX_SORT32_ITEMS(4);
+        DSX_SORT32_ITEMS(6);
+        DSX_SORT32_ITEMS(8);
+        DSX_SORT32_ITEMS(kSortItemsMax32);
     }
-    if(large)
-        return sort32_passes<uint32_t, kListSortThreads, kListSortItems>(count, key_bits, keys_a, vals_a, keys_b, vals_b,
-                                                                         iota_values, keep_keys, sort_ws,
-                                                                         "onesweep32_kernel<sort>", stream, keys_out,
-                                                                         vals_out, gather_src, gather_dst);
-    return sort32_passes<uint32_t, kDepthSortThreads, kDepthSortItems>(count, key_bits, keys_a, vals_a, keys_b, vals_b,
-                                                                       iota_values, keep_keys, sort_ws,
-                                                                       "onesweep32_kernel<sort>", stream, keys_out,
-                                                                       vals_out, gather_src, gather_dst);
+#undef DSX_SORT32_ITEMS
+    return DSX_ERR_RUNTIME;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1442,7 +1445,7 @@ ListsWorkspace lists_workspace(int64_t k, int num_tiles, bool binned)
     w.ids_alt = off;
     off = align(off + (size_t)k * 4);
     w.sort = off;
-    off += sort32_workspace(k, slot_bits(num_tiles), kListSortTile).bytes;
+    off += sort32_workspace(k, slot_bits(num_tiles), sort32_tile_keys(k)).bytes;
     w.bytes = align(off);
     return w;
 }
@@ -1483,7 +1486,7 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
     SlotT* slots_a = (kMasks && even) ? slots_final : slots_other;
     SlotT* slots_b = (kMasks && even) ? slots_other : slots_final;
     int rc = DSX_OK;
-    const Sort32Workspace sw = sort32_workspace(k, bits, kListSortTile);
+    const Sort32Workspace sw = sort32_workspace(k, bits, sort32_tile_keys(k));
     {
         DSX_TIMED("emit_ordered_kernel", stream);
         // outputs per workgroup: a multiple of 256 between 256 and kEmitChunkMax
@@ -1502,11 +1505,25 @@ static int tile_lists_impl(const dsx_camera& cam, int64_t n, int64_t k, int num_
     uint32_t* vo;
     // per-tile lists: the sorted slots themselves are not needed (the ranges are known already);
     // binned lists: they are kept for their masks
-    rc = sort32_passes<SlotT, kListSortThreads, kListSortItems>(k, bits, slots_a, vals_a, slots_b, vals_b, false,
-                                                                kMasks, base + w.sort,
-                                                                "onesweep32_kernel<tile partition>", stream, &ko, &vo,
-                                                                nullptr, nullptr,
-                                                                reinterpret_cast<const uint32_t*>(obase + o.slot_hist));
+    rc = DSX_ERR_RUNTIME;
+#define DSX_PARTITION_ITEMS(ITEMS)                                                                                    \
+    case ITEMS:                                                                                                       \
+        rc = sort32_passes<SlotT, kSortThreads32, ITEMS>(k, bits, slots_a, vals_a, slots_b, vals_b, false, kMasks,     \
+                                                         base + w.sort, "onesweep32_kernel<tile partition>", stream,  \
+                                                         &ko, &vo, nullptr, nullptr,                                  \
+                                                         reinterpret_cast<const uint32_t*>(obase + o.slot_hist));     \
+        break
+    switch(sort32_items(k))
+    {
+        DSX_PARTITION_ITEMS(1);
+        DSX_PARTITION_ITEMS(2);
+        DSX_PARTITION_ITEMS(3);
+        DSX_PARTITION_ITEMS(4);
+        DSX_PARTITION_ITEMS(6);
+        DSX_PARTITION_ITEMS(8);
+        DSX_PARTITION_ITEMS(kSortItemsMax32);
+    }
+#undef DSX_PARTITION_ITEMS
     if(rc)
         return rc;
     if(kMasks && ko != slots_final)
