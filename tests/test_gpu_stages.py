@@ -224,7 +224,11 @@ def test_sort_pairs_vs_oracle_on_emitted_keys(oracle):
 @pytest.mark.parametrize("count,key_bits,ties", [(2, 32, False), (1000, 32, False), (8192, 8, True), (8193, 13, False),
                                                  (70_000, 15, True), (1_000_003, 32, False), (300_001, 32, True),
                                                  (200_000, 1, True), (123_457, 17, False),
-                                                 (1_500_000, 32, False), (2_345_679, 24, True)])  # large-tile plan
+                                                 (1_500_000, 32, False), (2_345_679, 24, True),
+                                                 # every tile size of the pass kernel (1, 2, 3, 4, 6, 8, 12 keys per
+                                                 # thread by input size) and the step from one size to the next
+                                                 (262_144, 32, False), (262_145, 32, True), (700_001, 32, True),
+                                                 (1_900_003, 20, False)])
 def test_sort_pairs_u32_matches_stable_sort(count, key_bits, ties):
     """Stable ascending unsigned sort of keys that use their low key_bits bits."""
     st_ = _stages()
@@ -267,7 +271,11 @@ def test_sort_pairs_u32_orders_depth_bits_like_the_64_bit_keys():
                                                   (500, 64, 48, 3.0, 120), (1, 32, 32, 1.0, 0), (2, 32, 32, 1.0, 0),
                                                   (60000, 512, 384, 3.0, 500), (4000, 40, 30, 8.0, 50),
                                                   (30000, 3840, 2160, 6.0, 300), (20000, 16400, 1040, 8.0, 100),
-                                                  (40, 640, 480, 1.0, 0), (60, 1920, 1080, 2.0, 30)])
+                                                  (40, 640, 480, 1.0, 0), (60, 1920, 1080, 2.0, 30),
+                                                  # 0.57, 0.90, 1.30 and 1.79 M pairs: the partition's tiles of
+                                                  # 3, 4, 6 and 8 keys per thread, with 16-bit slots
+                                                  (10000, 512, 384, 3.0, 100), (16000, 512, 384, 3.0, 100),
+                                                  (23000, 512, 384, 3.0, 100), (32000, 512, 384, 3.0, 100)])
 def test_tile_lists_bit_exact(oracle, list_bin, n, W, H, scale_mul, flip, giants=0, camera="identity"):
     """Depth order + ordered emission + tile partition give the oracle's sorted ids and ranges
     (the result of the stable 64-bit sort of the emitted keys) bit for bit, including keys with
