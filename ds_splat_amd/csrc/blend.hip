@@ -11,14 +11,14 @@ namespace dsx
 
 constexpr float kAlphaThreshold = 1.0f / 255.0f;
 
-// exp through the hardware base-2 exponential (the reference is built with fast-math).  The
-// factor log2(e) is not applied per pixel: the three conic coefficients are multiplied by it
-// once, when an entry is staged in LDS, so the quadratic form below comes out in base 2.
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
-__device__ __forceinline__ float exp2_of(float x)
+// exp through the hardware base-2 exponential (the reference is built with fast-math).  The factor
+// log2(e) is applied to the finished exponent, per pixel: folded into the conic coefficients when an
+// entry is staged it would save that multiply, but every term of the quadratic form would carry one
+// more rounding, and where the terms are large and cancel (thin, long splats far from their centre)
+// the image then moves 1.6 times as far from the reference's as it does now.
+__device__ __forceinline__ float fast_exp(float x)
 {
-    return __builtin_amdgcn_exp2f(x);
+    return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
 }
 
 // The exponent of a splat at a pixel, -1/2 (a dx^2 + c dy^2) - b dx dy with d = pixel - mean, in
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                                                              uint8_t* __restrict__ prep_marks,
                                                              const BinLists lists)
 {
-    __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic -a/2, conic b (a, b, c times log2 e)
+    __shared__ float4 s_a[kFwdBatch]; // pixel x, pixel y, conic -a/2, conic b
     __shared__ float4 s_b[kFwdBatch]; // conic c/2, opacity, red, green
     __shared__ float s_c[kFwdBatch];  // blue
     // the queue of the tile's own entries (binned lists) lives in s_a between two rounds: up to 128 ids
@@ -370,8 +370,8 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
             {
                 const float4* rec = splats + 3 * (int64_t)g;
                 const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
-                s_a[slot] = make_float4(q0.x, q0.y, q1.x * (-0.5f * kLog2e), q1.y * kLog2e);
-                s_b[slot] = make_float4(q1.z * (0.5f * kLog2e), q1.w, q2.x, q2.y);
+                s_a[slot] = make_float4(q0.x, q0.y, q1.x * -0.5f, q1.y);
+                s_b[slot] = make_float4(q1.z * 0.5f, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
                 useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
             }
@@ -411,7 +411,7 @@ __global__ __launch_bounds__(DSX_WAVE) __attribute__((amdgpu_waves_per_eu(8, 8))
                 {
                     const float power = exponent_xy(ex, B.x, pyf[p] - A.y);
                     // (a NaN opacity gives alpha = 0.999 here as in the reference: fminf drops the NaN)
-                    const float alpha = fminf(0.999f, B.y * exp2_of(power));
+                    const float alpha = fminf(0.999f, B.y * fast_exp(power));
                     // the three decisions as wavefront masks (each is its compare's own result register),
                     // combined on the scalar unit and handed back to the lanes as conditions
                     // (1 - alpha) T in one rounding
@@ -655,7 +655,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
     const float* __restrict__ bg, float* grads, uint8_t* marks, int W, int H, int ntx, uint32_t last_id, int k,
     const int32_t* __restrict__ header, int header_shift, const BinLists lists, const ZeroJobs zeros)
 {
-    __shared__ float4 s_a[kBwdBatch]; // pixel x, pixel y, conic -a/2, conic b (a, b, c times log2 e)
+    __shared__ float4 s_a[kBwdBatch]; // pixel x, pixel y, conic -a/2, conic b
     __shared__ float4 s_b[kBwdBatch]; // conic c/2, opacity, red, green
     __shared__ float s_c[kBwdBatch];  // blue
     __shared__ int s_id[kBwdBatch];
@@ -818,8 +818,8 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             {
                 const float4* rec = splats + 3 * (int64_t)g;
                 const float4 q0 = rec[0], q1 = rec[1], q2 = rec[2];
-                s_a[slot] = make_float4(q0.x, q0.y, q1.x * (-0.5f * kLog2e), q1.y * kLog2e);
-                s_b[slot] = make_float4(q1.z * (0.5f * kLog2e), q1.w, q2.x, q2.y);
+                s_a[slot] = make_float4(q0.x, q0.y, q1.x * -0.5f, q1.y);
+                s_b[slot] = make_float4(q1.z * 0.5f, q1.w, q2.x, q2.y);
                 s_c[slot] = q2.z;
                 s_id[slot] = g;
                 useful = entry_reaches_tile(q0.x, q0.y, q1.x, q1.y, q1.z, q1.w, box_x0, box_y0, span_y);
@@ -859,7 +859,7 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             {
                 dy[p] = pyf[p] - A.y;
                 const float power = exponent_xy(ex, B.x, dy[p]);
-                vis[p] = exp2_of(power);
+                vis[p] = fast_exp(power);
                 alpha[p] = fminf(0.99f, B.y * vis[p]);
                 m_valid[p] = __builtin_amdgcn_ballot_w64(idx <= bin_final[p]) &
                              __builtin_amdgcn_ballot_w64(!(power > 0.0f)) &
@@ -902,12 +902,12 @@ __global__ __launch_bounds__(DSX_WAVE) void blend_bwd_kernel(
             const float dx = -dxf;
             S0 *= -B.y;
             S1 *= B.y;
-            // (the staged coefficients are -a/2, b and c/2 times log2(e): the factors are taken out of the
-            // two sums that use them; A.z * dxf and A.w * dxf are the exponent's own first products)
+            // (the staged coefficients are -a/2, b and c/2; A.z * dxf and A.w * dxf are the exponent's own
+            // first products)
             {
 #pragma clang fp contract(off)
-                g[0] = __builtin_fmaf(A.w, S1 * kLn2, (A.z * dxf) * (S0 * (2.0f * kLn2)));  // v_sigma (a dx + b dy)
-                g[1] = __builtin_fmaf(B.x, S1 * (2.0f * kLn2), -((A.w * dxf) * (S0 * kLn2))); // v_sigma (b dx + c dy)
+                g[0] = __builtin_fmaf(A.w, S1, (A.z * dxf) * (S0 * 2.0f));    // v_sigma (a dx + b dy)
+                g[1] = __builtin_fmaf(B.x, S1 * 2.0f, -((A.w * dxf) * S0)); // v_sigma (b dx + c dy)
             }
             g[2] = 0.5f * dx * dx * S0;
             g[3] = dx * S1;
